@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the DIA product path on one MI355X.
+
+A step is one pass of the hot path over one batch: the three calls a locally
+connected RBM layer makes on the 16384-unit / 49-diagonal / batch-128
+configuration --
+    up-pass          H  = A * V                    (prod 'n', beta 0)
+    down-pass        V' = 0.5*V' + A^T * H         (prod 't', beta 0.5)
+    weight gradient  G  = 0.9*G + (1/128)*proj_diag(Vg * Hg^T)   (densedense_to_dia)
+launched back to back on one stream with every operand already in HBM.  The
+operands rotate through enough distinct buffer sets (default: > 512 MB in
+total) that a step cannot be served from the 256 MB Infinity Cache; `--sets 1`
+gives the cache-warm figure instead.
+
+value = algorithmic bytes of the step / step time (GB/s); the algorithmic bytes
+count every operand once and only the valid diagonal slots
+(cuv_amd.workloads.spmm_bytes / dd2dia_bytes).  `roofline` describes the
+slowest of the three kernels, timed on its own with HIP events on the launch
+stream.  `cpu_baseline` is the single-threaded CPU oracle (a restatement of the
+reference's host loops) on the same step, on this machine's host cores.
+
+Prints one JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+FP32_VALU_PEAK_TFLOPS = 157.3  # published vector fp32 (packed); the kernels use no MFMA
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--sets", type=int, default=0,
+                    help="distinct operand sets rotated through (0: enough for > 512 MB)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch from a Python loop instead of replaying HIP graphs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path uses no collectives and every "
+              "configuration fits one MI355X; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from cuv_amd import _lib, dia as D, workloads as W
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback exists for the product path)", file=sys.stderr)
+        sys.exit(2)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    L = _lib.lib()
+
+    w1, w2, w3 = W.cfg1(), W.cfg2(), W.cfg3()
+    p = w1.pattern
+    batch = w1.batch
+    step_bytes = w1.bytes + w2.bytes + w3.bytes
+    step_flops = w1.flops + w2.flops + w3.flops
+
+    # one set = every buffer a step touches
+    set_bytes = 4 * (2 * p.nd * p.stride + 5 * p.h * batch)
+    nsets = args.sets if args.sets > 0 else max(2, -(-600_000_000 // set_bytes))
+
+    def dia_from(vals):
+        m = D.dev_dia_matrix_f(p.h, p.w, p.nd, p.stride, 1, device=dev)
+        m.set_offsets(p.offsets)
+        m.push(vals)
+        return m
+
+    sets = []
+    for _ in range(nsets):
+        sets.append(dict(
+            A=dia_from(w1.vals), V=D.to_device_colmajor(w1.X, dev),
+            H=torch.empty(batch, p.h, device=dev),
+            Hs=D.to_device_colmajor(w2.X, dev), Vp=D.to_device_colmajor(w2.dst, dev),
+            G=dia_from(w3.vals), Ga=D.to_device_colmajor(w3.A, dev), Gb=D.to_device_colmajor(w3.B, dev)))
+    for s in sets:
+        s["A"].desc, s["G"].desc                      # build descriptors outside the timed region
+        s["bd"] = D.dev_block_descriptor_f(s["G"])
+
+    def up(s):
+        D.prod(s["H"], s["A"], s["V"], "n", "n", w1.alpha, w1.beta, sync=False)
+
+    def down(s):
+        D.prod(s["Vp"], s["A"], s["Hs"], "t", "n", w2.alpha, w2.beta, sync=False)
+
+    def grad(s):
+        D.densedense_to_dia(s["G"], s["bd"], s["Ga"], s["Gb"], w3.alpha, w3.beta, sync=False)
+
+    def step(i):
+        s = sets[i % nsets]
+        up(s); down(s); grad(s)
+
+    # ---- parity of exactly these buffers, before they are mutated by repetition
+    checked = None
+    if not args.no_check:
+        from oracle import oracle as O
+        s = sets[0]
+        step(0)
+        torch.cuda.synchronize()
+        od = O.Dia(p.h, p.w, p.offsets, p.stride, 1, w1.vals)
+
+        def worst(got, ref, mag):
+            return float((np.abs(got.astype(np.float64) - ref) / np.maximum(mag, 1e-30)).max())
+        e1 = worst(D.to_host_colmajor(s["H"]), O.prod(od, w1.X), O.prod_mag(od, w1.X))
+        e2 = worst(D.to_host_colmajor(s["Vp"]), O.prod(od, w2.X, w2.dst, "t", 1.0, 0.5),
+                   O.prod_mag(od, w2.X, w2.dst, "t", 1.0, 0.5))
+        valid = O.valid_mask(od)
+        ref3 = O.dd2dia(od, w3.A, w3.B, w3.alpha, w3.beta)
+        mag3 = O.dd2dia_f64(O.Dia(p.h, p.w, p.offsets, p.stride, 1, np.abs(w3.vals)), w3.A, w3.B,
+                            w3.alpha, w3.beta)
+        e3 = worst(s["G"].pull()[valid], ref3[valid], mag3[valid])
+        checked = dict(tolerance=1e-5, up_pass=e1, down_pass=e2, weight_gradient=e3,
+                       ok=bool(max(e1, e2, e3) <= 1e-5))
+        if not checked["ok"]:
+            print("PARITY FAILURE: %r" % checked, file=sys.stderr)
+            sys.exit(1)
+        # restore the mutated buffers of set 0
+        s["Vp"].copy_(D.to_device_colmajor(w2.dst, dev)); s["G"].push(w3.vals)
+
+    stream = torch.cuda.current_stream()
+
+    # The kernels run for a few microseconds; a Python launch loop cannot feed
+    # them that fast.  Launches are therefore captured into HIP graphs (one
+    # graph = one rotation through the buffer sets) and the graphs replayed.
+    def capture(fn, count):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(count):
+                fn(i)
+        return g
+
+    def timed(fn, n):
+        """Exactly n calls fn(0..n-1) (fn must depend on i only through i % nsets)
+        between two HIP events on the launch stream; returns ms per call."""
+        if args.no_graph:
+            plan = None
+        else:
+            full, rest = divmod(n, nsets)
+            gfull = capture(fn, nsets) if full else None
+            grest = capture(fn, rest) if rest else None
+            for g in (gfull, grest):                      # untimed first launch of each graph
+                if g is not None:
+                    g.replay()
+            plan = (gfull, full, grest)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        if plan is None:
+            for i in range(n):
+                fn(i)
+        else:
+            gfull, full, grest = plan
+            for _ in range(full):
+                gfull.replay()
+            if grest is not None:
+                grest.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_step = timed(step, args.steps)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # graph replays must reproduce the eager result: the up-pass is idempotent,
+    # so after all those replays H of set 0 must equal a fresh eager H bit for bit
+    if not args.no_graph:
+        h_graph = sets[0]["H"].clone()
+        sets[0]["H"].fill_(float("nan"))
+        up(sets[0])
+        torch.cuda.synchronize()
+        if not torch.equal(h_graph, sets[0]["H"]):
+            print("GRAPH REPLAY MISMATCH against the eager launch", file=sys.stderr)
+            sys.exit(1)
+
+    # per-kernel figures: each operation alone, same rotation, same stream
+    per = {}
+    for name, fn, wl in (("up_pass", up, w1), ("down_pass", down, w2), ("weight_gradient", grad, w3)):
+        ms = timed(lambda i, fn=fn: fn(sets[i % nsets]), args.steps)
+        per[name] = dict(us=ms * 1e3, bytes=wl.bytes, flops=wl.flops,
+                         gbs=wl.bytes / (ms * 1e-3) / 1e9, gflops=wl.flops / (ms * 1e-3) / 1e9,
+                         frac_hbm=wl.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+    # cache-warm variant (one buffer set) for reference
+    warm = {}
+    for name, fn in (("up_pass", up), ("down_pass", down), ("weight_gradient", grad)):
+        ms = timed(lambda i, fn=fn: fn(sets[0]), args.steps)
+        warm[name] = ms * 1e3
+    kernel_names = {"up_pass": "spmm_tiled_kernel", "down_pass": "spmm_tiled_kernel",
+                    "weight_gradient": "dd2dia_tiled_kernel"}
+    dom = max(per, key=lambda k: per[k]["us"])
+    roofline = dict(bound="hbm", achieved=per[dom]["gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=per[dom]["gbs"] / HBM_PEAK_GBS, traffic=None,
+                    kernel=kernel_names[dom], op=dom, us_per_launch=per[dom]["us"],
+                    algorithmic_bytes=per[dom]["bytes"])
+
+    out = dict(
+        metric="achieved HBM GB/s, DIA SpMM (both transposes) + densedense_to_dia step",
+        value=step_bytes / (ms_step * 1e-3) / 1e9, unit="GB/s",
+        n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_step,
+        higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
+        config=dict(workload="cfg1+cfg2+cfg3: 16384x16384 DIA, 49 diagonals (7x7 window on a 128x128 map), "
+                             "batch 128; up-pass A*V, down-pass 0.5*V'+A^T*H, gradient 0.9*G+(1/128)*proj(Vg*Hg^T)",
+                    rows=p.h, diagonals=p.nd, batch=batch, buffer_sets=nsets,
+                    step_bytes=step_bytes, step_flops=step_flops),
+        frac_of_hbm_peak=step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        gflops=step_flops / (ms_step * 1e-3) / 1e9,
+        wall_ms_per_step_incl_capture=wall_ms, launch="eager" if args.no_graph else "hip_graph",
+        ops=per, warm_us=warm, parity=checked, roofline=roofline)
+
+    if not args.no_cpu:
+        from oracle import oracle as O
+        od = O.Dia(p.h, p.w, p.offsets, p.stride, 1, w1.vals)
+        reps = []
+        for _ in range(5):
+            t = time.perf_counter()
+            O.prod(od, w1.X)
+            O.prod(od, w2.X, w2.dst, "t", 1.0, 0.5)
+            O.dd2dia(od, w3.A, w3.B, w3.alpha, w3.beta)
+            reps.append(time.perf_counter() - t)
+        med = statistics.median(reps)
+        out["cpu_baseline"] = dict(value=step_bytes / med / 1e9, unit="GB/s", cores=1, kind="port",
+                                   sample="the full step (cfg1+cfg2+cfg3), median of 5 repetitions",
+                                   ms_per_step=med * 1e3, gflops=step_flops / med / 1e9)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,9 @@
+"""MI355X-native diagonal-sparse (DIA) matrix products behind CUV's interface.
+
+The compute lives in lib/libcuvdia.so (hand-written HIP for gfx950, C ABI in
+include/cuvdia.h).  `cuv_amd.dia` is the Python surface, `cuv_amd/include/cuv`
+the C++ one; `cuv_amd.workloads` generates the measured configurations.
+"""
+from . import _lib  # noqa: F401
+
+__all__ = ["_lib", "dia", "workloads"]

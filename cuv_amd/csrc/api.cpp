@@ -1,0 +1,354 @@
+// C ABI of libcuvdia (declared in include/cuvdia.h): argument validation,
+// descriptors, the offsets-keyed descriptor cache and kernel-family selection.
+#include "cuvdia.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cstdint>
+#include <cstring>
+#include <list>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "kernels.hpp"
+#include "plan.hpp"
+
+using namespace cuvdia;
+
+struct cuvdia_desc {
+    int h, w, nd, stride, rf;
+    int device;
+    std::vector<int> offsets;        // host copy, table order
+    long long nnz;
+    int n_chunks_n, n_chunks_t;
+    void *dev_block;                 // one allocation: offsets | chunks_n | chunks_t
+    DiaView view;
+};
+
+namespace {
+
+std::atomic_int g_path{CUVDIA_PATH_AUTO};
+thread_local int t_last_path = 0;
+thread_local std::string t_hip_error;
+
+// Batches narrower than this go to the generic kernel: the tiled SpMM puts
+// one batch column on each of 64 lanes.
+constexpr int SPMM_TILED_MIN_BATCH = 24;
+// Largest h, w and |offset| the kernels' 32-bit row arithmetic allows.
+constexpr long long DIM_LIMIT = 1LL << 30;
+
+int hip_fail(hipError_t e, const char *what)
+{
+    t_hip_error = std::string(what) + ": " + hipGetErrorString(e);
+    return CUVDIA_EHIP;
+}
+
+int validate_shape(const int *offsets, int nd, int h, int w, int stride, int rf)
+{
+    if (!offsets || nd < 1 || h < 1 || w < 1 || rf < 1 || stride < 1) return CUVDIA_EINVAL;
+    // src/cuv/basics/dia_matrix.hpp:131
+    if (!(stride >= h || stride >= w)) return CUVDIA_EINVAL;
+    if (h > DIM_LIMIT || w > DIM_LIMIT) return CUVDIA_EUNSUPPORTED;
+    // A diagonal is stored by row: its last valid row must fit in its own
+    // stride, or it would alias the next diagonal's storage.
+    for (int d = 0; d < nd; ++d) {
+        const long long k = offsets[d];
+        if (k >= DIM_LIMIT || k <= -DIM_LIMIT) return CUVDIA_EUNSUPPORTED;
+        const long long i0 = (long long)rf * std::max<long long>(0, -k);
+        const long long j0 = std::max<long long>(0, k);
+        const long long n = std::min<long long>(h - i0, (long long)rf * (w - j0));
+        if (n > 0 && i0 + n > stride) return CUVDIA_ESHAPE;
+    }
+    return CUVDIA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int cuvdia_abi_version(void) { return 1; }
+
+const char *cuvdia_strerror(int code)
+{
+    switch (code) {
+        case CUVDIA_OK: return "ok";
+        case CUVDIA_EINVAL: return "invalid argument";
+        case CUVDIA_ESHAPE: return "operand shapes do not match the matrix";
+        case CUVDIA_EHIP: return "HIP runtime call failed";
+        case CUVDIA_ENOMEM: return "out of memory";
+        case CUVDIA_EUNSUPPORTED: return "unsupported request";
+        case CUVDIA_ENODEVICE: return "no gfx950 device";
+        default: return "unknown cuvdia error";
+    }
+}
+
+const char *cuvdia_last_hip_error(void) { return t_hip_error.c_str(); }
+
+int cuvdia_set_path(int path)
+{
+    if (path != CUVDIA_PATH_AUTO && path != CUVDIA_PATH_GENERIC && path != CUVDIA_PATH_TILED)
+        return CUVDIA_EINVAL;
+    g_path.store(path);
+    return CUVDIA_OK;
+}
+
+int cuvdia_last_path(void) { return t_last_path; }
+
+int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
+                       int *s0, int *len, int *slot, int cap)
+{
+    if (!offsets_host || nd < 1) return CUVDIA_EINVAL;
+    std::vector<Chunk> ch;
+    try {
+        ch = plan_chunks(offsets_host, nd, transposed != 0);
+    } catch (const std::bad_alloc &) {
+        return CUVDIA_ENOMEM;
+    }
+    const int n = (int)ch.size();
+    if (n <= cap && s0 && len && slot) {
+        for (int c = 0; c < n; ++c) {
+            s0[c] = ch[c].s0;
+            len[c] = ch[c].len;
+            for (int j = 0; j < CHUNK_MAX; ++j) slot[c * CHUNK_MAX + j] = j < ch[c].len ? ch[c].slot[j] : -1;
+        }
+    }
+    return n;
+}
+
+int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
+                       int h, int w, int stride, int row_fact)
+{
+    if (!out) return CUVDIA_EINVAL;
+    *out = nullptr;
+    const int rc = validate_shape(offsets_host, nd, h, w, stride, row_fact);
+    if (rc) return rc;
+
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev < 1) {
+        t_hip_error = std::string("hipGetDeviceCount: ") + hipGetErrorString(e);
+        (void)hipGetLastError();
+        return CUVDIA_ENODEVICE;
+    }
+
+    cuvdia_desc *d = nullptr;
+    std::vector<Chunk> cn, ct;
+    try {
+        d = new cuvdia_desc();
+        d->offsets.assign(offsets_host, offsets_host + nd);
+        cn = plan_chunks(offsets_host, nd, false);
+        ct = plan_chunks(offsets_host, nd, true);
+    } catch (const std::bad_alloc &) {
+        delete d;
+        return CUVDIA_ENOMEM;
+    }
+    d->h = h; d->w = w; d->nd = nd; d->stride = stride; d->rf = row_fact;
+    d->nnz = count_valid(offsets_host, nd, h, w, row_fact);
+    d->n_chunks_n = (int)cn.size();
+    d->n_chunks_t = (int)ct.size();
+    d->dev_block = nullptr;
+    if ((e = hipGetDevice(&d->device)) != hipSuccess) { delete d; return hip_fail(e, "hipGetDevice"); }
+
+    // one device block: offsets (padded to 64 B) | chunks_n | chunks_t
+    const size_t off_bytes = ((size_t)nd * sizeof(int) + 63) / 64 * 64;
+    const size_t cn_bytes = cn.size() * sizeof(Chunk), ct_bytes = ct.size() * sizeof(Chunk);
+    std::vector<unsigned char> staging(off_bytes + cn_bytes + ct_bytes, 0);
+    std::memcpy(staging.data(), offsets_host, (size_t)nd * sizeof(int));
+    std::memcpy(staging.data() + off_bytes, cn.data(), cn_bytes);
+    std::memcpy(staging.data() + off_bytes + cn_bytes, ct.data(), ct_bytes);
+    if ((e = hipMalloc(&d->dev_block, staging.size())) != hipSuccess) {
+        delete d;
+        return e == hipErrorOutOfMemory ? CUVDIA_ENOMEM : hip_fail(e, "hipMalloc(descriptor)");
+    }
+    if ((e = hipMemcpy(d->dev_block, staging.data(), staging.size(), hipMemcpyHostToDevice)) != hipSuccess) {
+        (void)hipFree(d->dev_block);
+        delete d;
+        return hip_fail(e, "hipMemcpy(descriptor)");
+    }
+    unsigned char *base = static_cast<unsigned char *>(d->dev_block);
+    d->view = DiaView{h, w, nd, stride, row_fact,
+                      reinterpret_cast<const int *>(base),
+                      reinterpret_cast<const Chunk *>(base + off_bytes), d->n_chunks_n,
+                      reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t};
+    *out = d;
+    return CUVDIA_OK;
+}
+
+int cuvdia_desc_destroy(cuvdia_desc *desc)
+{
+    if (!desc) return CUVDIA_OK;
+    int rc = CUVDIA_OK;
+    if (desc->dev_block) {
+        const hipError_t e = hipFree(desc->dev_block);
+        if (e != hipSuccess) rc = hip_fail(e, "hipFree(descriptor)");
+    }
+    delete desc;
+    return rc;
+}
+
+int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t, long long *nnz)
+{
+    if (!desc) return CUVDIA_EINVAL;
+    if (chunks_n) *chunks_n = desc->n_chunks_n;
+    if (chunks_t) *chunks_t = desc->n_chunks_t;
+    if (nnz) *nnz = desc->nnz;
+    return CUVDIA_OK;
+}
+
+int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
+                    float *dst, long long ldd, int batch, char transA,
+                    float alpha, float beta, void *stream)
+{
+    if (!desc || !A_vals || batch < 0) return CUVDIA_EINVAL;
+    // make_spmv_header.pl:121-123: anything but 'n' / 't' is an error
+    if (transA != 'n' && transA != 't') return CUVDIA_EINVAL;
+    if (batch == 0) return CUVDIA_OK;
+    if (!B || !dst) return CUVDIA_EINVAL;
+    const bool trans = transA == 't';
+    const int n_out = trans ? desc->w : desc->h;
+    const int n_in = trans ? desc->h : desc->w;
+    if (ldb < n_in || ldd < n_out) return CUVDIA_ESHAPE;
+
+    const int forced = g_path.load();
+    const bool tiled_possible = desc->rf == 1;
+    bool tiled;
+    if (forced == CUVDIA_PATH_TILED) {
+        if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
+        tiled = true;
+    } else if (forced == CUVDIA_PATH_GENERIC) {
+        tiled = false;
+    } else {
+        tiled = tiled_possible && batch >= SPMM_TILED_MIN_BATCH;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const hipError_t e = tiled
+        ? launch_spmm_tiled(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, s)
+        : launch_spmm_generic(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, s);
+    t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
+    return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "spmm kernel launch");
+}
+
+int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, long long lda,
+                      const float *B, long long ldb, int batch,
+                      float alpha, float beta, void *stream)
+{
+    if (!desc || !C_vals || batch < 0) return CUVDIA_EINVAL;
+    if (batch > 0 && (!A || !B)) return CUVDIA_EINVAL;
+    if (batch > 0 && (lda < desc->h || ldb < desc->w)) return CUVDIA_ESHAPE;
+
+    const int forced = g_path.load();
+    const bool tiled_possible = desc->rf == 1;
+    bool tiled;
+    if (forced == CUVDIA_PATH_TILED) {
+        if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
+        tiled = true;
+    } else if (forced == CUVDIA_PATH_GENERIC) {
+        tiled = false;
+    } else {
+        tiled = tiled_possible;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const hipError_t e = tiled
+        ? launch_dd2dia_tiled(desc->view, C_vals, A, lda, B, ldb, batch, alpha, beta, s)
+        : launch_dd2dia_generic(desc->view, C_vals, A, lda, B, ldb, batch, alpha, beta, s);
+    t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
+    return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "dd2dia kernel launch");
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------- descriptor cache ----
+namespace {
+
+struct CacheEntry {
+    int h, w, stride, rf, device;
+    std::vector<int> offsets;
+    cuvdia_desc *desc;
+};
+std::mutex g_cache_mutex;
+std::list<CacheEntry> g_cache;              // most recently used first
+constexpr size_t CACHE_CAPACITY = 32;
+
+int cached_desc(const int *offsets, int nd, int stride, int h, int w, int rf, cuvdia_desc **out)
+{
+    *out = nullptr;
+    if (!offsets || nd < 1) return CUVDIA_EINVAL;
+    int device = 0;
+    const hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return CUVDIA_ENODEVICE;
+    }
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
+        if (it->h == h && it->w == w && it->stride == stride && it->rf == rf &&
+            it->device == device && (int)it->offsets.size() == nd &&
+            std::memcmp(it->offsets.data(), offsets, (size_t)nd * sizeof(int)) == 0) {
+            g_cache.splice(g_cache.begin(), g_cache, it);
+            *out = g_cache.front().desc;
+            return CUVDIA_OK;
+        }
+    }
+    cuvdia_desc *d = nullptr;
+    const int rc = cuvdia_desc_create(&d, offsets, nd, h, w, stride, rf);
+    if (rc) return rc;
+    try {
+        g_cache.push_front(CacheEntry{h, w, stride, rf, device, std::vector<int>(offsets, offsets + nd), d});
+    } catch (const std::bad_alloc &) {
+        cuvdia_desc_destroy(d);
+        return CUVDIA_ENOMEM;
+    }
+    if (g_cache.size() > CACHE_CAPACITY) {
+        // Work enqueued with the evicted table may still be running.
+        (void)hipDeviceSynchronize();
+        cuvdia_desc_destroy(g_cache.back().desc);
+        g_cache.pop_back();
+    }
+    *out = d;
+    return CUVDIA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int cuvdia_cache_clear(void)
+{
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    if (!g_cache.empty()) (void)hipDeviceSynchronize();
+    int rc = CUVDIA_OK;
+    for (auto &e : g_cache) {
+        const int r = cuvdia_desc_destroy(e.desc);
+        if (r) rc = r;
+    }
+    g_cache.clear();
+    return rc;
+}
+
+int cuvdia_spmm_offsets_f32(const float *A_vals, const int *offsets_host, int nd, int stride,
+                            int h, int w, int row_fact, const float *B, long long ldb,
+                            float *dst, long long ldd, int batch, char transA,
+                            float alpha, float beta, void *stream)
+{
+    cuvdia_desc *d = nullptr;
+    const int rc = cached_desc(offsets_host, nd, stride, h, w, row_fact, &d);
+    if (rc) return rc;
+    return cuvdia_spmm_f32(d, A_vals, B, ldb, dst, ldd, batch, transA, alpha, beta, stream);
+}
+
+int cuvdia_dd2dia_offsets_f32(float *C_vals, const int *offsets_host, int nd, int stride,
+                              int h, int w, int row_fact, const float *A, long long lda,
+                              const float *B, long long ldb, int batch,
+                              float alpha, float beta, void *stream)
+{
+    cuvdia_desc *d = nullptr;
+    const int rc = cached_desc(offsets_host, nd, stride, h, w, row_fact, &d);
+    if (rc) return rc;
+    return cuvdia_dd2dia_f32(d, C_vals, A, lda, B, ldb, batch, alpha, beta, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,47 @@
+// Launch interface between the C ABI (api.cpp) and the gfx950 kernels
+// (kernels.hip).  Everything here is host-callable; shapes have been validated
+// by the caller.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include "plan.hpp"
+
+namespace cuvdia {
+
+struct DiaView {
+    int h, w, nd, stride, rf;
+    const int *offsets_dev;      // nd ints, table order
+    const Chunk *chunks_n_dev;   // shifts = offsets
+    int n_chunks_n;
+    const Chunk *chunks_t_dev;   // shifts = -offsets
+    int n_chunks_t;
+};
+
+// dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch
+// columns per thread; honours row_fact.
+hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float *B, long long ldb,
+                               float *dst, long long ldd, int batch, bool trans,
+                               float alpha, float beta, hipStream_t stream);
+
+// Same contract, row_fact == 1 only: 64 output rows x 64 batch columns per
+// workgroup, dense tile staged through LDS once per run chunk, lanes own
+// batch columns and keep a sliding register window along the rows, diagonal
+// values arrive through the scalar unit.
+hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
+                             float *dst, long long ldd, int batch, bool trans,
+                             float alpha, float beta, hipStream_t stream);
+
+// C_d[i] = beta*C_d[i] + alpha*sum_c A[i,c]*B[k_d + i/rf, c] on valid slots.
+// One thread per slot, serial over the batch; honours row_fact.
+hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, long long lda,
+                                 const float *B, long long ldb, int batch,
+                                 float alpha, float beta, hipStream_t stream);
+
+// Same contract, row_fact == 1 only: a workgroup owns 256 rows of one run
+// chunk; each lane keeps 4 rows x 8 diagonals of partial sums, the four
+// waves split the batch and are summed through LDS in wave order.
+hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
+                               const float *B, long long ldb, int batch,
+                               float alpha, float beta, hipStream_t stream);
+
+}  // namespace cuvdia

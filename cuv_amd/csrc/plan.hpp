@@ -1,0 +1,34 @@
+// Host-side decomposition of a DIA offset table into run chunks.
+//
+// A tiled kernel does not walk the offset table diagonal by diagonal; it
+// walks *chunks*: up to CHUNK_MAX consecutive shifts (s0, s0+1, ...) whose
+// dense-operand rows overlap, so one staged window of the dense tile serves
+// all of them.  For the normal product the shift of diagonal d is its offset
+// k_d (input row = output row + k_d); for the transposed product it is -k_d.
+#pragma once
+#include <vector>
+
+namespace cuvdia {
+
+constexpr int CHUNK_MAX = 8;
+
+// 48 bytes; read by the kernels through scalar loads.
+struct Chunk {
+    int s0;                 // shift of the first diagonal in the chunk
+    int len;                // number of diagonals, 1..CHUNK_MAX
+    int slot[CHUNK_MAX];    // table position (d) of each, so values sit at vals[slot*stride + ...]
+    int pad[2];
+};
+static_assert(sizeof(Chunk) == 48, "Chunk layout is part of the device table");
+
+// Sort shifts (stable in table position), cut into maximal runs of
+// consecutive shifts -- a repeated shift starts a new run -- and split each
+// run into near-equal chunks of at most CHUNK_MAX.
+std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed);
+
+// Number of matrix elements stored (slots the reference host loops touch):
+// sum over diagonals of min(h - rf*max(0,-k), rf*(w - max(0,k))), clamped at 0
+// (src/cuv/matrix_ops/spmv.cu:183-189).
+long long count_valid(const int *offsets, int nd, int h, int w, int rf);
+
+}  // namespace cuvdia

@@ -1,0 +1,155 @@
+"""Python surface over the C ABI, mirroring the reference's Boost.Python export
+of the DIA path (src/cuv_python/export_dia_mat.cpp:113-235): a device DIA
+matrix type, `prod(C, A_dia, B, transA, transB, factAB, factC)` and
+`densedense_to_dia(C_dia, bd, A, B, factAB, factC)`.
+
+Dense operands are 2-d torch CUDA tensors holding a column-major matrix, i.e.
+a tensor of shape (batch, rows) that is contiguous (`t.t()` is the rows x batch
+view).  torch only provides device memory and the stream here.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+def _stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check_dense(t, rows, name):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.dim() == 2):
+        raise TypeError("%s must be a 2-d float32 CUDA tensor" % name)
+    if t.stride(1) != 1:
+        raise ValueError("%s must be column-major: shape (batch, rows) with unit stride along rows" % name)
+    if t.shape[1] != rows:
+        raise RuntimeError("%s has %d rows, expected %d" % (name, t.shape[1], rows))
+    return t.shape[0], max(t.stride(0), rows) if t.shape[0] > 1 else max(rows, 1)
+
+
+class dev_dia_matrix_f:
+    """DIA matrix in device memory: element (i, j) at vec[d*stride + i] with
+    offsets[d] == j - i//row_fact (src/cuv/basics/dia_matrix.hpp:57-276)."""
+
+    def __init__(self, h, w, num_dia, stride, row_fact=1, device="cuda:0"):
+        if row_fact <= 0:
+            raise RuntimeError("m_row_fact>0")
+        if not (stride >= h or stride >= w):
+            raise RuntimeError("m_stride >= this->h() || m_stride >= this->w()")
+        self.h, self.w, self.num_dia, self.stride, self.row_fact = h, w, num_dia, stride, row_fact
+        self.vec = torch.zeros(num_dia * stride, dtype=torch.float32, device=device)
+        self._offsets = np.zeros(num_dia, np.int32)
+        self._desc = None
+
+    def __del__(self):
+        self._drop_desc()
+
+    def _drop_desc(self):
+        if getattr(self, "_desc", None):
+            torch.cuda.synchronize()
+            _lib.lib().cuvdia_desc_destroy(self._desc)
+            self._desc = None
+
+    def set_offsets(self, offsets):
+        offsets = np.ascontiguousarray(offsets, dtype=np.int32)
+        if offsets.size != self.num_dia:
+            raise RuntimeError("expected %d offsets" % self.num_dia)
+        self._offsets = offsets.copy()
+        self._drop_desc()
+
+    def get_offsets(self):
+        return self._offsets.copy()
+
+    @property
+    def desc(self):
+        if self._desc is None:
+            d = ctypes.c_void_p()
+            with torch.cuda.device(self.vec.device):
+                _lib.check(_lib.lib().cuvdia_desc_create(
+                    ctypes.byref(d), self._offsets.ctypes.data_as(ctypes.POINTER(ctypes.c_int)),
+                    self.num_dia, self.h, self.w, self.stride, self.row_fact), "cuvdia_desc_create")
+            self._desc = d
+        return self._desc
+
+    def info(self):
+        cn, ct, nnz = ctypes.c_int(), ctypes.c_int(), ctypes.c_longlong()
+        _lib.check(_lib.lib().cuvdia_desc_info(self.desc, ctypes.byref(cn), ctypes.byref(ct),
+                                               ctypes.byref(nnz)), "cuvdia_desc_info")
+        return dict(chunks_n=cn.value, chunks_t=ct.value, nnz=nnz.value)
+
+    def push(self, host_vals):
+        """Host -> device copy of the value vector (convert(dev_dia, host_dia),
+        src/cuv/convert/convert.cu:71-90)."""
+        v = torch.from_numpy(np.ascontiguousarray(host_vals, dtype=np.float32).reshape(-1))
+        if v.numel() != self.vec.numel():
+            raise RuntimeError("value vector has %d entries, expected %d" % (v.numel(), self.vec.numel()))
+        self.vec.copy_(v)
+        return self
+
+    def pull(self):
+        return self.vec.cpu().numpy()
+
+
+class dev_block_descriptor_f:
+    """Kept for signature compatibility with densedense_to_dia(C, bd, A, B, ...)
+    (src/cuv/matrix_ops/densedense_to_sparse.hpp:69-105); the run table lives in
+    the matrix's own descriptor, so this only pins it."""
+
+    def __init__(self, dia):
+        self.dia = dia
+        self._desc = dia.desc
+
+    def len(self):
+        return self.dia.info()["chunks_n"]
+
+
+def prod(dst, A, B, transA="n", transB="n", factAB=1.0, factC=0.0, sync=True):
+    """dst = factC*dst + factAB*op(A)*B (src/cuv/matrix_ops/spmv.cu:221-247)."""
+    if transB != "n":
+        raise RuntimeError("transB == 'n'")
+    if transA not in ("n", "t"):
+        raise RuntimeError("transA must be 'n' or 't'")
+    n_out, n_in = (A.w, A.h) if transA == "t" else (A.h, A.w)
+    bb, ldb = _check_dense(B, n_in, "B")
+    bd, ldd = _check_dense(dst, n_out, "dst")
+    if bb != bd:
+        raise RuntimeError("dst.shape()[1] == B.shape()[1]")
+    with torch.cuda.device(dst.device):
+        _lib.check(_lib.lib().cuvdia_spmm_f32(
+            A.desc, A.vec.data_ptr(), B.data_ptr(), ldb, dst.data_ptr(), ldd, bb,
+            transA.encode(), factAB, factC, _stream_ptr()), "cuvdia_spmm_f32")
+        if sync:
+            torch.cuda.current_stream().synchronize()
+    return dst
+
+
+def densedense_to_dia(C, bd, A, B, factAB=1.0, factC=0.0, sync=True):
+    """C = factC*C + factAB*proj(A*B') on C's stored diagonals
+    (src/cuv/matrix_ops/densedense_to_sparse.hpp:107-129)."""
+    ba, lda = _check_dense(A, C.h, "A")
+    bb, ldb = _check_dense(B, C.w, "B")
+    if ba != bb:
+        raise RuntimeError("A.shape()[1] == B.shape()[1]")
+    with torch.cuda.device(C.vec.device):
+        _lib.check(_lib.lib().cuvdia_dd2dia_f32(
+            C.desc, C.vec.data_ptr(), A.data_ptr(), lda, B.data_ptr(), ldb, ba,
+            factAB, factC, _stream_ptr()), "cuvdia_dd2dia_f32")
+        if sync:
+            torch.cuda.current_stream().synchronize()
+    return C
+
+
+def to_device_colmajor(a, device="cuda:0"):
+    """numpy (rows, batch) array -> torch (batch, rows) contiguous CUDA tensor
+    holding the same column-major matrix."""
+    a = np.asarray(a, dtype=np.float32)
+    if a.ndim == 1:
+        a = a.reshape(-1, 1)
+    return torch.from_numpy(np.ascontiguousarray(a.T)).to(device)
+
+
+def to_host_colmajor(t):
+    """Inverse of to_device_colmajor: returns a Fortran-ordered (rows, batch) array."""
+    return np.asfortranarray(t.detach().cpu().numpy().T)

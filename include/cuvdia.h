@@ -1,0 +1,155 @@
+/*
+ * cuvdia.h -- C ABI of the MI355X (gfx950) diagonal-sparse product library.
+ *
+ * This is the drop-in boundary for CUV's DIA matrix path: the entry points
+ * below are what the dev_memory_space specialisations of cuv::prod /
+ * cuv::spmv / cuv::densedense_to_dia bind instead of launching the CUDA
+ * kernels.  Reference files are cited relative to the CUV checkout.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every float/int buffer named "device"
+ *     is a raw hipMalloc pointer on the current device; "host" buffers are
+ *     ordinary host memory;
+ *   - dense operands are fp32, column-major, with an explicit leading
+ *     dimension in elements (the reference always uses ld == rows,
+ *     src/cuv/matrix_ops/spmv.cu:243-244);
+ *   - a DIA matrix stores element (i, j) at vals[d*stride + i] where
+ *     offsets[d] == j - i/row_fact (src/cuv/basics/dia_matrix.hpp:228-243);
+ *     slots of a stored diagonal that map to no matrix element (padding) are
+ *     never read and never written;
+ *   - every call returns CUVDIA_OK (0) or a negative CUVDIA_E* code and
+ *     never throws; kernels are enqueued on `stream` (a hipStream_t passed
+ *     as void*, NULL = the default stream) and the call returns without
+ *     synchronising -- the C++ mirror synchronises to keep the reference's
+ *     "results visible on return" behaviour (spmv.cu:99,
+ *     densedense_to_sparse.cu:295);
+ *   - no entry point allocates device memory except cuvdia_desc_create and
+ *     the first use of a new offset table by the *_offsets_* forms.
+ */
+#ifndef CUVDIA_H
+#define CUVDIA_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CUVDIA_OK            0
+#define CUVDIA_EINVAL       -1  /* null pointer, bad flag, non-positive size     */
+#define CUVDIA_ESHAPE       -2  /* operand shapes inconsistent with the matrix    */
+#define CUVDIA_EHIP         -3  /* a HIP runtime call failed                      */
+#define CUVDIA_ENOMEM       -4  /* host or device allocation failed               */
+#define CUVDIA_EUNSUPPORTED -5  /* valid request this build has no kernel for     */
+#define CUVDIA_ENODEVICE    -6  /* no gfx950 device visible                       */
+
+/* Kernel families, for cuvdia_set_path / cuvdia_last_path. */
+#define CUVDIA_PATH_AUTO     0  /* pick by shape (default)                        */
+#define CUVDIA_PATH_GENERIC  1  /* one-thread-per-output kernels, any row_fact    */
+#define CUVDIA_PATH_TILED    2  /* LDS-staged, register-blocked kernels (rf == 1) */
+
+/* Opaque description of one diagonal pattern: shape, offset table, and the
+ * device-resident run table the tiled kernels walk.  Replaces the contents of
+ * dev_block_descriptor (src/cuv/matrix_ops/densedense_to_sparse.hpp:69-105,
+ * built in densedense_to_sparse.cu:123-171) -- O(num_dia) instead of one
+ * entry per 16x16 block -- and the device copy of dia_matrix::m_offsets
+ * (src/cuv/basics/dia_matrix.hpp:75). */
+typedef struct cuvdia_desc cuvdia_desc;
+
+/* Builds a descriptor from a HOST offset table (table order is preserved:
+ * vals slot d belongs to offsets_host[d]).  Requires nd >= 1, h, w >= 1,
+ * row_fact >= 1 and stride >= h or stride >= w (dia_matrix.hpp:106,131).
+ * Allocates a few KB of device memory. */
+int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
+                       int h, int w, int stride, int row_fact);
+
+/* Frees the descriptor and its device table.  NULL is accepted. */
+int cuvdia_desc_destroy(cuvdia_desc *desc);
+
+/* Host-side facts about a descriptor (any pointer may be NULL):
+ * number of run chunks for the normal and transposed traversal, and the
+ * number of valid (non-padding) elements. */
+int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t,
+                     long long *nnz);
+
+/* Pure host function (no GPU needed): decomposes an offset table into the
+ * run chunks the tiled kernels walk.  Shifts are the offsets themselves
+ * (transposed == 0) or their negation (transposed != 0), sorted ascending;
+ * a run is a maximal sequence of consecutive shifts and is cut into chunks
+ * of at most 8.  Chunk c covers shifts s0[c] .. s0[c]+len[c]-1 and
+ * slot[8*c + j] is the table position of the j-th one.  Returns the number
+ * of chunks (also when it exceeds cap; then nothing is written), or a
+ * negative error. */
+int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
+                       int *s0, int *len, int *slot, int cap);
+
+/* dst = beta*dst + alpha*op(A)*B for a batch of dense columns.
+ * Replaces prod<float,dev_memory_space,column_major>(dst, dia A, B, transA,
+ * 'n', factAB, factC) (src/cuv/matrix_ops/spmv.cu:221-247), the spmv it
+ * forwards to (spmv.cu:89-101,130-139) and the generated kernel dispatcher
+ * (src/cuv/matrix_ops/make_spmv_header.pl:94-127, kernels in
+ * src/cuv/matrix_ops/spmv_kernel.cuh:55-300).
+ *   transA == 'n': A is h x w, B is w x batch (ldb >= w), dst h x batch (ldd >= h)
+ *   transA == 't': B is h x batch (ldb >= h), dst is w x batch (ldd >= w)
+ * beta == 0 follows the reference HOST rule (spmv.cu:152-156): dst is
+ * overwritten and never read, so it may hold NaN.  batch == 0 is a no-op.
+ * B and dst must not overlap. */
+int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals_device,
+                    const float *B_device, long long ldb,
+                    float *dst_device, long long ldd, int batch,
+                    char transA, float alpha, float beta, void *stream);
+
+/* C = beta*C + alpha*proj(A*B') restricted to the stored diagonals of C:
+ *   C_d[i] = beta*C_d[i] + alpha * sum_c A[i,c] * B[offsets[d] + i/row_fact, c]
+ * for every valid slot.  Replaces densedense_to_dia<float,column_major>
+ * (dev) (src/cuv/matrix_ops/densedense_to_sparse.cu:253-308) and its kernel
+ * dense2dia_mm (densedense_to_sparse.cu:51-120), with the documented
+ * contract of src/cuv/matrix_ops/densedense_to_sparse.hpp:107-121.
+ * A is h x batch (lda >= h), B is w x batch (ldb >= w).  beta == 0 never
+ * reads C.  batch == 0 scales C by beta (zero-fills valid slots if beta == 0). */
+int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals_device,
+                      const float *A_device, long long lda,
+                      const float *B_device, long long ldb, int batch,
+                      float alpha, float beta, void *stream);
+
+/* The same two operations taking the offset table from HOST memory on every
+ * call, for callers that hold only a dia_matrix (the reference signatures
+ * carry no descriptor for prod).  A descriptor is created on first sight of
+ * an (offsets, h, w, stride, row_fact) combination and kept in a small
+ * process-wide cache (device allocation on a miss only). */
+int cuvdia_spmm_offsets_f32(const float *A_vals_device, const int *offsets_host,
+                            int nd, int stride, int h, int w, int row_fact,
+                            const float *B_device, long long ldb,
+                            float *dst_device, long long ldd, int batch,
+                            char transA, float alpha, float beta, void *stream);
+
+int cuvdia_dd2dia_offsets_f32(float *C_vals_device, const int *offsets_host,
+                              int nd, int stride, int h, int w, int row_fact,
+                              const float *A_device, long long lda,
+                              const float *B_device, long long ldb, int batch,
+                              float alpha, float beta, void *stream);
+
+/* Drops every descriptor held by the *_offsets_* cache. */
+int cuvdia_cache_clear(void);
+
+/* Forces a kernel family for subsequent calls (process-wide; tests use it to
+ * run both families on the same inputs).  CUVDIA_PATH_TILED on a request the
+ * tiled kernels cannot serve (row_fact > 1) returns CUVDIA_EUNSUPPORTED from
+ * the compute call. */
+int cuvdia_set_path(int path);
+
+/* Which family the most recent compute call on this thread launched
+ * (CUVDIA_PATH_GENERIC or CUVDIA_PATH_TILED; 0 before any call). */
+int cuvdia_last_path(void);
+
+/* Static string for an error code. */
+const char *cuvdia_strerror(int code);
+
+/* Text of the last HIP failure seen by this thread ("" if none). */
+const char *cuvdia_last_hip_error(void);
+
+/* ABI revision of this header. */
+int cuvdia_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUVDIA_H */

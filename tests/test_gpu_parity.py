@@ -1,0 +1,285 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle
+on the same seeded inputs.
+
+Tolerance (fp32): |gpu - oracle| <= 1e-5 * sum|terms| per element and
+<= 1e-5 * max|oracle| in the max norm (see _gpu_util.assert_close_mag); the
+closed-form sequence() fixtures of the reference's own tests must come out
+exactly (their sums are integers below 2^24).
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.fixture(scope="module")
+def gu():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    import _gpu_util
+    return _gpu_util
+
+
+def _load(name):
+    with open(os.path.join(HERE, "golden", name)) as f:
+        return json.load(f)
+
+
+def _seq(rows, cols):
+    return np.arange(rows * cols, dtype=np.float32).reshape(cols, rows).T.copy(order="F")
+
+
+def _rand_dia(o, rng, h, w, offsets, rf=1, stride=None, pad=np.nan, lo=-1.0, hi=1.0):
+    d = o.Dia(h, w, offsets, stride, rf)
+    d.vals[:] = pad
+    m = o.valid_mask(d)
+    d.vals[m] = rng.uniform(lo, hi, int(m.sum())).astype(np.float32)
+    return d
+
+
+def _paths(rf):
+    from cuv_amd import _lib
+    return [_lib.PATH_GENERIC] if rf != 1 else [_lib.PATH_GENERIC, _lib.PATH_TILED]
+
+
+# ------------------------------------------- the reference's own fixtures ---
+def test_reference_spmv_fixture_exact(oracle, gu):
+    # src/tests/spmv.cpp:103-143
+    fx = _load("spmv_fixture.json")
+    A = oracle.Dia(fx["h"], fx["w"], fx["offsets"], fx["stride"], 1)
+    A.vals[:] = np.arange(A.vals.size, dtype=np.float32)
+    B, C = _seq(fx["w"], fx["batch"]), _seq(fx["h"], fx["batch"])
+    for path in _paths(1):
+        got, ran = gu.gpu_prod(A, B, None, "n", 1.0, 0.0, path)
+        assert ran == path
+        assert np.array_equal(got, np.asarray(fx["AB"], np.float32))
+        got, _ = gu.gpu_prod(A, C, None, "t", 1.0, 0.0, path)
+        assert np.array_equal(got, np.asarray(fx["AtC"], np.float32))
+        got, _ = gu.gpu_prod(A, B, C, "n", 2.0, 1.3, path)
+        np.testing.assert_allclose(got, np.asarray(fx["n_alpha2_beta1p3"]), rtol=2e-6)
+        got, _ = gu.gpu_prod(A, C, B, "t", 2.0, 1.3, path)
+        np.testing.assert_allclose(got, np.asarray(fx["t_alpha2_beta1p3"]), rtol=2e-6)
+
+
+def test_reference_dd2dia_fixture_exact(oracle, gu):
+    # src/tests/densedense_to_dia.cpp:109-197 -- row_fact 4, on the device
+    fx = _load("dd2dia_fixture.json")
+    C = oracle.Dia(fx["h"], fx["w"], fx["offsets"], fx["stride"], fx["rf"])
+    A, B = _seq(fx["h"], fx["batch"]), _seq(fx["w"], fx["batch"])
+    exp = np.asarray([[np.nan if v is None else v for v in row] for row in fx["expected"]]).reshape(-1)
+    valid = ~np.isnan(exp)
+    got, _ = gu.gpu_dd2dia(C, A, B, 1.0, 0.0)
+    assert np.array_equal(got[valid].astype(np.float64), exp[valid])
+    assert np.all(got[~valid] == 0)
+    assert np.array_equal(got, oracle.dd2dia_literal(C, A, B))      # dd2s_cmp_dev_host
+
+
+def test_reference_dd2dia_fixture_rf1_both_paths(oracle, gu):
+    fx = _load("dd2dia_fixture.json")
+    C = oracle.Dia(fx["h"], fx["w"], fx["offsets"], fx["stride"], 1)
+    A, B = _seq(fx["h"], fx["batch"]), _seq(fx["w"], fx["batch"])
+    ref = oracle.dd2dia_literal(C, A, B)
+    for path in _paths(1):
+        got, ran = gu.gpu_dd2dia(C, A, B, 1.0, 0.0, path)
+        assert ran == path
+        assert np.array_equal(got, ref)
+
+
+# ------------------------------------------------------- shapes and edges ---
+SHAPES = [
+    # h, w, offsets, rf, batch
+    (32, 16, [-3, -2, -1, 0, 1, 2, 3], 1, 6),
+    (16, 32, [0, 1, -1], 1, 70),                    # unsorted, wide, batch not a tile multiple
+    (40, 40, [5, -7, 0, 39, -39], 1, 64),           # corner diagonals
+    (36, 19, [-3, -2, -1, 0, 1, 2, 3], 4, 16),      # steep (generic kernels)
+    (24, 12, [2, -1, 0, 4], 2, 5),
+    (200, 333, list(range(-20, 21)), 1, 33),        # long run -> several chunks
+    (333, 200, [-300, -64, -63, -62, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 150, 199], 1, 128),
+    (1000, 1000, [0, 0, 3, 2000, -2000, 3], 1, 40), # duplicates and out-of-range offsets
+    (130, 130, [1], 1, 1),
+    (64, 64, [0], 1, 64),
+    (700, 650, [d * 25 + e for d in range(-2, 3) for e in range(-2, 3)], 1, 96),
+]
+
+
+@pytest.mark.parametrize("h,w,offs,rf,batch", SHAPES)
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_spmm_shapes(oracle, gu, h, w, offs, rf, batch, trans):
+    rng = np.random.default_rng(h * 1000 + w + batch)
+    A = _rand_dia(oracle, rng, h, w, offs, rf)          # NaN in every padding slot
+    n_in, n_out = (h, w) if trans == "t" else (w, h)
+    B = np.asfortranarray(rng.uniform(-1, 1, (n_in, batch)).astype(np.float32))
+    dst = np.asfortranarray(rng.uniform(-1, 1, (n_out, batch)).astype(np.float32))
+    for path in _paths(rf):
+        # beta == 0: destination starts as NaN and must come out finite
+        gu.check_prod(oracle, A, B, None, trans, 1.0, 0.0, path, "beta0 path%d" % path)
+        gu.check_prod(oracle, A, B, dst, trans, 0.75, -1.5, path, "scaled path%d" % path)
+
+
+@pytest.mark.parametrize("h,w,offs,rf,batch", SHAPES)
+def test_dd2dia_shapes(oracle, gu, h, w, offs, rf, batch):
+    if h % rf:
+        pytest.skip("reference loop undefined when rows are not a multiple of row_fact")
+    rng = np.random.default_rng(h * 77 + w + batch)
+    C = _rand_dia(oracle, rng, h, w, offs, rf, pad=np.nan)
+    A = np.asfortranarray(rng.uniform(-1, 1, (h, batch)).astype(np.float32))
+    B = np.asfortranarray(rng.uniform(-1, 1, (w, batch)).astype(np.float32))
+    for path in _paths(rf):
+        gu.check_dd2dia(oracle, C, A, B, 1.0 / batch, 0.9, path, "dd2dia path%d" % path)
+        Cn = oracle.Dia(h, w, offs, C.stride, rf, np.full_like(C.vals, np.nan))
+        gu.check_dd2dia(oracle, Cn, A, B, 1.0, 0.0, path, "dd2dia beta0 path%d" % path)
+
+
+def test_leading_dimensions_and_views(oracle, gu):
+    """Operands that are column slices of wider allocations (ld > rows)."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    rng = np.random.default_rng(9)
+    h, w, offs, batch = 300, 260, [-5, -4, -3, 0, 1, 2, 40], 48
+    A = _rand_dia(oracle, rng, h, w, offs)
+    B = np.asfortranarray(rng.uniform(-1, 1, (w, batch)).astype(np.float32))
+    Ad = gu.make_dev_dia(A)
+    ldb, ldd = w + 12, h + 20
+    Bbig = torch.zeros(batch, ldb, device="cuda:0")
+    Bbig[:, :w] = D.to_device_colmajor(B)
+    Dbig = torch.full((batch, ldd), -7.0, device="cuda:0")
+    for path in _paths(1):
+        _lib.lib().cuvdia_set_path(path)
+        try:
+            D.prod(Dbig[:, :h], Ad, Bbig[:, :w], "n", "n", 1.0, 0.0)
+        finally:
+            _lib.lib().cuvdia_set_path(_lib.PATH_AUTO)
+        got = D.to_host_colmajor(Dbig[:, :h])
+        gu.assert_close_mag(got, oracle.prod(A, B), oracle.prod_mag(A, B), "ld view")
+        assert torch.all(Dbig[:, h:] == -7.0)          # nothing past the rows was touched
+
+
+def test_batch_zero_and_errors(oracle, gu):
+    import ctypes
+    import torch
+    from cuv_amd import _lib, dia as D
+    L = _lib.lib()
+    A = oracle.Dia(32, 16, [-1, 0, 1], 32, 1)
+    Ad = gu.make_dev_dia(A)
+    x = torch.zeros(4, 16, device="cuda:0")
+    y = torch.zeros(4, 32, device="cuda:0")
+    sp = ctypes.c_void_p(0)
+    assert L.cuvdia_spmm_f32(Ad.desc, Ad.vec.data_ptr(), x.data_ptr(), 16, y.data_ptr(), 32, 0, b"n", 1.0, 0.0, sp) == 0
+    assert L.cuvdia_spmm_f32(Ad.desc, Ad.vec.data_ptr(), x.data_ptr(), 16, y.data_ptr(), 32, 4, b"x", 1.0, 0.0, sp) == _lib.EINVAL
+    assert L.cuvdia_spmm_f32(Ad.desc, Ad.vec.data_ptr(), x.data_ptr(), 15, y.data_ptr(), 32, 4, b"n", 1.0, 0.0, sp) == _lib.ESHAPE
+    assert L.cuvdia_spmm_f32(Ad.desc, Ad.vec.data_ptr(), None, 16, y.data_ptr(), 32, 4, b"n", 1.0, 0.0, sp) == _lib.EINVAL
+    assert L.cuvdia_spmm_f32(None, Ad.vec.data_ptr(), x.data_ptr(), 16, y.data_ptr(), 32, 4, b"n", 1.0, 0.0, sp) == _lib.EINVAL
+    # transposed product needs B with h rows
+    with pytest.raises(RuntimeError):
+        D.prod(y, Ad, x, "t")
+    with pytest.raises(RuntimeError):
+        D.prod(y, Ad, x, "n", "t")
+    d = ctypes.c_void_p()
+    offs = np.array([0, 1], np.int32)
+    ip = ctypes.POINTER(ctypes.c_int)
+    assert L.cuvdia_desc_create(ctypes.byref(d), offs.ctypes.data_as(ip), 2, 32, 16, 8, 1) == _lib.EINVAL   # stride < h and < w
+    low = np.array([0, -20], np.int32)          # rows 20..31 of a stride-16 diagonal alias the next one
+    assert L.cuvdia_desc_create(ctypes.byref(d), low.ctypes.data_as(ip), 2, 32, 16, 16, 1) == _lib.ESHAPE
+    assert L.cuvdia_desc_create(ctypes.byref(d), offs.ctypes.data_as(ip), 2, 32, 16, 16, 1) == 0
+    assert L.cuvdia_desc_destroy(d) == 0
+    assert L.cuvdia_desc_create(ctypes.byref(d), offs.ctypes.data_as(ip), 0, 32, 16, 32, 1) == _lib.EINVAL
+    assert L.cuvdia_desc_create(ctypes.byref(d), offs.ctypes.data_as(ip), 2, 32, 16, 32, 0) == _lib.EINVAL
+    # a steep matrix cannot be forced onto the tiled kernels
+    S = oracle.Dia(36, 19, [0, 1], 36, 4)
+    Sd = gu.make_dev_dia(S)
+    L.cuvdia_set_path(_lib.PATH_TILED)
+    try:
+        xs = torch.zeros(32, 19, device="cuda:0")
+        ys = torch.zeros(32, 36, device="cuda:0")
+        assert L.cuvdia_spmm_f32(Sd.desc, Sd.vec.data_ptr(), xs.data_ptr(), 19, ys.data_ptr(), 36, 32, b"n", 1.0, 0.0, sp) == _lib.EUNSUPPORTED
+    finally:
+        L.cuvdia_set_path(_lib.PATH_AUTO)
+
+
+def test_offsets_entry_points_use_the_cache(oracle, gu):
+    import ctypes
+    import torch
+    from cuv_amd import _lib, dia as D
+    L = _lib.lib()
+    rng = np.random.default_rng(21)
+    A = _rand_dia(oracle, rng, 128, 96, [-2, 0, 1, 30])
+    B = np.asfortranarray(rng.uniform(-1, 1, (96, 32)).astype(np.float32))
+    vals = torch.from_numpy(A.vals).cuda()
+    Bd = D.to_device_colmajor(B)
+    out = torch.full((32, 128), float("nan"), device="cuda:0")
+    ip = ctypes.POINTER(ctypes.c_int)
+    for _ in range(3):
+        rc = L.cuvdia_spmm_offsets_f32(vals.data_ptr(), A.offsets.ctypes.data_as(ip), A.nd, A.stride, A.h, A.w, 1,
+                                       Bd.data_ptr(), 96, out.data_ptr(), 128, 32, b"n", 1.0, 0.0, None)
+        assert rc == 0
+    torch.cuda.synchronize()
+    gu.assert_close_mag(D.to_host_colmajor(out), oracle.prod(A, B), oracle.prod_mag(A, B), "offsets form")
+    C = _rand_dia(oracle, rng, 128, 96, [-2, 0, 1, 30], pad=5.0)
+    Ah = np.asfortranarray(rng.uniform(-1, 1, (128, 32)).astype(np.float32))
+    cv = torch.from_numpy(C.vals).cuda()
+    rc = L.cuvdia_dd2dia_offsets_f32(cv.data_ptr(), C.offsets.ctypes.data_as(ip), C.nd, C.stride, C.h, C.w, 1,
+                                     D.to_device_colmajor(Ah).data_ptr(), 128, Bd.data_ptr(), 96, 32, 0.5, 0.25, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = oracle.dd2dia(C, Ah, B, 0.5, 0.25)
+    np.testing.assert_allclose(cv.cpu().numpy(), ref, rtol=1e-5, atol=1e-6)
+    assert L.cuvdia_cache_clear() == 0
+
+
+# ------------------------------------------------- the measured workloads ---
+def _o_dia(oracle, wl):
+    p = wl.pattern
+    return oracle.Dia(p.h, p.w, p.offsets, p.stride, p.rf, wl.vals)
+
+
+def test_cfg0_spmv(oracle, gu):
+    from cuv_amd import workloads as W
+    for trans in ("n", "t"):
+        wl = W.cfg0(trans)
+        for path in _paths(1):
+            gu.check_prod(oracle, _o_dia(oracle, wl), wl.X, None, trans, 1.0, 0.0, path, wl.name)
+
+
+def test_cfg1_up_pass(oracle, gu):
+    from cuv_amd import workloads as W, _lib
+    wl = W.cfg1()
+    _, ran = gu.check_prod(oracle, _o_dia(oracle, wl), wl.X, None, "n", 1.0, 0.0, _lib.PATH_AUTO, wl.name)
+    assert ran == _lib.PATH_TILED
+
+
+def test_cfg2_down_pass(oracle, gu):
+    from cuv_amd import workloads as W, _lib
+    wl = W.cfg2()
+    _, ran = gu.check_prod(oracle, _o_dia(oracle, wl), wl.X, wl.dst, "t", 1.0, 0.5, _lib.PATH_AUTO, wl.name)
+    assert ran == _lib.PATH_TILED
+
+
+def test_cfg3_weight_gradient(oracle, gu):
+    from cuv_amd import workloads as W, _lib
+    wl = W.cfg3()
+    _, ran = gu.check_dd2dia(oracle, _o_dia(oracle, wl), wl.A, wl.B, wl.alpha, wl.beta, _lib.PATH_AUTO, wl.name)
+    assert ran == _lib.PATH_TILED
+
+
+def test_cfg1_generic_matches_too(oracle, gu):
+    from cuv_amd import workloads as W, _lib
+    wl = W.cfg1()
+    gu.check_prod(oracle, _o_dia(oracle, wl), wl.X[:, :16], None, "n", 1.0, 0.0, _lib.PATH_GENERIC, "cfg1 generic")
+    wl3 = W.cfg3()
+    gu.check_dd2dia(oracle, _o_dia(oracle, wl3), wl3.A[:, :24], wl3.B[:, :24], 1.0 / 24, 0.9, _lib.PATH_GENERIC, "cfg3 generic")
+
+
+def test_cfg4_reduced_multichannel(oracle, gu):
+    """The large layer's offset structure (4 channel shifts x 13x13 window) at a
+    map size the oracle finishes in seconds: 64x64x4 rows, batch 72."""
+    from cuv_amd import workloads as W, _lib
+    for trans in ("n", "t"):
+        wl = W.cfg4("spmm", trans, px=64, batch=72)
+        gu.check_prod(oracle, _o_dia(oracle, wl), wl.X, None, trans, 1.0, 0.0, _lib.PATH_TILED, wl.name)
+    wl = W.cfg4("dd2dia", px=64, batch=72, beta=0.9)
+    gu.check_dd2dia(oracle, _o_dia(oracle, wl), wl.A, wl.B, 1.0 / 72, 0.9, _lib.PATH_TILED, wl.name)
