@@ -173,7 +173,10 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     d->view = DiaView{h, w, nd, stride, row_fact,
                       reinterpret_cast<const int *>(base),
                       reinterpret_cast<const Chunk *>(base + off_bytes), d->n_chunks_n,
-                      reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t};
+                      reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t,
+                      0, 0};
+    for (const Chunk &c : cn) d->view.max_len_n = std::max(d->view.max_len_n, c.len);
+    for (const Chunk &c : ct) d->view.max_len_t = std::max(d->view.max_len_t, c.len);
     *out = d;
     return CUVDIA_OK;
 }

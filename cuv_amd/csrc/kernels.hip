@@ -27,12 +27,10 @@ namespace cuvdia {
 namespace {
 
 // Loads through this address space are issued on the scalar unit when the
-// address is wave-uniform: diagonal values and the chunk table reach the
-// FMAs as SGPR operands and cost no vector-memory or LDS bandwidth.
-typedef const float __attribute__((address_space(4))) *sc_float_ptr;
+// address is wave-uniform: the chunk table is read into SGPRs and costs no
+// vector-memory or LDS bandwidth.
 typedef const Chunk __attribute__((address_space(4))) *sc_chunk_ptr;
 
-__device__ __forceinline__ sc_float_ptr scalar_ptr(const float *p) { return (sc_float_ptr)p; }
 __device__ __forceinline__ sc_chunk_ptr scalar_ptr(const Chunk *p) { return (sc_chunk_ptr)p; }
 
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and each
@@ -142,36 +140,97 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 
 // -------------------------------------------------------------- tiled spmm --
 //
-// Workgroup = 64 output rows x 64 batch columns, WAVES waves of T = 64/WAVES
-// rows each.  Lane l of every wave owns batch column col0 + l and T running
-// sums.  Per run chunk (<= 8 consecutive shifts starting at s0):
+// Workgroup = 64 output rows x 64 batch columns, 4 waves of 16 rows each.
+// Lane l of every wave owns batch column col0 + l and 16 running sums.  Per
+// run chunk (<= 8 consecutive shifts starting at s0):
 //   1. the dense rows [row0 + s0, row0 + s0 + 72) of the 64 columns are
 //      loaded with lanes along rows (coalesced 256-byte segments) and written
-//      to LDS column by column, pitch 76 floats;
-//   2. each lane reads its column's window of T + len - 1 values with 16-byte
+//      to LDS column by column, pitch 76 floats; each wave also loads the
+//      chunk's diagonal values for its 16 rows (8 x 16 floats) and parks them
+//      in LDS.  Loads use clamped addresses and what was out of range (rows,
+//      columns, diagonal slots) is written to LDS as 0, so the arithmetic
+//      below needs no guards and never sees padding;
+//   2. each lane reads its column's window of 16 + len - 1 values with 16-byte
 //      LDS reads (pitch/4 is odd, so the 64 lanes spread over all banks);
-//   3. for each diagonal j and row t: acc[t] = fma(A_j[row], win[t + j], acc[t])
-//      where A_j[row] is wave-uniform and arrives as an SGPR operand.
-// The next chunk's global loads are issued before the FMAs of the current one
-// and written to the other LDS buffer afterwards (one barrier per chunk).
+//      Every chunk is processed as LCK diagonals, LCK = the longest chunk of
+//      the table (template parameter); shorter chunks carry zeros;
+//   3. for each diagonal j the wave reads A_j[16 rows] into one VGPR (lane & 15
+//      selects the row) and issues 16 FMAs whose first operand is that VGPR
+//      broadcast within each 16-lane row by DPP (row_newbcast:t):
+//          acc[t] = fma(A_j[row t], win[t + j], acc[t]).
+// Global loads run two chunks ahead of the FMAs: one chunk in flight in
+// registers, one staged in the other LDS buffer (one barrier per chunk).
 // The epilogue transposes the sums through LDS so the store to dst is again
 // lanes-along-rows.
 
 constexpr int SP_ROWS = 64;        // output rows per workgroup
 constexpr int SP_COLS = 64;        // batch columns per workgroup (one per lane)
-constexpr int SP_STAGED = 72;      // rows staged per chunk: 64 + CHUNK_MAX
+constexpr int SP_WAVES = 4;
+constexpr int SP_T = 16;           // rows per wave == lanes per DPP row
 constexpr int SP_PITCH = 76;       // floats between staged columns
 constexpr int SP_OPITCH = 68;      // floats between columns in the epilogue
+constexpr int SP_CPW = SP_COLS / SP_WAVES;      // columns each wave stages
+constexpr int SP_HALO = SP_CPW / 8;             // halo loads per wave (8 rows x 8 columns each)
+constexpr int SP_AVALS = CHUNK_MAX * SP_T;      // diagonal values per wave per chunk
+constexpr int SP_STAGE_FLOATS = SP_COLS * SP_PITCH + SP_WAVES * SP_AVALS;
 
-template <int T, int LC, bool GUARD>
-__device__ __forceinline__ void spmm_chunk(float (&acc)[T], const float *win_lds,
-                                           sc_float_ptr vals, sc_chunk_ptr ck, int s0,
-                                           long long stride, long long arow, int ashift,
-                                           int n_out, int n_in)
+struct SpStage {
+    float x[SP_CPW + SP_HALO];
+    float a[SP_AVALS / 64];
+};
+
+// acc[t] += bcast_t(a) * win[t + J], t = 0..15.  The DPP operand must not have
+// been written by a VALU instruction in the two preceding issue slots; the
+// leading s_nop covers whatever the compiler placed before each block.
+template <int J, int N>
+__device__ __forceinline__ void fma_row16(float (&acc)[SP_T], float a, const float (&win)[N])
 {
-    constexpr int WIN = T + LC - 1;
+    asm(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %8, %9 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %1, %8, %10 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %2, %8, %11 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %3, %8, %12 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %4, %8, %13 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %5, %8, %14 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %6, %8, %15 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %7, %8, %16 row_newbcast:7 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]),
+          "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+        : "v"(a), "v"(win[J + 0]), "v"(win[J + 1]), "v"(win[J + 2]), "v"(win[J + 3]),
+          "v"(win[J + 4]), "v"(win[J + 5]), "v"(win[J + 6]), "v"(win[J + 7]));
+    asm(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %8, %9 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %1, %8, %10 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %2, %8, %11 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %3, %8, %12 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %4, %8, %13 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %5, %8, %14 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %6, %8, %15 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %7, %8, %16 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc[8]), "+v"(acc[9]), "+v"(acc[10]), "+v"(acc[11]),
+          "+v"(acc[12]), "+v"(acc[13]), "+v"(acc[14]), "+v"(acc[15])
+        : "v"(a), "v"(win[J + 8]), "v"(win[J + 9]), "v"(win[J + 10]), "v"(win[J + 11]),
+          "v"(win[J + 12]), "v"(win[J + 13]), "v"(win[J + 14]), "v"(win[J + 15]));
+}
+
+template <int LC, int J, int N>
+__device__ __forceinline__ void spmm_rows(float (&acc)[SP_T], const float (&a)[LC], const float (&win)[N])
+{
+    if constexpr (J < LC) {
+        fma_row16<J>(acc, a[J], win);
+        spmm_rows<LC, J + 1>(acc, a, win);
+    }
+}
+
+template <int LC>
+__device__ __forceinline__ void spmm_chunk(float (&acc)[SP_T], const float *win_lds, const float *a_lds)
+{
+    constexpr int WIN = SP_T + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
     float win[WQ * 4];
+    float a[LC];
     const float4 *p4 = reinterpret_cast<const float4 *>(win_lds);
 #pragma unroll
     for (int q = 0; q < WQ; ++q) {
@@ -179,35 +238,17 @@ __device__ __forceinline__ void spmm_chunk(float (&acc)[T], const float *win_lds
         win[4 * q + 0] = v.x; win[4 * q + 1] = v.y; win[4 * q + 2] = v.z; win[4 * q + 3] = v.w;
     }
 #pragma unroll
-    for (int j = 0; j < LC; ++j) {
-        const long long abase = (long long)ck->slot[j] * stride + arow + (ashift ? s0 + j : 0);
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            float a;
-            if (!GUARD) {
-                a = vals[abase + t];
-            } else {
-                const long long o = arow + t;
-                const long long in = o + s0 + j;
-                const bool ok = (o < n_out) & (in >= 0) & (in < n_in);
-                a = vals[ok ? abase + t : 0];
-                a = ok ? a : 0.f;
-            }
-            acc[t] = __builtin_fmaf(a, win[t + j], acc[t]);
-        }
-    }
+    for (int j = 0; j < LC; ++j) a[j] = a_lds[j * SP_T];
+    spmm_rows<LC, 0>(acc, a, win);
 }
 
-template <int T, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void spmm_tiled_kernel(
+template <int LCK>
+__global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles)
 {
-    static_assert(T * WAVES == SP_ROWS, "a workgroup covers 64 rows");
-    constexpr int CPW = SP_COLS / WAVES;        // columns each wave stages
-    constexpr int HALO = (CPW + 7) / 8;         // halo loads per wave (8 rows x 8 columns each)
-    __shared__ __attribute__((aligned(16))) float lds[2][SP_COLS * SP_PITCH];
+    __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -216,91 +257,105 @@ __global__ __launch_bounds__(64 * WAVES) void spmm_tiled_kernel(
     const int row0 = rowtile * SP_ROWS;
     const int col0 = (tile - rowtile * col_tiles) * SP_COLS;
     const sc_chunk_ptr cks = scalar_ptr(chunks);
-    const sc_float_ptr svals = scalar_ptr(vals);
 
-    float acc[T];
+    float acc[SP_T];
 #pragma unroll
-    for (int t = 0; t < T; ++t) acc[t] = 0.f;
-    float pre[CPW + HALO];
+    for (int t = 0; t < SP_T; ++t) acc[t] = 0.f;
 
     const int hcol = lane >> 3, hrow = SP_ROWS + (lane & 7);
+    const long long arow = (long long)row0 + wave * SP_T + (lane & 15);   // this lane's diagonal-value row
+    const int aj = lane >> 4;                                              // and diagonal (plus 4 per pass)
 
-    auto issue = [&](int c) {
-        const long long base = (long long)row0 + cks[c].s0;
-        const bool interior = (base >= 0) & (base + SP_STAGED <= n_in) & (col0 + SP_COLS <= batch);
-        if (interior) {
-#pragma unroll
-            for (int q = 0; q < CPW; ++q)
-                pre[q] = X[(long long)(col0 + wave * CPW + q) * ldx + base + lane];
-#pragma unroll
-            for (int q = 0; q < HALO; ++q) {
-                const int col = wave * CPW + q * 8 + hcol;
-                pre[CPW + q] = (q * 8 + hcol < CPW) ? X[(long long)(col0 + col) * ldx + base + hrow] : 0.f;
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < CPW; ++q) {
-                const int col = col0 + wave * CPW + q;
-                const long long r = base + lane;
-                pre[q] = (col < batch && r >= 0 && r < n_in) ? X[(long long)col * ldx + r] : 0.f;
-            }
-#pragma unroll
-            for (int q = 0; q < HALO; ++q) {
-                const int col = col0 + wave * CPW + q * 8 + hcol;
-                const long long r = base + hrow;
-                pre[CPW + q] = (q * 8 + hcol < CPW && col < batch && r >= 0 && r < n_in)
-                                   ? X[(long long)col * ldx + r] : 0.f;
-            }
-        }
-    };
-    auto commit = [&](float *buf) {
-#pragma unroll
-        for (int q = 0; q < CPW; ++q) buf[(wave * CPW + q) * SP_PITCH + lane] = pre[q];
-#pragma unroll
-        for (int q = 0; q < HALO; ++q)
-            if (q * 8 + hcol < CPW) buf[(wave * CPW + q * 8 + hcol) * SP_PITCH + hrow] = pre[CPW + q];
-    };
-
-    issue(0);
-    commit(lds[0]);
-    __syncthreads();
-
-    const long long arow = (long long)row0 + wave * T;
-    for (int c = 0; c < nchunks; ++c) {
-        const bool more = c + 1 < nchunks;
-        if (more) issue(c + 1);
-
-        const sc_chunk_ptr ck = cks + c;
-        const int s0 = ck->s0;
-        const int len = ck->len;
-        const float *win_lds = &lds[c & 1][lane * SP_PITCH + wave * T];
+    // Every load below uses an address clamped into its operand, so it can be
+    // issued unconditionally and back to back; what was out of range is
+    // replaced by 0 when the stage is written to LDS.
+    const int a_rows = ashift ? n_in : n_out;          // rows of a stored diagonal
+    auto issue = [&](int c, SpStage &st) {
+        const int s0 = cks[c].s0;
         const long long base = (long long)row0 + s0;
-        const bool interior = (base >= 0) & (base + SP_STAGED <= n_in) & (row0 + SP_ROWS <= n_out);
-#define CUVDIA_SPMM_CASE(L)                                                                   \
-        case L:                                                                               \
-            if (interior) spmm_chunk<T, L, false>(acc, win_lds, svals, ck, s0, stride, arow, ashift, n_out, n_in); \
-            else          spmm_chunk<T, L, true >(acc, win_lds, svals, ck, s0, stride, arow, ashift, n_out, n_in); \
-            break;
-        switch (len) {
-            CUVDIA_SPMM_CASE(1) CUVDIA_SPMM_CASE(2) CUVDIA_SPMM_CASE(3) CUVDIA_SPMM_CASE(4)
-            CUVDIA_SPMM_CASE(5) CUVDIA_SPMM_CASE(6) CUVDIA_SPMM_CASE(7) CUVDIA_SPMM_CASE(8)
-            default: break;
+        const long long r_main = min(max(base + lane, 0LL), (long long)n_in - 1);
+        const long long r_halo = min(max(base + hrow, 0LL), (long long)n_in - 1);
+#pragma unroll
+        for (int q = 0; q < SP_CPW; ++q) {
+            const int col = min(col0 + wave * SP_CPW + q, batch - 1);
+            st.x[q] = X[(long long)col * ldx + r_main];
         }
-#undef CUVDIA_SPMM_CASE
-        if (more) commit(lds[(c + 1) & 1]);
+#pragma unroll
+        for (int q = 0; q < SP_HALO; ++q) {
+            const int col = min(col0 + wave * SP_CPW + q * 8 + hcol, batch - 1);
+            st.x[SP_CPW + q] = X[(long long)col * ldx + r_halo];
+        }
+        // diagonal values: lane -> (diagonal aj + 4*q of the chunk, row arow);
+        // the slot table comes through the scalar unit and is selected per lane
+#pragma unroll
+        for (int q = 0; q < SP_AVALS / 64; ++q) {
+            const int sl0 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 0]);
+            const int sl1 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 1]);
+            const int sl2 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 2]);
+            const int sl3 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 3]);
+            const int sl = aj < 2 ? (aj == 0 ? sl0 : sl1) : (aj == 2 ? sl2 : sl3);
+            const long long ar = ashift ? arow + s0 + aj + 4 * q : arow;
+            st.a[q] = vals[(long long)sl * stride + min(max(ar, 0LL), (long long)a_rows - 1)];
+        }
+    };
+    auto commit = [&](int c, const SpStage &st, float *buf) {
+        const int s0 = cks[c].s0;
+        const int len = cks[c].len;
+        const long long base = (long long)row0 + s0;
+        const bool main_ok = (base + lane >= 0) & (base + lane < n_in);
+        const bool halo_ok = (base + hrow >= 0) & (base + hrow < n_in);
+#pragma unroll
+        for (int q = 0; q < SP_CPW; ++q) {
+            const bool ok = main_ok & (col0 + wave * SP_CPW + q < batch);
+            buf[(wave * SP_CPW + q) * SP_PITCH + lane] = ok ? st.x[q] : 0.f;
+        }
+#pragma unroll
+        for (int q = 0; q < SP_HALO; ++q) {
+            const bool ok = halo_ok & (col0 + wave * SP_CPW + q * 8 + hcol < batch);
+            buf[(wave * SP_CPW + q * 8 + hcol) * SP_PITCH + hrow] = ok ? st.x[SP_CPW + q] : 0.f;
+        }
+#pragma unroll
+        for (int q = 0; q < SP_AVALS / 64; ++q) {
+            const int j = aj + 4 * q;
+            const long long in = arow + s0 + j;
+            const bool ok = (j < len) & (arow < n_out) & (in >= 0) & (in < n_in);
+            buf[SP_COLS * SP_PITCH + wave * SP_AVALS + q * 64 + lane] = ok ? st.a[q] : 0.f;
+        }
+    };
+    auto compute = [&](const float *buf) {
+        const float *win_lds = buf + lane * SP_PITCH + wave * SP_T;
+        const float *a_lds = buf + SP_COLS * SP_PITCH + wave * SP_AVALS + (lane & 15);
+        spmm_chunk<LCK>(acc, win_lds, a_lds);
+    };
+    // chunk c is computed from lds[c & 1] while chunk c+1 lands in `next` and
+    // chunk c+2 is requested into `fresh`
+    auto iteration = [&](int c, SpStage &fresh, SpStage &next) {
+        if (c + 2 < nchunks) issue(c + 2, fresh);
+        compute(lds[c & 1]);
+        if (c + 1 < nchunks) commit(c + 1, next, lds[(c + 1) & 1]);
         __syncthreads();
+    };
+
+    SpStage s0, s1;
+    issue(0, s0);
+    if (nchunks > 1) issue(1, s1);
+    commit(0, s0, lds[0]);
+    __syncthreads();
+    for (int c = 0; c < nchunks; c += 2) {
+        iteration(c, s0, s1);
+        if (c + 1 < nchunks) iteration(c + 1, s1, s0);
     }
 
     // epilogue: lanes-along-columns -> lanes-along-rows through LDS
     float *out = &lds[0][0];
 #pragma unroll
-    for (int t = 0; t < T; ++t) out[lane * SP_OPITCH + wave * T + t] = acc[t];
+    for (int t = 0; t < SP_T; ++t) out[lane * SP_OPITCH + wave * SP_T + t] = acc[t];
     __syncthreads();
     const long long row = (long long)row0 + lane;
     if (row < n_out) {
 #pragma unroll
-        for (int q = 0; q < CPW; ++q) {
-            const int col = wave * CPW + q;
+        for (int q = 0; q < SP_CPW; ++q) {
+            const int col = wave * SP_CPW + q;
             if (col0 + col < batch) {
                 const float v = out[col * SP_OPITCH + lane];
                 float *y = Y + (long long)(col0 + col) * ldy + row;
@@ -507,10 +562,20 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     if (row_tiles * col_tiles > 0x7fffffffLL) return hipErrorInvalidValue;
     const Chunk *chunks = trans ? A.chunks_t_dev : A.chunks_n_dev;
     const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
-    constexpr int T = 16, WAVES = 4;
-    hipLaunchKernelGGL((spmm_tiled_kernel<T, WAVES>), dim3((unsigned)(row_tiles * col_tiles)),
-                       dim3(64 * WAVES), 0, stream, chunks, nchunks, vals, A.stride, trans ? 1 : 0,
-                       B, ldb, dst, ldd, n_out, n_in, batch, alpha, beta, (int)col_tiles);
+    const int lck = trans ? A.max_len_t : A.max_len_n;
+    const dim3 grid((unsigned)(row_tiles * col_tiles)), block(64 * SP_WAVES);
+#define CUVDIA_SPMM_LAUNCH(L)                                                                       \
+    case L:                                                                                         \
+        hipLaunchKernelGGL(spmm_tiled_kernel<L>, grid, block, 0, stream, chunks, nchunks, vals,     \
+                           A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha,    \
+                           beta, (int)col_tiles);                                                   \
+        break;
+    switch (lck) {
+        CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
+        CUVDIA_SPMM_LAUNCH(5) CUVDIA_SPMM_LAUNCH(6) CUVDIA_SPMM_LAUNCH(7) CUVDIA_SPMM_LAUNCH(8)
+        default: return hipErrorInvalidValue;
+    }
+#undef CUVDIA_SPMM_LAUNCH
     return hipGetLastError();
 }
 

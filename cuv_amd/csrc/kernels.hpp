@@ -15,6 +15,7 @@ struct DiaView {
     int n_chunks_n;
     const Chunk *chunks_t_dev;   // shifts = -offsets
     int n_chunks_t;
+    int max_len_n, max_len_t;    // longest chunk of each table
 };
 
 // dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch
