@@ -142,24 +142,30 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 //
 // Workgroup = 64 output rows x 64 batch columns, 4 waves of 16 rows each.
 // Lane l of every wave owns batch column col0 + l and 16 running sums.  Per
-// run chunk (<= 8 consecutive shifts starting at s0):
-//   1. the dense rows [row0 + s0, row0 + s0 + 72) of the 64 columns are
-//      loaded with lanes along rows (coalesced 256-byte segments) and written
-//      to LDS column by column, pitch 76 floats; each wave also loads the
-//      chunk's diagonal values for its 16 rows (8 x 16 floats) and parks them
-//      in LDS.  Loads use clamped addresses and what was out of range (rows,
-//      columns, diagonal slots) is written to LDS as 0, so the arithmetic
+// run chunk (<= 8 consecutive shifts starting at s0, s0 = M mod 4 for every
+// chunk of the table):
+//   1. the dense rows [a0, a0 + 80), a0 = row0 + s0 - M (a multiple of 4), of
+//      the 64 columns are fetched with 16-byte buffer loads, 20 lanes per
+//      column and 3 columns per instruction, so every cache line of a column
+//      is requested by one instruction only, and written to LDS with 16-byte
+//      stores, columns 84 floats apart.  Each wave also fetches two of the
+//      chunk's eight diagonals for all 64 rows (one 256-byte row segment per
+//      instruction) and parks them in LDS.  Rows outside the operand and
+//      diagonal slots outside the matrix become zeros (out-of-range buffer
+//      offsets, plus a masked write on boundary tiles), so the arithmetic
 //      below needs no guards and never sees padding;
-//   2. each lane reads its column's window of 16 + len - 1 values with 16-byte
-//      LDS reads (pitch/4 is odd, so the 64 lanes spread over all banks);
-//      Every chunk is processed as LCK diagonals, LCK = the longest chunk of
-//      the table (template parameter); shorter chunks carry zeros;
+//   2. each lane reads its column's window of 16 + LCK - 1 + M values with
+//      16-byte LDS reads (pitch/4 is odd, so the 64 lanes spread over all
+//      banks).  Every chunk is processed as LCK diagonals, LCK = the longest
+//      chunk of the table; shorter chunks carry zeros;
 //   3. for each diagonal j the wave reads A_j[16 rows] into one VGPR (lane & 15
 //      selects the row) and issues 16 FMAs whose first operand is that VGPR
 //      broadcast within each 16-lane row by DPP (row_newbcast:t):
-//          acc[t] = fma(A_j[row t], win[t + j], acc[t]).
-// Global loads run two chunks ahead of the FMAs: one chunk in flight in
-// registers, one staged in the other LDS buffer (one barrier per chunk).
+//          acc[t] = fma(A_j[row t], win[t + j + M], acc[t]).
+// The loop is software-pipelined three chunks deep: while the FMAs of chunk c
+// run out of registers, chunk c+1 is being written to the other LDS buffer
+// (its window is read right after the barrier), chunk c+2 is in flight from
+// memory and chunk c+3 has just been requested.
 // The epilogue transposes the sums through LDS so the store to dst is again
 // lanes-along-rows.
 
@@ -167,21 +173,43 @@ constexpr int SP_ROWS = 64;        // output rows per workgroup
 constexpr int SP_COLS = 64;        // batch columns per workgroup (one per lane)
 constexpr int SP_WAVES = 4;
 constexpr int SP_T = 16;           // rows per wave == lanes per DPP row
-constexpr int SP_PITCH = 76;       // floats between staged columns
+constexpr int SP_QUADS = 20;       // 16-byte pieces staged per column (80 rows)
+constexpr int SP_CPI = 3;          // columns per load instruction (3 x 20 lanes)
+constexpr int SP_GROUPS = (SP_COLS + SP_CPI - 1) / SP_CPI;             // 22 column groups
+constexpr int SP_LOADS = (SP_GROUPS + SP_WAVES - 1) / SP_WAVES;        // 6 per wave per chunk
+constexpr int SP_PITCH = 84;       // floats between staged columns
 constexpr int SP_OPITCH = 68;      // floats between columns in the epilogue
-constexpr int SP_CPW = SP_COLS / SP_WAVES;      // columns each wave stages
-constexpr int SP_HALO = SP_CPW / 8;             // halo loads per wave (8 rows x 8 columns each)
-constexpr int SP_AVALS = CHUNK_MAX * SP_T;      // diagonal values per wave per chunk
-constexpr int SP_STAGE_FLOATS = SP_COLS * SP_PITCH + SP_WAVES * SP_AVALS;
+constexpr int SP_CPW = SP_COLS / SP_WAVES;      // columns each wave stores in the epilogue
+constexpr int SP_XFLOATS = SP_COLS * SP_PITCH;
+constexpr int SP_AVALS = CHUNK_MAX * SP_ROWS;   // diagonal values per workgroup per chunk
+constexpr int SP_DUMP = SP_XFLOATS + SP_AVALS;  // where idle lanes write
+constexpr int SP_STAGE_FLOATS = SP_DUMP + 4;
+constexpr int SP_APW = CHUNK_MAX / SP_WAVES;    // diagonals each wave fetches per chunk
 
 struct SpStage {
-    float x[SP_CPW + SP_HALO];
-    float a[SP_AVALS / 64];
+    float4 x[SP_LOADS];
+    float a[SP_APW];
+    int rows_ok;            // bit k: dense row of x[].k exists
+    bool edge;              // some staged row does not exist (wave-uniform)
+};
+
+// One chunk-table entry as a wave needs it: shift, length, and the table
+// positions of the two diagonals this wave fetches.
+struct SpInfo {
+    int s0, len;
+    int slot[SP_APW];
+};
+
+template <int LCK, int M>
+struct SpWindow {
+    static constexpr int WQ = (SP_T + LCK - 1 + M + 3) / 4;
+    float w[WQ * 4];
+    float a[LCK];
 };
 
 // acc[t] += bcast_t(a) * win[t + J], t = 0..15.  The DPP operand must not have
 // been written by a VALU instruction in the two preceding issue slots; the
-// leading s_nop covers whatever the compiler placed before each block.
+// leading s_nop covers whatever the compiler placed before the block.
 template <int J, int N>
 __device__ __forceinline__ void fma_row16(float (&acc)[SP_T], float a, const float (&win)[N])
 {
@@ -215,38 +243,53 @@ __device__ __forceinline__ void fma_row16(float (&acc)[SP_T], float a, const flo
           "v"(win[J + 12]), "v"(win[J + 13]), "v"(win[J + 14]), "v"(win[J + 15]));
 }
 
-template <int LC, int J, int N>
-__device__ __forceinline__ void spmm_rows(float (&acc)[SP_T], const float (&a)[LC], const float (&win)[N])
+template <int LCK, int M, int J>
+__device__ __forceinline__ void spmm_rows(float (&acc)[SP_T], const SpWindow<LCK, M> &win)
 {
-    if constexpr (J < LC) {
-        fma_row16<J>(acc, a[J], win);
-        spmm_rows<LC, J + 1>(acc, a, win);
+    if constexpr (J < LCK) {
+        fma_row16<J + M>(acc, win.a[J], win.w);
+        spmm_rows<LCK, M, J + 1>(acc, win);
     }
 }
 
-template <int LC>
-__device__ __forceinline__ void spmm_chunk(float (&acc)[SP_T], const float *win_lds, const float *a_lds)
+template <int LCK, int M>
+__device__ __forceinline__ void spmm_read_window(SpWindow<LCK, M> &win, const float *win_lds,
+                                                 const float *a_lds)
 {
-    constexpr int WIN = SP_T + LC - 1;
-    constexpr int WQ = (WIN + 3) / 4;
-    float win[WQ * 4];
-    float a[LC];
     const float4 *p4 = reinterpret_cast<const float4 *>(win_lds);
 #pragma unroll
-    for (int q = 0; q < WQ; ++q) {
+    for (int q = 0; q < SpWindow<LCK, M>::WQ; ++q) {
         const float4 v = p4[q];
-        win[4 * q + 0] = v.x; win[4 * q + 1] = v.y; win[4 * q + 2] = v.z; win[4 * q + 3] = v.w;
+        win.w[4 * q + 0] = v.x; win.w[4 * q + 1] = v.y; win.w[4 * q + 2] = v.z; win.w[4 * q + 3] = v.w;
     }
 #pragma unroll
-    for (int j = 0; j < LC; ++j) a[j] = a_lds[j * SP_T];
-    spmm_rows<LC, 0>(acc, a, win);
+    for (int j = 0; j < LCK; ++j) win.a[j] = a_lds[j * SP_ROWS];
 }
 
-template <int LCK>
+// Buffer resource over [base, base + bytes): loads take a 32-bit VGPR byte
+// offset, and an offset at or beyond `bytes` makes the hardware return 0
+// instead of touching memory -- which is how rows before the operand, rows
+// past its end and diagonal slots outside the matrix become zeros without a
+// compare-and-select per load.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t r, unsigned voff)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, 0, 0));
+}
+__device__ __forceinline__ float4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned voff)
+{
+    return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+}
+constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used here
+
+template <int LCK, int M>
 __global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
-    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles)
+    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes)
 {
     __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
 
@@ -256,97 +299,137 @@ __global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
     const int rowtile = tile / col_tiles;
     const int row0 = rowtile * SP_ROWS;
     const int col0 = (tile - rowtile * col_tiles) * SP_COLS;
-    const sc_chunk_ptr cks = scalar_ptr(chunks);
-
     float acc[SP_T];
 #pragma unroll
     for (int t = 0; t < SP_T; ++t) acc[t] = 0.f;
 
-    const int hcol = lane >> 3, hrow = SP_ROWS + (lane & 7);
-    const long long arow = (long long)row0 + wave * SP_T + (lane & 15);   // this lane's diagonal-value row
-    const int aj = lane >> 4;                                              // and diagonal (plus 4 per pass)
+    // dense operand: resource from this tile's first column to the end of the
+    // last valid column, so nothing outside the operand is ever touched.
+    // Columns past the batch are replaced by the last valid one (their sums
+    // are never stored).
+    const int cols_here = min(SP_COLS, batch - col0);
+    const __amdgpu_buffer_rsrc_t xr =
+        make_rsrc(X + (long long)col0 * ldx, (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4));
+    const int grp = lane / SP_QUADS;               // column within the instruction's group (3: idle lane)
+    const int quad = lane - grp * SP_QUADS;        // 16-byte piece within the column
+    unsigned col_off[SP_LOADS];                    // byte offset of this lane's column per load
+    int lds_at[SP_LOADS];                          // float index in the stage buffer it is written to
+#pragma unroll
+    for (int it = 0; it < SP_LOADS; ++it) {
+        const int col = (wave + SP_WAVES * it) * SP_CPI + grp;
+        const bool live = (grp < SP_CPI) & (col < SP_COLS);
+        col_off[it] = live ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) : OOB_OFFSET;
+        lds_at[it] = live ? col * SP_PITCH + 4 * quad : SP_DUMP;
+    }
+    // diagonal values: wave w fetches diagonals w and w + 4 of the chunk for
+    // the workgroup's 64 rows
+    const __amdgpu_buffer_rsrc_t ar = make_rsrc(vals, a_bytes);
+    const int arow = row0 + lane;
 
-    // Every load below uses an address clamped into its operand, so it can be
-    // issued unconditionally and back to back; what was out of range is
-    // replaced by 0 when the stage is written to LDS.
-    const int a_rows = ashift ? n_in : n_out;          // rows of a stored diagonal
-    auto issue = [&](int c, SpStage &st) {
-        const int s0 = cks[c].s0;
-        const long long base = (long long)row0 + s0;
-        const long long r_main = min(max(base + lane, 0LL), (long long)n_in - 1);
-        const long long r_halo = min(max(base + hrow, 0LL), (long long)n_in - 1);
+    // The chunk table is read with vector loads at wave-uniform addresses, one
+    // chunk ahead of its use.  Scalar loads would share a counter with the
+    // LDS traffic and can only be waited for by draining it, which would
+    // serialise the LDS writes, the window reads and the FMAs of every
+    // iteration; vector loads retire in order and are waited for exactly.
+    const __amdgpu_buffer_rsrc_t cr = make_rsrc(chunks, (unsigned)nchunks * (unsigned)sizeof(Chunk));
+    auto fetch_info = [&](int c, SpInfo &info) {
+        const unsigned base = (unsigned)min(c, nchunks - 1) * (unsigned)sizeof(Chunk);
+        const auto sl = __builtin_amdgcn_raw_buffer_load_b64(cr, base, 0, 0);
+        info.s0 = sl[0];
+        info.len = sl[1];
 #pragma unroll
-        for (int q = 0; q < SP_CPW; ++q) {
-            const int col = min(col0 + wave * SP_CPW + q, batch - 1);
-            st.x[q] = X[(long long)col * ldx + r_main];
-        }
-#pragma unroll
-        for (int q = 0; q < SP_HALO; ++q) {
-            const int col = min(col0 + wave * SP_CPW + q * 8 + hcol, batch - 1);
-            st.x[SP_CPW + q] = X[(long long)col * ldx + r_halo];
-        }
-        // diagonal values: lane -> (diagonal aj + 4*q of the chunk, row arow);
-        // the slot table comes through the scalar unit and is selected per lane
-#pragma unroll
-        for (int q = 0; q < SP_AVALS / 64; ++q) {
-            const int sl0 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 0]);
-            const int sl1 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 1]);
-            const int sl2 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 2]);
-            const int sl3 = __builtin_amdgcn_readfirstlane(cks[c].slot[4 * q + 3]);
-            const int sl = aj < 2 ? (aj == 0 ? sl0 : sl1) : (aj == 2 ? sl2 : sl3);
-            const long long ar = ashift ? arow + s0 + aj + 4 * q : arow;
-            st.a[q] = vals[(long long)sl * stride + min(max(ar, 0LL), (long long)a_rows - 1)];
-        }
+        for (int q = 0; q < SP_APW; ++q)
+            info.slot[q] = __builtin_amdgcn_raw_buffer_load_b32(cr, base + 8u + 4u * (unsigned)(wave + SP_WAVES * q), 0, 0);
     };
-    auto commit = [&](int c, const SpStage &st, float *buf) {
-        const int s0 = cks[c].s0;
-        const int len = cks[c].len;
-        const long long base = (long long)row0 + s0;
-        const bool main_ok = (base + lane >= 0) & (base + lane < n_in);
-        const bool halo_ok = (base + hrow >= 0) & (base + hrow < n_in);
+
+    auto issue = [&](const SpInfo &info, SpStage &st) {
+        const int s0 = info.s0;
+        const int a0 = row0 + s0 - M;
+        const unsigned row_off = (unsigned)((a0 + 4 * quad) * 4);     // wraps out of range when negative
 #pragma unroll
-        for (int q = 0; q < SP_CPW; ++q) {
-            const bool ok = main_ok & (col0 + wave * SP_CPW + q < batch);
-            buf[(wave * SP_CPW + q) * SP_PITCH + lane] = ok ? st.x[q] : 0.f;
-        }
+        for (int it = 0; it < SP_LOADS; ++it)
+            st.x[it] = buffer_load_f32x4(xr, col_off[it] == OOB_OFFSET ? OOB_OFFSET : col_off[it] + row_off);
 #pragma unroll
-        for (int q = 0; q < SP_HALO; ++q) {
-            const bool ok = halo_ok & (col0 + wave * SP_CPW + q * 8 + hcol < batch);
-            buf[(wave * SP_CPW + q * 8 + hcol) * SP_PITCH + hrow] = ok ? st.x[SP_CPW + q] : 0.f;
+        for (int q = 0; q < SP_APW; ++q) {
+            const int j = wave + SP_WAVES * q;
+            const int sl = info.slot[q];
+            const int in = arow + s0 + j;                  // dense row this value multiplies
+            const int vrow = ashift ? in : arow;           // row of the value inside its diagonal
+            const bool ok = (j < info.len) & (sl >= 0) & (arow < n_out) & (in >= 0) & (in < n_in);
+            const unsigned off = ((unsigned)sl * (unsigned)stride + (unsigned)vrow) * 4u;
+            st.a[q] = buffer_load_f32(ar, ok ? off : OOB_OFFSET);
         }
+        // which of this lane's four rows exist (bit k: row a0 + 4*quad + k);
+        // all ones away from the operand's first and last rows
+        const int r = a0 + 4 * quad;
+        int bits = 0;
 #pragma unroll
-        for (int q = 0; q < SP_AVALS / 64; ++q) {
-            const int j = aj + 4 * q;
-            const long long in = arow + s0 + j;
-            const bool ok = (j < len) & (arow < n_out) & (in >= 0) & (in < n_in);
-            buf[SP_COLS * SP_PITCH + wave * SP_AVALS + q * 64 + lane] = ok ? st.a[q] : 0.f;
+        for (int k = 0; k < 4; ++k) {
+            const bool exists = (r + k >= 0) && (r + k < n_in);
+            bits |= exists ? (1 << k) : 0;
         }
+        st.rows_ok = bits;
+        st.edge = (a0 < 0) | (a0 + 4 * SP_QUADS > n_in);              // wave-uniform
     };
-    auto compute = [&](const float *buf) {
-        const float *win_lds = buf + lane * SP_PITCH + wave * SP_T;
-        const float *a_lds = buf + SP_COLS * SP_PITCH + wave * SP_AVALS + (lane & 15);
-        spmm_chunk<LCK>(acc, win_lds, a_lds);
+    auto commit = [&](const SpStage &st, float *buf) {
+        if (!st.edge) {
+#pragma unroll
+            for (int it = 0; it < SP_LOADS; ++it)
+                *reinterpret_cast<float4 *>(buf + lds_at[it]) = st.x[it];
+        } else {
+            // rows of neighbouring columns or beyond the operand: write zeros
+#pragma unroll
+            for (int it = 0; it < SP_LOADS; ++it) {
+                float4 v;
+                v.x = (st.rows_ok & 1) ? st.x[it].x : 0.f; v.y = (st.rows_ok & 2) ? st.x[it].y : 0.f;
+                v.z = (st.rows_ok & 4) ? st.x[it].z : 0.f; v.w = (st.rows_ok & 8) ? st.x[it].w : 0.f;
+                *reinterpret_cast<float4 *>(buf + lds_at[it]) = v;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < SP_APW; ++q)
+            buf[SP_XFLOATS + (wave + SP_WAVES * q) * SP_ROWS + lane] = st.a[q];
     };
-    // chunk c is computed from lds[c & 1] while chunk c+1 lands in `next` and
-    // chunk c+2 is requested into `fresh`
-    auto iteration = [&](int c, SpStage &fresh, SpStage &next) {
-        if (c + 2 < nchunks) issue(c + 2, fresh);
-        compute(lds[c & 1]);
-        if (c + 1 < nchunks) commit(c + 1, next, lds[(c + 1) & 1]);
+    auto read_window = [&](SpWindow<LCK, M> &win, const float *buf) {
+        spmm_read_window<LCK, M>(win, buf + lane * SP_PITCH + wave * SP_T,
+                                 buf + SP_XFLOATS + wave * SP_T + (lane & 15));
+    };
+    // Chunk k travels through stage set k & 1, LDS buffer k & 1, window set
+    // k & 1 and table-entry set k & 1.  Entering iteration c: window(c) is in
+    // registers, chunk c+1 has landed (or is landing) in `next`, chunk c+2 is
+    // in flight in the other stage set, `info` holds table entry c+3.
+    auto iteration = [&](int c, SpStage &next, SpWindow<LCK, M> &win_cur, SpWindow<LCK, M> &win_next,
+                         SpInfo &info, SpInfo &info_next) {
+        if (c + 1 < nchunks) commit(next, lds[(c + 1) & 1]);
+        fetch_info(c + 4, info_next);
+        if (c + 3 < nchunks) issue(info, next);
+        spmm_rows<LCK, M, 0>(acc, win_cur);
         __syncthreads();
+        if (c + 1 < nchunks) read_window(win_next, lds[(c + 1) & 1]);
     };
 
-    SpStage s0, s1;
-    issue(0, s0);
-    if (nchunks > 1) issue(1, s1);
-    commit(0, s0, lds[0]);
+    SpStage st0, st1;
+    SpWindow<LCK, M> w0, w1;
+    SpInfo i0, i1;
+    fetch_info(0, i0);
+    fetch_info(1, i1);
+    issue(i0, st0);
+    fetch_info(2, i0);
+    if (nchunks > 1) issue(i1, st1);
+    fetch_info(3, i1);
+    commit(st0, lds[0]);
+    if (nchunks > 2) issue(i0, st0);
     __syncthreads();
+    read_window(w0, lds[0]);
     for (int c = 0; c < nchunks; c += 2) {
-        iteration(c, s0, s1);
-        if (c + 1 < nchunks) iteration(c + 1, s1, s0);
+        iteration(c, st1, w0, w1, i1, i0);
+        if (c + 1 < nchunks) iteration(c + 1, st0, w1, w0, i0, i1);
     }
 
-    // epilogue: lanes-along-columns -> lanes-along-rows through LDS
+    // epilogue: lanes-along-columns -> lanes-along-rows through LDS (every
+    // wave is past the last barrier, and the last window read came from the
+    // other buffer or has completed)
+    __syncthreads();
     float *out = &lds[0][0];
 #pragma unroll
     for (int t = 0; t < SP_T; ++t) out[lane * SP_OPITCH + wave * SP_T + t] = acc[t];
@@ -493,7 +576,9 @@ __device__ __forceinline__ void dd2dia_tile(float *lds, sc_chunk_ptr ck, int row
             red[(wave * 32 + t * LC + j) * 64 + lane] = acc[t][j];
     __syncthreads();
     for (int j = wave; j < LC; j += 4) {
-        float *cd = C + (long long)ck->slot[j] * stride;
+        const int sl = ck->slot[j];
+        if (sl < 0) continue;                  // position no diagonal occupies
+        float *cd = C + (long long)sl * stride;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int ai = (t * LC + j) * 64 + lane;
@@ -551,6 +636,15 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
     return hipGetLastError();
 }
 
+bool spmm_tiled_ok(const DiaView &A, long long ldb, bool trans)
+{
+    // buffer resources address 32-bit byte offsets below the out-of-range marker
+    const long long n_in = trans ? A.h : A.w;
+    const long long x_bytes = ((SP_COLS - 1) * ldb + n_in) * 4;
+    const long long a_bytes = (long long)A.nd * A.stride * 4;
+    return A.rf == 1 && x_bytes < (long long)OOB_OFFSET && a_bytes < (long long)OOB_OFFSET;
+}
+
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, hipStream_t stream)
@@ -563,18 +657,24 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const Chunk *chunks = trans ? A.chunks_t_dev : A.chunks_n_dev;
     const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
     const int lck = trans ? A.max_len_t : A.max_len_n;
+    const int res = trans ? A.res_t : A.res_n;
+    const unsigned a_bytes = (unsigned)((long long)A.nd * A.stride * 4);
     const dim3 grid((unsigned)(row_tiles * col_tiles)), block(64 * SP_WAVES);
-#define CUVDIA_SPMM_LAUNCH(L)                                                                       \
-    case L:                                                                                         \
-        hipLaunchKernelGGL(spmm_tiled_kernel<L>, grid, block, 0, stream, chunks, nchunks, vals,     \
-                           A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha,    \
-                           beta, (int)col_tiles);                                                   \
+#define CUVDIA_SPMM_LAUNCH(L, R)                                                                    \
+    case (L) * 4 + (R):                                                                             \
+        hipLaunchKernelGGL((spmm_tiled_kernel<L, R>), grid, block, 0, stream, chunks, nchunks,      \
+                           vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch,     \
+                           alpha, beta, (int)col_tiles, a_bytes);                                   \
         break;
-    switch (lck) {
-        CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
-        CUVDIA_SPMM_LAUNCH(5) CUVDIA_SPMM_LAUNCH(6) CUVDIA_SPMM_LAUNCH(7) CUVDIA_SPMM_LAUNCH(8)
+#define CUVDIA_SPMM_LAUNCH4(L) \
+    CUVDIA_SPMM_LAUNCH(L, 0) CUVDIA_SPMM_LAUNCH(L, 1) CUVDIA_SPMM_LAUNCH(L, 2) CUVDIA_SPMM_LAUNCH(L, 3)
+    if (lck < 1 || lck > CHUNK_MAX || res < 0 || res > 3) return hipErrorInvalidValue;
+    switch (lck * 4 + res) {
+        CUVDIA_SPMM_LAUNCH4(1) CUVDIA_SPMM_LAUNCH4(2) CUVDIA_SPMM_LAUNCH4(3) CUVDIA_SPMM_LAUNCH4(4)
+        CUVDIA_SPMM_LAUNCH4(5) CUVDIA_SPMM_LAUNCH4(6) CUVDIA_SPMM_LAUNCH4(7) CUVDIA_SPMM_LAUNCH4(8)
         default: return hipErrorInvalidValue;
     }
+#undef CUVDIA_SPMM_LAUNCH4
 #undef CUVDIA_SPMM_LAUNCH
     return hipGetLastError();
 }

@@ -16,6 +16,7 @@ struct DiaView {
     const Chunk *chunks_t_dev;   // shifts = -offsets
     int n_chunks_t;
     int max_len_n, max_len_t;    // longest chunk of each table
+    int res_n, res_t;            // s0 mod 4, common to every chunk of the table
 };
 
 // dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch
@@ -31,6 +32,10 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, hipStream_t stream);
+
+// Whether the tiled SpMM can serve these operands (row_fact 1, operand extents
+// within its 32-bit buffer addressing).
+bool spmm_tiled_ok(const DiaView &A, long long ldb, bool trans);
 
 // C_d[i] = beta*C_d[i] + alpha*sum_c A[i,c]*B[k_d + i/rf, c] on valid slots.
 // One thread per slot, serial over the batch; honours row_fact.
