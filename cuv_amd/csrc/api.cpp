@@ -105,7 +105,6 @@ int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
     std::vector<Chunk> ch;
     try {
         ch = plan_chunks(offsets_host, nd, transposed != 0);
-        if (common_residue(ch) < 0) ch = plan_chunks(offsets_host, nd, transposed != 0, true);
     } catch (const std::bad_alloc &) {
         return CUVDIA_ENOMEM;
     }
@@ -141,13 +140,8 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     try {
         d = new cuvdia_desc();
         d->offsets.assign(offsets_host, offsets_host + nd);
-        // chunks of one table must start at the same residue mod 4 (it is a
-        // template parameter of the tiled SpMM); re-plan on aligned starts
-        // when the natural runs disagree
         cn = plan_chunks(offsets_host, nd, false);
-        if (common_residue(cn) < 0) cn = plan_chunks(offsets_host, nd, false, true);
         ct = plan_chunks(offsets_host, nd, true);
-        if (common_residue(ct) < 0) ct = plan_chunks(offsets_host, nd, true, true);
     } catch (const std::bad_alloc &) {
         delete d;
         return CUVDIA_ENOMEM;
@@ -180,7 +174,7 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
                       reinterpret_cast<const int *>(base),
                       reinterpret_cast<const Chunk *>(base + off_bytes), d->n_chunks_n,
                       reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t,
-                      0, 0, common_residue(cn), common_residue(ct)};
+                      0, 0};
     for (const Chunk &c : cn) d->view.max_len_n = std::max(d->view.max_len_n, c.len);
     for (const Chunk &c : ct) d->view.max_len_t = std::max(d->view.max_len_t, c.len);
     *out = d;

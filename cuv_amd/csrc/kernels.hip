@@ -142,26 +142,27 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 //
 // Workgroup = 64 output rows x 64 batch columns, 4 waves of 16 rows each.
 // Lane l of every wave owns batch column col0 + l and 16 running sums.  Per
-// run chunk (<= 8 consecutive shifts starting at s0, s0 = M mod 4 for every
-// chunk of the table):
-//   1. the dense rows [a0, a0 + 80), a0 = row0 + s0 - M (a multiple of 4), of
-//      the 64 columns are fetched with 16-byte buffer loads, 20 lanes per
-//      column and 3 columns per instruction, so every cache line of a column
-//      is requested by one instruction only, and written to LDS with 16-byte
-//      stores, columns 84 floats apart.  Each wave also fetches two of the
+// run chunk (<= 8 consecutive shifts starting at s0):
+//   1. the dense rows [a0, a0 + 80), a0 = row0 + s0, of the 64 columns are
+//      fetched with 16-byte buffer loads (4-byte aligned is all they need),
+//      20 lanes per column and 3 columns per instruction, so every cache line
+//      of a column is requested by one instruction only, and written to LDS
+//      with 16-byte stores, columns 84 floats apart: LDS row i of a column
+//      holds dense row a0 + i.  Each wave also fetches two of the
 //      chunk's eight diagonals for all 64 rows (one 256-byte row segment per
 //      instruction) and parks them in LDS.  Rows outside the operand and
-//      diagonal slots outside the matrix become zeros (out-of-range buffer
-//      offsets, plus a masked write on boundary tiles), so the arithmetic
-//      below needs no guards and never sees padding;
-//   2. each lane reads its column's window of 16 + LCK - 1 + M values with
+//      diagonal slots outside the matrix become zeros: they are given an
+//      out-of-range buffer offset (tiles touching the operand's first or last
+//      rows load row by row for that), so the arithmetic below needs no
+//      guards and never sees padding;
+//   2. each lane reads its column's window of 16 + LCK - 1 values with
 //      16-byte LDS reads (pitch/4 is odd, so the 64 lanes spread over all
 //      banks).  Every chunk is processed as LCK diagonals, LCK = the longest
 //      chunk of the table; shorter chunks carry zeros;
 //   3. for each diagonal j the wave reads A_j[16 rows] into one VGPR (lane & 15
 //      selects the row) and issues 16 FMAs whose first operand is that VGPR
 //      broadcast within each 16-lane row by DPP (row_newbcast:t):
-//          acc[t] = fma(A_j[row t], win[t + j + M], acc[t]).
+//          acc[t] = fma(A_j[row t], win[t + j], acc[t]).
 // The loop is software-pipelined three chunks deep: while the FMAs of chunk c
 // run out of registers, chunk c+1 is being written to the other LDS buffer
 // (its window is read right after the barrier), chunk c+2 is in flight from
@@ -189,8 +190,6 @@ constexpr int SP_APW = CHUNK_MAX / SP_WAVES;    // diagonals each wave fetches p
 struct SpStage {
     float4 x[SP_LOADS];
     float a[SP_APW];
-    int rows_ok;            // bit k: dense row of x[].k exists
-    bool edge;              // some staged row does not exist (wave-uniform)
 };
 
 // One chunk-table entry as a wave needs it: shift, length, and the table
@@ -200,9 +199,9 @@ struct SpInfo {
     int slot[SP_APW];
 };
 
-template <int LCK, int M>
+template <int LCK>
 struct SpWindow {
-    static constexpr int WQ = (SP_T + LCK - 1 + M + 3) / 4;
+    static constexpr int WQ = (SP_T + LCK - 1 + 3) / 4;
     float w[WQ * 4];
     float a[LCK];
 };
@@ -243,22 +242,22 @@ __device__ __forceinline__ void fma_row16(float (&acc)[SP_T], float a, const flo
           "v"(win[J + 12]), "v"(win[J + 13]), "v"(win[J + 14]), "v"(win[J + 15]));
 }
 
-template <int LCK, int M, int J>
-__device__ __forceinline__ void spmm_rows(float (&acc)[SP_T], const SpWindow<LCK, M> &win)
+template <int LCK, int J>
+__device__ __forceinline__ void spmm_rows(float (&acc)[SP_T], const SpWindow<LCK> &win)
 {
     if constexpr (J < LCK) {
-        fma_row16<J + M>(acc, win.a[J], win.w);
-        spmm_rows<LCK, M, J + 1>(acc, win);
+        fma_row16<J>(acc, win.a[J], win.w);
+        spmm_rows<LCK, J + 1>(acc, win);
     }
 }
 
-template <int LCK, int M>
-__device__ __forceinline__ void spmm_read_window(SpWindow<LCK, M> &win, const float *win_lds,
+template <int LCK>
+__device__ __forceinline__ void spmm_read_window(SpWindow<LCK> &win, const float *win_lds,
                                                  const float *a_lds)
 {
     const float4 *p4 = reinterpret_cast<const float4 *>(win_lds);
 #pragma unroll
-    for (int q = 0; q < SpWindow<LCK, M>::WQ; ++q) {
+    for (int q = 0; q < SpWindow<LCK>::WQ; ++q) {
         const float4 v = p4[q];
         win.w[4 * q + 0] = v.x; win.w[4 * q + 1] = v.y; win.w[4 * q + 2] = v.z; win.w[4 * q + 3] = v.w;
     }
@@ -285,7 +284,7 @@ __device__ __forceinline__ float4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, un
 }
 constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used here
 
-template <int LCK, int M>
+template <int LCK>
 __global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
@@ -344,11 +343,27 @@ __global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
 
     auto issue = [&](const SpInfo &info, SpStage &st) {
         const int s0 = info.s0;
-        const int a0 = row0 + s0 - M;
-        const unsigned row_off = (unsigned)((a0 + 4 * quad) * 4);     // wraps out of range when negative
+        const int a0 = row0 + s0;
+        const int r = a0 + 4 * quad;                       // first dense row of this lane's piece
+        if ((a0 >= 0) & (a0 + 4 * SP_QUADS <= n_in)) {     // wave-uniform: every staged row exists
+            const unsigned row_off = (unsigned)r * 4u;
 #pragma unroll
-        for (int it = 0; it < SP_LOADS; ++it)
-            st.x[it] = buffer_load_f32x4(xr, col_off[it] == OOB_OFFSET ? OOB_OFFSET : col_off[it] + row_off);
+            for (int it = 0; it < SP_LOADS; ++it)
+                st.x[it] = buffer_load_f32x4(xr, col_off[it] == OOB_OFFSET ? OOB_OFFSET : col_off[it] + row_off);
+        } else {
+            // first or last rows of the operand: row by row, a missing row gets
+            // the out-of-range offset and reads as 0
+#pragma unroll
+            for (int it = 0; it < SP_LOADS; ++it) {
+                float v[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const bool ok = (r + k >= 0) & (r + k < n_in) & (col_off[it] != OOB_OFFSET);
+                    v[k] = buffer_load_f32(xr, ok ? col_off[it] + (unsigned)(r + k) * 4u : OOB_OFFSET);
+                }
+                st.x[it] = make_float4(v[0], v[1], v[2], v[3]);
+            }
+        }
 #pragma unroll
         for (int q = 0; q < SP_APW; ++q) {
             const int j = wave + SP_WAVES * q;
@@ -359,57 +374,35 @@ __global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
             const unsigned off = ((unsigned)sl * (unsigned)stride + (unsigned)vrow) * 4u;
             st.a[q] = buffer_load_f32(ar, ok ? off : OOB_OFFSET);
         }
-        // which of this lane's four rows exist (bit k: row a0 + 4*quad + k);
-        // all ones away from the operand's first and last rows
-        const int r = a0 + 4 * quad;
-        int bits = 0;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const bool exists = (r + k >= 0) && (r + k < n_in);
-            bits |= exists ? (1 << k) : 0;
-        }
-        st.rows_ok = bits;
-        st.edge = (a0 < 0) | (a0 + 4 * SP_QUADS > n_in);              // wave-uniform
     };
     auto commit = [&](const SpStage &st, float *buf) {
-        if (!st.edge) {
 #pragma unroll
-            for (int it = 0; it < SP_LOADS; ++it)
-                *reinterpret_cast<float4 *>(buf + lds_at[it]) = st.x[it];
-        } else {
-            // rows of neighbouring columns or beyond the operand: write zeros
-#pragma unroll
-            for (int it = 0; it < SP_LOADS; ++it) {
-                float4 v;
-                v.x = (st.rows_ok & 1) ? st.x[it].x : 0.f; v.y = (st.rows_ok & 2) ? st.x[it].y : 0.f;
-                v.z = (st.rows_ok & 4) ? st.x[it].z : 0.f; v.w = (st.rows_ok & 8) ? st.x[it].w : 0.f;
-                *reinterpret_cast<float4 *>(buf + lds_at[it]) = v;
-            }
-        }
+        for (int it = 0; it < SP_LOADS; ++it)
+            *reinterpret_cast<float4 *>(buf + lds_at[it]) = st.x[it];
 #pragma unroll
         for (int q = 0; q < SP_APW; ++q)
             buf[SP_XFLOATS + (wave + SP_WAVES * q) * SP_ROWS + lane] = st.a[q];
     };
-    auto read_window = [&](SpWindow<LCK, M> &win, const float *buf) {
-        spmm_read_window<LCK, M>(win, buf + lane * SP_PITCH + wave * SP_T,
+    auto read_window = [&](SpWindow<LCK> &win, const float *buf) {
+        spmm_read_window<LCK>(win, buf + lane * SP_PITCH + wave * SP_T,
                                  buf + SP_XFLOATS + wave * SP_T + (lane & 15));
     };
     // Chunk k travels through stage set k & 1, LDS buffer k & 1, window set
     // k & 1 and table-entry set k & 1.  Entering iteration c: window(c) is in
     // registers, chunk c+1 has landed (or is landing) in `next`, chunk c+2 is
     // in flight in the other stage set, `info` holds table entry c+3.
-    auto iteration = [&](int c, SpStage &next, SpWindow<LCK, M> &win_cur, SpWindow<LCK, M> &win_next,
+    auto iteration = [&](int c, SpStage &next, SpWindow<LCK> &win_cur, SpWindow<LCK> &win_next,
                          SpInfo &info, SpInfo &info_next) {
         if (c + 1 < nchunks) commit(next, lds[(c + 1) & 1]);
         fetch_info(c + 4, info_next);
         if (c + 3 < nchunks) issue(info, next);
-        spmm_rows<LCK, M, 0>(acc, win_cur);
+        spmm_rows<LCK, 0>(acc, win_cur);
         __syncthreads();
         if (c + 1 < nchunks) read_window(win_next, lds[(c + 1) & 1]);
     };
 
     SpStage st0, st1;
-    SpWindow<LCK, M> w0, w1;
+    SpWindow<LCK> w0, w1;
     SpInfo i0, i1;
     fetch_info(0, i0);
     fetch_info(1, i1);
@@ -657,24 +650,19 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const Chunk *chunks = trans ? A.chunks_t_dev : A.chunks_n_dev;
     const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
     const int lck = trans ? A.max_len_t : A.max_len_n;
-    const int res = trans ? A.res_t : A.res_n;
     const unsigned a_bytes = (unsigned)((long long)A.nd * A.stride * 4);
     const dim3 grid((unsigned)(row_tiles * col_tiles)), block(64 * SP_WAVES);
-#define CUVDIA_SPMM_LAUNCH(L, R)                                                                    \
-    case (L) * 4 + (R):                                                                             \
-        hipLaunchKernelGGL((spmm_tiled_kernel<L, R>), grid, block, 0, stream, chunks, nchunks,      \
-                           vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch,     \
-                           alpha, beta, (int)col_tiles, a_bytes);                                   \
+#define CUVDIA_SPMM_LAUNCH(L)                                                                       \
+    case L:                                                                                         \
+        hipLaunchKernelGGL(spmm_tiled_kernel<L>, grid, block, 0, stream, chunks, nchunks, vals,     \
+                           A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha,    \
+                           beta, (int)col_tiles, a_bytes);                                          \
         break;
-#define CUVDIA_SPMM_LAUNCH4(L) \
-    CUVDIA_SPMM_LAUNCH(L, 0) CUVDIA_SPMM_LAUNCH(L, 1) CUVDIA_SPMM_LAUNCH(L, 2) CUVDIA_SPMM_LAUNCH(L, 3)
-    if (lck < 1 || lck > CHUNK_MAX || res < 0 || res > 3) return hipErrorInvalidValue;
-    switch (lck * 4 + res) {
-        CUVDIA_SPMM_LAUNCH4(1) CUVDIA_SPMM_LAUNCH4(2) CUVDIA_SPMM_LAUNCH4(3) CUVDIA_SPMM_LAUNCH4(4)
-        CUVDIA_SPMM_LAUNCH4(5) CUVDIA_SPMM_LAUNCH4(6) CUVDIA_SPMM_LAUNCH4(7) CUVDIA_SPMM_LAUNCH4(8)
+    switch (lck) {
+        CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
+        CUVDIA_SPMM_LAUNCH(5) CUVDIA_SPMM_LAUNCH(6) CUVDIA_SPMM_LAUNCH(7) CUVDIA_SPMM_LAUNCH(8)
         default: return hipErrorInvalidValue;
     }
-#undef CUVDIA_SPMM_LAUNCH4
 #undef CUVDIA_SPMM_LAUNCH
     return hipGetLastError();
 }

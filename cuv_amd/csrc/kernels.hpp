@@ -16,7 +16,6 @@ struct DiaView {
     const Chunk *chunks_t_dev;   // shifts = -offsets
     int n_chunks_t;
     int max_len_n, max_len_t;    // longest chunk of each table
-    int res_n, res_t;            // s0 mod 4, common to every chunk of the table
 };
 
 // dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch

@@ -6,7 +6,7 @@
 
 namespace cuvdia {
 
-std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, bool align4)
+std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed)
 {
     std::vector<std::pair<long long, int>> s(nd);      // (shift, table position)
     for (int d = 0; d < nd; ++d)
@@ -20,41 +20,21 @@ std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, bool
     while (i < nd) {
         int j = i + 1;
         while (j < nd && s[j].first == s[j - 1].first + 1) ++j;
-        // positions = diagonals of the run, preceded by `lead` empty ones when
-        // chunk starts must be multiples of 4
-        const long long first = s[i].first;
-        const int lead = align4 ? (int)(((first % 4) + 4) % 4) : 0;
-        const int run = (j - i) + lead;
+        const int run = j - i;
         const int pieces = (run + CHUNK_MAX - 1) / CHUNK_MAX;
         int done = 0;
         for (int p = 0; p < pieces; ++p) {
-            // aligned plans cut at multiples of 4 positions; free plans balance the pieces
-            int len = align4 ? std::min(CHUNK_MAX, run - done)
-                             : (run - done + (pieces - p) - 1) / (pieces - p);
+            const int len = (run - done + (pieces - p) - 1) / (pieces - p);
             Chunk c{};
-            c.s0 = (int)(first - lead + done);
+            c.s0 = (int)s[i + done].first;
             c.len = len;
-            for (int q = 0; q < CHUNK_MAX; ++q) {
-                const int pos = done + q - lead;            // index into the run's diagonals
-                c.slot[q] = (q < len && pos >= 0) ? s[i + pos].second : -1;
-            }
+            for (int q = 0; q < CHUNK_MAX; ++q) c.slot[q] = q < len ? s[i + done + q].second : -1;
             out.push_back(c);
             done += len;
         }
         i = j;
     }
     return out;
-}
-
-int common_residue(const std::vector<Chunk> &chunks)
-{
-    int res = -1;
-    for (const Chunk &c : chunks) {
-        const int r = ((c.s0 % 4) + 4) % 4;
-        if (res >= 0 && r != res) return -1;
-        res = r;
-    }
-    return res;
 }
 
 long long count_valid(const int *offsets, int nd, int h, int w, int rf)

@@ -24,13 +24,9 @@ static_assert(sizeof(Chunk) == 48, "Chunk layout is part of the device table");
 
 // Sort shifts (stable in table position), cut into maximal runs of
 // consecutive shifts -- a repeated shift starts a new run -- and split each
-// run into near-equal chunks of at most CHUNK_MAX.  With align4 every chunk
-// starts at a multiple of 4: a run that starts elsewhere gets up to three
-// leading empty positions (slot -1).
-std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, bool align4 = false);
-
-// s0 mod 4 (in 0..3) if every chunk agrees, otherwise -1.
-int common_residue(const std::vector<Chunk> &chunks);
+// run into near-equal chunks of at most CHUNK_MAX.  Positions past a chunk's
+// length carry slot -1.
+std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed);
 
 // Number of matrix elements stored (slots the reference host loops touch):
 // sum over diagonals of min(h - rf*max(0,-k), rf*(w - max(0,k))), clamped at 0

@@ -75,12 +75,9 @@ int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t,
  * (transposed == 0) or their negation (transposed != 0), sorted ascending;
  * a run is a maximal sequence of consecutive shifts and is cut into chunks
  * of at most 8.  Chunk c covers shifts s0[c] .. s0[c]+len[c]-1 and
- * slot[8*c + j] is the table position of the j-th one, or -1 for a position
- * no diagonal occupies.  All chunks of a plan start at the same residue
- * mod 4: when the natural runs disagree, runs are padded with leading empty
- * positions so that every chunk starts at a multiple of 4.  Returns the
- * number of chunks (also when it exceeds cap; then nothing is written), or
- * a negative error. */
+ * slot[8*c + j] is the table position of the j-th one (-1 for j >= len[c]).
+ * Returns the number of chunks (also when it exceeds cap; then nothing is
+ * written), or a negative error. */
 int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
                        int *s0, int *len, int *slot, int cap);
 

@@ -1,0 +1,214 @@
+// The reference's device-side DIA tests, re-expressed against the C++ mirror.
+// Needs a GPU: every case runs the device path (the HIP kernels behind the
+// C ABI) and compares with the host twin or a dense product.
+//
+//   src/tests/spmv.cpp:103-129            spmv_dev_correctness{,_trans}
+//   src/tests/densedense_to_dia.cpp:109-197  dd2s_correctness_dev, dd2s_cmp_dev_host (row_fact 4)
+//   src/tests/dia_mat.cpp:103-132         spmv_uninit, spmv_host2dev
+#include <cuv.hpp>
+#include <cuv_host_ops.hpp>
+
+#include "check.hpp"
+
+using namespace cuv;
+
+static const int n = 32, m = 16, k = 6;
+
+struct Fix {
+    dia_matrix<float, host_memory_space> A;
+    tensor<float, host_memory_space, column_major> B, C;
+    Fix() : A(n, m, 7, 32, 1), B(m, k), C(n, k)
+    {
+        std::vector<int> off;
+        for (int i = -3; i <= 3; i++) off.push_back(i);
+        A.set_offsets(off);
+        sequence(A.vec()); sequence(C); sequence(B);
+    }
+};
+
+TEST_CASE(spmv_dev_correctness_trans)
+{
+    Fix f;
+    dia_matrix<float, dev_memory_space> A2(n, m, f.A.num_dia(), f.A.stride(), 1);
+    convert(A2, f.A);
+    tensor<float, dev_memory_space, column_major> C2(f.C.shape());
+    convert(C2, f.C);
+    tensor<float, dev_memory_space, column_major> B2(f.B.shape());
+    convert(B2, f.B);
+    prod(f.B, f.A, f.C, 't', 'n');
+    prod(B2, A2, C2, 't', 'n');
+    MAT_CMP(f.B, B2, 0.1f);
+}
+
+TEST_CASE(spmv_dev_correctness)
+{
+    Fix f;
+    dia_matrix<float, dev_memory_space> A2(n, m, f.A.num_dia(), f.A.stride(), 1);
+    convert(A2, f.A);
+    tensor<float, dev_memory_space, column_major> C2(f.C.shape());
+    convert(C2, f.C);
+    tensor<float, dev_memory_space, column_major> B2(f.B.shape());
+    convert(B2, f.B);
+    const float factAv = 2.f, factC = 1.3f;
+    prod(f.C, f.A, f.B, 'n', 'n', factAv, factC);
+    prod(C2, A2, B2, 'n', 'n', factAv, factC);
+    MAT_CMP(f.C, C2, 0.1f);
+}
+
+TEST_CASE(spmv_dev_flat_vectors)
+{
+    // cuv::spmv on flat tensors holding several columns (spmv.cu:243-245)
+    Fix f;
+    dia_matrix<float, dev_memory_space> A2(n, m, f.A.num_dia(), f.A.stride(), 1);
+    convert(A2, f.A);
+    tensor<float, dev_memory_space> x(m * k), y(n * k);
+    tensor<float, host_memory_space> xh(m * k), yh(n * k), yd(n * k);
+    sequence(xh); fill(yh, 0);
+    convert(x, xh);
+    spmv(y, A2, x, 'n', 1.f, 0.f);
+    convert(yd, y);
+    for (int c = 0; c < k; c++) {
+        tensor<float, host_memory_space> xv(indices[index_range(0, m)], xh.ptr() + c * m);
+        tensor<float, host_memory_space> yv(indices[index_range(0, n)], yh.ptr() + c * n);
+        spmv(yv, f.A, xv, 'n', 1.f, 0.f);
+    }
+    for (int i = 0; i < n * k; i++) CHECK((float)yd[i] == (float)yh[i]);
+}
+
+struct DdFix {
+    static const int n = 36, m = 19, k = 16, rf = 4;
+    dia_matrix<float, dev_memory_space> C;
+    tensor<float, dev_memory_space, column_major> C_, A, B;
+    DdFix() : C(n, m, 7, 36, rf), C_(n, m), A(n, k), B(m, k)
+    {
+        std::vector<int> off;
+        for (int i = -3; i <= 3; i++) off.push_back(i);
+        C.set_offsets(off);
+        sequence(A); sequence(B);
+        fill(C.vec(), 0);
+    }
+};
+
+TEST_CASE(dd2s_correctness_dev)
+{
+    DdFix f;
+    dev_block_descriptor<float> bd(f.C);
+    densedense_to_dia(f.C, bd, f.A, f.B);
+    tensor<float, host_memory_space, column_major> Ah(f.A.shape()), Bh(f.B.shape()), dense(DdFix::n, DdFix::m);
+    convert(Ah, f.A); convert(Bh, f.B);
+    fill(dense, 0);
+    prod(dense, Ah, Bh, 'n', 't');
+    int seen = 0;
+    for (int i = 0; i < DdFix::n; i++)
+        for (int j = 0; j < DdFix::m; j++)
+            if (f.C(i, j) != 0) {
+                CHECK(close_pct(f.C(i, j), (float)dense(i, j), 0.01f));
+                ++seen;
+            }
+    CHECK(seen > 200);
+}
+
+TEST_CASE(dd2s_cmp_dev_host)
+{
+    DdFix f;
+    dia_matrix<float, host_memory_space> C2(DdFix::n, DdFix::m, f.C.num_dia(), f.C.stride(), DdFix::rf);
+    tensor<float, host_memory_space, column_major> A2(f.A.shape()), B2(f.B.shape());
+    convert(C2, f.C); convert(A2, f.A); convert(B2, f.B);
+    dev_block_descriptor<float> bd(f.C);
+    host_block_descriptor<float> bdh(C2);
+    densedense_to_dia(f.C, bd, f.A, f.B);
+    densedense_to_dia(C2, bdh, A2, B2);
+    MAT_CMP(f.C, C2, 0.01f);
+    // documented factors, and the descriptor-free overload
+    densedense_to_dia(f.C, f.A, f.B, 0.5f, 0.25f);
+    densedense_to_dia(C2, bdh, A2, B2, 0.5f, 0.25f);
+    MAT_CMP(f.C, C2, 0.01f);
+}
+
+TEST_CASE(spmv_uninit)
+{
+    dia_matrix<float, host_memory_space> w(32, 16, 3, 32, 1);
+    std::vector<int> off;
+    off.push_back(0); off.push_back(1); off.push_back(-1);
+    w.set_offsets(off);
+    sequence(w.vec());
+    dia_matrix<float, dev_memory_space> wdev(32, 16, 3, 16, 1);
+    wdev.dealloc();
+    convert(wdev, w);
+    CHECK(wdev.vec_ptr() != NULL && wdev.stride() == 32);
+    MAT_CMP(w, wdev, 0.1f);
+}
+
+TEST_CASE(spmv_host2dev)
+{
+    dia_matrix<float, host_memory_space> w(32, 16, 3, 32, 1);
+    std::vector<int> off;
+    off.push_back(0); off.push_back(1); off.push_back(-1);
+    w.set_offsets(off);
+    sequence(w.vec());
+    dia_matrix<float, dev_memory_space> w2(32, 16, w.num_dia(), w.stride(), 1);
+    convert(w2, w);
+    MAT_CMP(w, w2, 0.1f);
+    fill(w.vec(), 0);
+    convert(w, w2);
+    MAT_CMP(w, w2, 0.1f);
+    CHECK(w(5, 6) == 32.f + 5);
+}
+
+TEST_CASE(dev_preconditions_throw)
+{
+    Fix f;
+    dia_matrix<float, dev_memory_space> A2(n, m, f.A.num_dia(), f.A.stride(), 1);
+    convert(A2, f.A);
+    tensor<float, dev_memory_space, column_major> B2(f.B.shape()), C2(f.C.shape()), narrow(n, 2);
+    CHECK_THROWS(prod(C2, A2, B2, 'n', 't'));       // transB == 'n'
+    CHECK_THROWS(prod(C2, A2, B2, 'x', 'n'));       // transA is 'n' or 't'
+    CHECK_THROWS(prod(C2, A2, C2, 'n', 'n'));       // rows of B
+    CHECK_THROWS(prod(B2, A2, B2, 't', 'n'));       // transposed product needs h rows in B
+    CHECK_THROWS(prod(narrow, A2, B2));             // batch mismatch
+    DdFix d;
+    tensor<float, dev_memory_space, column_major> wrongA(DdFix::n + 1, DdFix::k);
+    dev_block_descriptor<float> bd(d.C);
+    CHECK_THROWS(densedense_to_dia(d.C, bd, wrongA, d.B));
+    // a descriptor built for another pattern is rejected
+    dia_matrix<float, dev_memory_space> other(DdFix::n, DdFix::m, 7, 36, DdFix::rf);
+    std::vector<int> off;
+    for (int i = -2; i <= 4; i++) off.push_back(i);
+    other.set_offsets(off);
+    dev_block_descriptor<float> bd2(other);
+    CHECK_THROWS(densedense_to_dia(d.C, bd2, d.A, d.B));
+}
+
+TEST_CASE(locally_connected_layer)
+{
+    // a filter_factory pattern driven through all three operations, device vs host
+    filter_factory<float, host_memory_space> ff(16, 16, 5, 1, 1);
+    dia_matrix<float, host_memory_space> *W = ff.get_dia();
+    const int N = W->h(), batch = 40;
+    for (int i = 0; i < (int)W->vec().size(); i++) W->vec()[i] = 0.01f * (float)((i * 37) % 101 + 1);   // positive: no cancellation under the percent tolerance
+    tensor<float, host_memory_space, column_major> V(N, batch), H(N, batch), Hh(N, batch), Vh(N, batch);
+    for (int i = 0; i < N * batch; i++) { V[i] = (float)((i * 13) % 7) / 7.f; H[i] = (float)((i * 29) % 11) / 11.f; }
+    dia_matrix<float, dev_memory_space> Wd(N, N, W->num_dia(), W->stride(), 1);
+    convert(Wd, *W);
+    tensor<float, dev_memory_space, column_major> Vd(V.shape()), Hd(H.shape()), outd(N, batch);
+    convert(Vd, V); convert(Hd, H);
+    prod(outd, Wd, Vd, 'n', 'n');
+    prod(Hh, *W, V, 'n', 'n');
+    MAT_CMP(Hh, outd, 0.01f);
+    prod(outd, Wd, Hd, 't', 'n');
+    prod(Vh, *W, H, 't', 'n');
+    MAT_CMP(Vh, outd, 0.01f);
+    densedense_to_dia(Wd, Hd, Vd, 1.f / batch, 0.9f);
+    host_block_descriptor<float> bdh(*W);
+    densedense_to_dia(*W, bdh, H, V, 1.f / batch, 0.9f);
+    MAT_CMP(*W, Wd, 0.01f);
+    delete W;
+}
+
+int main(int argc, char **argv)
+{
+    initCUDA(CUDA_TEST_DEVICE);
+    const int rc = run_all(argc, argv);
+    exitCUDA();
+    return rc;
+}

@@ -1,0 +1,123 @@
+"""CPU-side checks of the shared library: it loads without a GPU, exports every
+entry point include/cuvdia.h declares, fails loudly (not silently) when asked
+to compute without a device, and its host-only chunk planner decomposes offset
+tables correctly."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "cuvdia.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cuvdia_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = _declared()
+    for must in ("cuvdia_spmm_f32", "cuvdia_dd2dia_f32", "cuvdia_desc_create", "cuvdia_desc_destroy",
+                 "cuvdia_strerror", "cuvdia_plan_chunks", "cuvdia_spmm_offsets_f32", "cuvdia_dd2dia_offsets_f32"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from cuv_amd import _lib
+    L = _lib.lib()
+    for name in _declared():
+        assert hasattr(L, name), "libcuvdia.so does not export %s" % name
+    assert L.cuvdia_abi_version() == 1
+    assert L.cuvdia_strerror(-2).decode() == "operand shapes do not match the matrix"
+    assert L.cuvdia_strerror(0).decode() == "ok"
+
+
+def test_no_device_is_an_error_not_a_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from cuv_amd import _lib
+    L = _lib.lib()
+    d = ctypes.c_void_p()
+    offs = np.array([0, 1], np.int32)
+    rc = L.cuvdia_desc_create(ctypes.byref(d), offs.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), 2, 8, 8, 8, 1)
+    assert rc == _lib.ENODEVICE and not d.value
+    # argument validation still happens first
+    rc = L.cuvdia_desc_create(ctypes.byref(d), offs.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), 2, 8, 8, 4, 1)
+    assert rc == _lib.EINVAL
+    assert L.cuvdia_spmm_f32(None, None, None, 0, None, 0, 1, b"n", 1.0, 0.0, None) == _lib.EINVAL
+    assert L.cuvdia_set_path(7) == _lib.EINVAL and L.cuvdia_set_path(0) == 0
+
+
+def _plan(offsets, transposed=False):
+    from cuv_amd import _lib
+    L = _lib.lib()
+    offs = np.ascontiguousarray(offsets, np.int32)
+    ip = ctypes.POINTER(ctypes.c_int)
+    n = L.cuvdia_plan_chunks(offs.ctypes.data_as(ip), offs.size, int(transposed), None, None, None, 0)
+    assert n > 0
+    s0, ln, sl = np.zeros(n, np.int32), np.zeros(n, np.int32), np.zeros(8 * n, np.int32)
+    assert L.cuvdia_plan_chunks(offs.ctypes.data_as(ip), offs.size, int(transposed), s0.ctypes.data_as(ip),
+                                ln.ctypes.data_as(ip), sl.ctypes.data_as(ip), n) == n
+    return s0, ln, sl.reshape(n, 8)
+
+
+def _check_plan_covers(offsets, transposed):
+    s0, ln, sl = _plan(offsets, transposed)
+    sign = -1 if transposed else 1
+    seen = []
+    for c in range(len(s0)):
+        assert 1 <= ln[c] <= 8
+        for j in range(8):
+            if j < ln[c] and sl[c, j] >= 0:
+                assert sign * offsets[sl[c, j]] == s0[c] + j       # the slot really has that shift
+                seen.append(int(sl[c, j]))
+            else:
+                assert sl[c, j] == -1
+    assert sorted(seen) == list(range(len(offsets)))             # every diagonal exactly once
+    assert all(s0[i] <= s0[i + 1] for i in range(len(s0) - 1))
+    return s0, ln, sl
+
+
+def test_plan_window_pattern():
+    offs = [dy * 128 + dx for dy in range(-3, 4) for dx in range(-3, 4)]
+    s0, ln, sl = _check_plan_covers(offs, False)
+    assert s0.tolist() == [dy * 128 - 3 for dy in range(-3, 4)] and ln.tolist() == [7] * 7
+    assert sl[0, :7].tolist() == list(range(7))
+    s0t, lnt, slt = _check_plan_covers(offs, True)
+    assert s0t.tolist() == [dy * 128 - 3 for dy in range(-3, 4)]
+    assert slt[0, :7].tolist() == [48, 47, 46, 45, 44, 43, 42]     # shifts are negated offsets
+
+
+def test_plan_long_runs_are_split_evenly():
+    s0, ln, _ = _check_plan_covers(list(range(-16, 17)), False)     # one run of 33
+    assert ln.tolist() == [7, 7, 7, 6, 6] and s0[0] == -16
+    offs = [c * 65536 + dy * 256 + dx for c in range(4) for dy in range(-6, 7) for dx in range(-6, 7)]
+    s0, ln, _ = _check_plan_covers(offs, False)                     # 52 runs of 13 -> 7 + 6
+    assert len(s0) == 104 and sorted(set(ln.tolist())) == [6, 7]
+
+
+def test_plan_isolated_and_adjacent_runs():
+    offs = [0, 1, -1, 10, 11, 12, 13, 14, 15, 16, 17, 18, 40]
+    s0, ln, sl = _check_plan_covers(offs, False)
+    assert s0.tolist() == [-1, 10, 15, 40] and ln.tolist() == [3, 5, 4, 1]
+    assert sl[0, :3].tolist() == [2, 0, 1]
+    _check_plan_covers(offs, True)
+
+
+def test_plan_unsorted_duplicates_and_extremes():
+    _check_plan_covers([5, -7, 0, 39, -39], False)
+    s0, ln, sl = _check_plan_covers([0, 0, 3, 2000, -2000, 3], False)   # a repeated offset opens a new run
+    assert len(s0) >= 5
+    _check_plan_covers([7], True)
+
+
+def test_plan_rejects_bad_arguments():
+    from cuv_amd import _lib
+    L = _lib.lib()
+    assert L.cuvdia_plan_chunks(None, 3, 0, None, None, None, 0) == _lib.EINVAL
+    offs = np.array([1], np.int32)
+    assert L.cuvdia_plan_chunks(offs.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), 0, 0, None, None, None, 0) == _lib.EINVAL
