@@ -24,6 +24,7 @@
 #include "kernels.hpp"
 
 namespace cuvdia {
+int g_spmm_rows_per_wave = 8;
 namespace {
 
 // Loads through this address space are issued on the scalar unit when the
@@ -151,10 +152,10 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 //      holds dense row a0 + i.  Each wave also fetches two of the
 //      chunk's eight diagonals for all 64 rows (one 256-byte row segment per
 //      instruction) and parks them in LDS.  Rows outside the operand and
-//      diagonal slots outside the matrix become zeros: they are given an
-//      out-of-range buffer offset (tiles touching the operand's first or last
-//      rows load row by row for that), so the arithmetic below needs no
-//      guards and never sees padding;
+//      diagonal slots outside the matrix become zeros (an out-of-range buffer
+//      offset reads as 0; pieces straddling the operand's first or last row
+//      are shifted into place on the way to LDS), so the arithmetic below
+//      needs no guards and never sees padding;
 //   2. each lane reads its column's window of 16 + LCK - 1 values with
 //      16-byte LDS reads (pitch/4 is odd, so the 64 lanes spread over all
 //      banks).  Every chunk is processed as LCK diagonals, LCK = the longest
@@ -172,92 +173,93 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 
 constexpr int SP_ROWS = 64;        // output rows per workgroup
 constexpr int SP_COLS = 64;        // batch columns per workgroup (one per lane)
-constexpr int SP_WAVES = 4;
-constexpr int SP_T = 16;           // rows per wave == lanes per DPP row
 constexpr int SP_QUADS = 20;       // 16-byte pieces staged per column (80 rows)
 constexpr int SP_CPI = 3;          // columns per load instruction (3 x 20 lanes)
 constexpr int SP_GROUPS = (SP_COLS + SP_CPI - 1) / SP_CPI;             // 22 column groups
-constexpr int SP_LOADS = (SP_GROUPS + SP_WAVES - 1) / SP_WAVES;        // 6 per wave per chunk
 constexpr int SP_PITCH = 84;       // floats between staged columns
 constexpr int SP_OPITCH = 68;      // floats between columns in the epilogue
-constexpr int SP_CPW = SP_COLS / SP_WAVES;      // columns each wave stores in the epilogue
 constexpr int SP_XFLOATS = SP_COLS * SP_PITCH;
 constexpr int SP_AVALS = CHUNK_MAX * SP_ROWS;   // diagonal values per workgroup per chunk
 constexpr int SP_DUMP = SP_XFLOATS + SP_AVALS;  // where idle lanes write
 constexpr int SP_STAGE_FLOATS = SP_DUMP + 4;
-constexpr int SP_APW = CHUNK_MAX / SP_WAVES;    // diagonals each wave fetches per chunk
+constexpr int SP_CHUNK_INTS = sizeof(Chunk) / 4;
+constexpr int SP_MAX_CHUNKS = 256;   // chunk-table entries kept in LDS
 
+// Per-wave shape: T rows (8 or 16, at most one DPP row of 16 lanes), so a
+// workgroup has 64 / T waves.
+template <int T>
+struct SpShape {
+    static_assert(T == 8 || T == 16, "rows per wave");
+    static constexpr int WAVES = SP_ROWS / T;
+    static constexpr int LOADS = (SP_GROUPS + WAVES - 1) / WAVES;      // 16-byte loads per wave per chunk
+    static constexpr int APW = CHUNK_MAX / WAVES;                      // diagonals each wave fetches per chunk
+    static constexpr int CPW = SP_COLS / WAVES;                        // columns each wave stores in the epilogue
+};
+
+template <int T>
 struct SpStage {
-    float4 x[SP_LOADS];
-    float a[SP_APW];
+    float4 x[SpShape<T>::LOADS];
+    float a[SpShape<T>::APW];
+    int shift;              // rows the pieces were fetched away from their place (0 except at the operand's ends)
+    bool edge;              // some staged row does not exist (wave-uniform)
 };
 
 // One chunk-table entry as a wave needs it: shift, length, and the table
-// positions of the two diagonals this wave fetches.
+// positions of the diagonals this wave fetches.
+template <int T>
 struct SpInfo {
     int s0, len;
-    int slot[SP_APW];
+    int slot[SpShape<T>::APW];
 };
 
-template <int LCK>
+template <int LCK, int T>
 struct SpWindow {
-    static constexpr int WQ = (SP_T + LCK - 1 + 3) / 4;
+    static constexpr int WQ = (T + LCK - 1 + 3) / 4;
     float w[WQ * 4];
     float a[LCK];
 };
 
-// acc[t] += bcast_t(a) * win[t + J], t = 0..15.  The DPP operand must not have
-// been written by a VALU instruction in the two preceding issue slots; the
-// leading s_nop covers whatever the compiler placed before the block.
-template <int J, int N>
-__device__ __forceinline__ void fma_row16(float (&acc)[SP_T], float a, const float (&win)[N])
+// acc[T0 + t] += bcast_{T0 + t}(a) * win[J + T0 + t], t = 0..7: eight FMAs whose
+// first operand is lane T0 + t of each 16-lane row of `a` (DPP row_newbcast).
+// A DPP operand must not have been written by a VALU instruction in the two
+// preceding issue slots; the leading s_nop covers whatever the compiler
+// placed before the block.
+template <int J, int T0, int NA, int NW>
+__device__ __forceinline__ void fma_block8(float (&acc)[NA], float a, const float (&win)[NW])
 {
-    asm(
-        "s_nop 1\n\t"
-        "v_fmac_f32_dpp %0, %8, %9 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %1, %8, %10 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %2, %8, %11 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %3, %8, %12 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %4, %8, %13 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %5, %8, %14 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %6, %8, %15 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %7, %8, %16 row_newbcast:7 row_mask:0xf bank_mask:0xf"
-        : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]),
-          "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
-        : "v"(a), "v"(win[J + 0]), "v"(win[J + 1]), "v"(win[J + 2]), "v"(win[J + 3]),
-          "v"(win[J + 4]), "v"(win[J + 5]), "v"(win[J + 6]), "v"(win[J + 7]));
-    asm(
-        "s_nop 1\n\t"
-        "v_fmac_f32_dpp %0, %8, %9 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %1, %8, %10 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %2, %8, %11 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %3, %8, %12 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %4, %8, %13 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %5, %8, %14 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %6, %8, %15 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %7, %8, %16 row_newbcast:15 row_mask:0xf bank_mask:0xf"
-        : "+v"(acc[8]), "+v"(acc[9]), "+v"(acc[10]), "+v"(acc[11]),
-          "+v"(acc[12]), "+v"(acc[13]), "+v"(acc[14]), "+v"(acc[15])
-        : "v"(a), "v"(win[J + 8]), "v"(win[J + 9]), "v"(win[J + 10]), "v"(win[J + 11]),
-          "v"(win[J + 12]), "v"(win[J + 13]), "v"(win[J + 14]), "v"(win[J + 15]));
+    asm("s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %8, %9 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %1, %8, %10 row_newbcast:%18 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %2, %8, %11 row_newbcast:%19 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %3, %8, %12 row_newbcast:%20 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %4, %8, %13 row_newbcast:%21 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %5, %8, %14 row_newbcast:%22 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %6, %8, %15 row_newbcast:%23 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %7, %8, %16 row_newbcast:%24 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc[T0 + 0]), "+v"(acc[T0 + 1]), "+v"(acc[T0 + 2]), "+v"(acc[T0 + 3]),
+          "+v"(acc[T0 + 4]), "+v"(acc[T0 + 5]), "+v"(acc[T0 + 6]), "+v"(acc[T0 + 7])
+        : "v"(a), "v"(win[J + T0 + 0]), "v"(win[J + T0 + 1]), "v"(win[J + T0 + 2]), "v"(win[J + T0 + 3]),
+          "v"(win[J + T0 + 4]), "v"(win[J + T0 + 5]), "v"(win[J + T0 + 6]), "v"(win[J + T0 + 7]),
+          "n"(T0 + 0), "n"(T0 + 1), "n"(T0 + 2), "n"(T0 + 3), "n"(T0 + 4), "n"(T0 + 5), "n"(T0 + 6), "n"(T0 + 7));
 }
 
-template <int LCK, int J>
-__device__ __forceinline__ void spmm_rows(float (&acc)[SP_T], const SpWindow<LCK> &win)
+template <int LCK, int T, int J>
+__device__ __forceinline__ void spmm_rows(float (&acc)[T], const SpWindow<LCK, T> &win)
 {
     if constexpr (J < LCK) {
-        fma_row16<J>(acc, win.a[J], win.w);
-        spmm_rows<LCK, J + 1>(acc, win);
+        fma_block8<J, 0>(acc, win.a[J], win.w);
+        if constexpr (T == 16) fma_block8<J, 8>(acc, win.a[J], win.w);
+        spmm_rows<LCK, T, J + 1>(acc, win);
     }
 }
 
-template <int LCK>
-__device__ __forceinline__ void spmm_read_window(SpWindow<LCK> &win, const float *win_lds,
+template <int LCK, int T>
+__device__ __forceinline__ void spmm_read_window(SpWindow<LCK, T> &win, const float *win_lds,
                                                  const float *a_lds)
 {
     const float4 *p4 = reinterpret_cast<const float4 *>(win_lds);
 #pragma unroll
-    for (int q = 0; q < SpWindow<LCK>::WQ; ++q) {
+    for (int q = 0; q < SpWindow<LCK, T>::WQ; ++q) {
         const float4 v = p4[q];
         win.w[4 * q + 0] = v.x; win.w[4 * q + 1] = v.y; win.w[4 * q + 2] = v.z; win.w[4 * q + 3] = v.w;
     }
@@ -284,13 +286,16 @@ __device__ __forceinline__ float4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, un
 }
 constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used here
 
-template <int LCK>
-__global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
+template <int LCK, int T>
+__global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes)
 {
+    typedef SpShape<T> S;
+    constexpr int SP_WAVES = S::WAVES, SP_LOADS = S::LOADS, SP_APW = S::APW, SP_CPW = S::CPW, SP_T = T;
     __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
+    __shared__ int ctab[SP_MAX_CHUNKS * SP_CHUNK_INTS];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -320,50 +325,43 @@ __global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
         col_off[it] = live ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) : OOB_OFFSET;
         lds_at[it] = live ? col * SP_PITCH + 4 * quad : SP_DUMP;
     }
-    // diagonal values: wave w fetches diagonals w and w + 4 of the chunk for
-    // the workgroup's 64 rows
+    // diagonal values: wave w fetches diagonals w, w + WAVES, ... of the chunk
+    // for the workgroup's 64 rows
     const __amdgpu_buffer_rsrc_t ar = make_rsrc(vals, a_bytes);
     const int arow = row0 + lane;
 
-    // The chunk table is read with vector loads at wave-uniform addresses, one
-    // chunk ahead of its use.  Scalar loads would share a counter with the
-    // LDS traffic and can only be waited for by draining it, which would
-    // serialise the LDS writes, the window reads and the FMAs of every
-    // iteration; vector loads retire in order and are waited for exactly.
-    const __amdgpu_buffer_rsrc_t cr = make_rsrc(chunks, (unsigned)nchunks * (unsigned)sizeof(Chunk));
-    auto fetch_info = [&](int c, SpInfo &info) {
-        const unsigned base = (unsigned)min(c, nchunks - 1) * (unsigned)sizeof(Chunk);
-        const auto sl = __builtin_amdgcn_raw_buffer_load_b64(cr, base, 0, 0);
-        info.s0 = sl[0];
-        info.len = sl[1];
+    // The chunk table sits in LDS for the whole kernel: reads of it retire in
+    // order with the other LDS traffic and can be waited for exactly.  (Scalar
+    // loads share the LDS counter but return out of order, so waiting for one
+    // drains every outstanding LDS operation; vector loads would queue behind
+    // the staging loads in flight.)
+    for (int i = threadIdx.x; i < nchunks * SP_CHUNK_INTS; i += 64 * SP_WAVES)
+        ctab[i] = reinterpret_cast<const int *>(chunks)[i];
+    __syncthreads();
+    auto fetch_info = [&](int c, SpInfo<T> &info) {
+        const int *e = ctab + min(c, nchunks - 1) * SP_CHUNK_INTS;
+        info.s0 = e[0];
+        info.len = e[1];
 #pragma unroll
-        for (int q = 0; q < SP_APW; ++q)
-            info.slot[q] = __builtin_amdgcn_raw_buffer_load_b32(cr, base + 8u + 4u * (unsigned)(wave + SP_WAVES * q), 0, 0);
+        for (int q = 0; q < SP_APW; ++q) info.slot[q] = e[2 + wave + SP_WAVES * q];
     };
 
-    auto issue = [&](const SpInfo &info, SpStage &st) {
+    // Dense rows come as 16-byte pieces.  A piece that straddles the operand's
+    // first or last row is fetched from the nearest in-range position instead
+    // (rows rc..rc+3) and shifted into place when it is written to LDS, so the
+    // loads themselves never branch.
+    auto issue = [&](const SpInfo<T> &info, SpStage<T> &st) {
         const int s0 = info.s0;
         const int a0 = row0 + s0;
         const int r = a0 + 4 * quad;                       // first dense row of this lane's piece
-        if ((a0 >= 0) & (a0 + 4 * SP_QUADS <= n_in)) {     // wave-uniform: every staged row exists
-            const unsigned row_off = (unsigned)r * 4u;
+        const int rc = min(max(r, 0), n_in - 4);
+        const bool any = (r > -4) & (r < n_in);            // at least one row of the piece exists
+        const unsigned row_off = (unsigned)rc * 4u;
 #pragma unroll
-            for (int it = 0; it < SP_LOADS; ++it)
-                st.x[it] = buffer_load_f32x4(xr, col_off[it] == OOB_OFFSET ? OOB_OFFSET : col_off[it] + row_off);
-        } else {
-            // first or last rows of the operand: row by row, a missing row gets
-            // the out-of-range offset and reads as 0
-#pragma unroll
-            for (int it = 0; it < SP_LOADS; ++it) {
-                float v[4];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const bool ok = (r + k >= 0) & (r + k < n_in) & (col_off[it] != OOB_OFFSET);
-                    v[k] = buffer_load_f32(xr, ok ? col_off[it] + (unsigned)(r + k) * 4u : OOB_OFFSET);
-                }
-                st.x[it] = make_float4(v[0], v[1], v[2], v[3]);
-            }
-        }
+        for (int it = 0; it < SP_LOADS; ++it)
+            st.x[it] = buffer_load_f32x4(xr, (any & (col_off[it] != OOB_OFFSET)) ? col_off[it] + row_off : OOB_OFFSET);
+        st.shift = rc - r;                                 // 0 except at the operand's ends
+        st.edge = (a0 < 0) | (a0 + 4 * SP_QUADS > n_in);   // wave-uniform
 #pragma unroll
         for (int q = 0; q < SP_APW; ++q) {
             const int j = wave + SP_WAVES * q;
@@ -375,49 +373,72 @@ __global__ __launch_bounds__(64 * SP_WAVES) void spmm_tiled_kernel(
             st.a[q] = buffer_load_f32(ar, ok ? off : OOB_OFFSET);
         }
     };
-    auto commit = [&](const SpStage &st, float *buf) {
+    auto commit = [&](const SpStage<T> &st, float *buf) {
+        if (!st.edge) {
 #pragma unroll
-        for (int it = 0; it < SP_LOADS; ++it)
-            *reinterpret_cast<float4 *>(buf + lds_at[it]) = st.x[it];
+            for (int it = 0; it < SP_LOADS; ++it)
+                *reinterpret_cast<float4 *>(buf + lds_at[it]) = st.x[it];
+        } else {
+            // out[k] = in[k - shift] where that exists, else 0
+            const int d = st.shift;
+#pragma unroll
+            for (int it = 0; it < SP_LOADS; ++it) {
+                const float v[4] = {st.x[it].x, st.x[it].y, st.x[it].z, st.x[it].w};
+                float o[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    float t = 0.f;
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) t = (k - d == m) ? v[m] : t;
+                    o[k] = t;
+                }
+                *reinterpret_cast<float4 *>(buf + lds_at[it]) = make_float4(o[0], o[1], o[2], o[3]);
+            }
+        }
 #pragma unroll
         for (int q = 0; q < SP_APW; ++q)
             buf[SP_XFLOATS + (wave + SP_WAVES * q) * SP_ROWS + lane] = st.a[q];
     };
-    auto read_window = [&](SpWindow<LCK> &win, const float *buf) {
-        spmm_read_window<LCK>(win, buf + lane * SP_PITCH + wave * SP_T,
-                                 buf + SP_XFLOATS + wave * SP_T + (lane & 15));
+    auto read_window = [&](SpWindow<LCK, T> &win, const float *buf) {
+        spmm_read_window<LCK, T>(win, buf + lane * SP_PITCH + wave * SP_T,
+                                 buf + SP_XFLOATS + wave * SP_T + (lane & (SP_T - 1)));
     };
     // Chunk k travels through stage set k & 1, LDS buffer k & 1, window set
     // k & 1 and table-entry set k & 1.  Entering iteration c: window(c) is in
     // registers, chunk c+1 has landed (or is landing) in `next`, chunk c+2 is
     // in flight in the other stage set, `info` holds table entry c+3.
-    auto iteration = [&](int c, SpStage &next, SpWindow<LCK> &win_cur, SpWindow<LCK> &win_next,
-                         SpInfo &info, SpInfo &info_next) {
-        if (c + 1 < nchunks) commit(next, lds[(c + 1) & 1]);
+    // Nothing in an iteration is conditional: past the end of the table the
+    // last chunk is staged again (and never used), so the number of loads in
+    // flight is the same on every path and each wait counts exactly.
+    auto iteration = [&](int c, SpStage<T> &next, SpWindow<LCK, T> &win_cur, SpWindow<LCK, T> &win_next,
+                         SpInfo<T> &info, SpInfo<T> &info_next) {
+        commit(next, lds[(c + 1) & 1]);
         fetch_info(c + 4, info_next);
-        if (c + 3 < nchunks) issue(info, next);
-        spmm_rows<LCK, 0>(acc, win_cur);
+        issue(info, next);
+        spmm_rows<LCK, T, 0>(acc, win_cur);
         __syncthreads();
-        if (c + 1 < nchunks) read_window(win_next, lds[(c + 1) & 1]);
+        read_window(win_next, lds[(c + 1) & 1]);
     };
 
-    SpStage st0, st1;
-    SpWindow<LCK> w0, w1;
-    SpInfo i0, i1;
+    SpStage<T> st0, st1;
+    SpWindow<LCK, T> w0, w1;
+    SpInfo<T> i0, i1;
     fetch_info(0, i0);
     fetch_info(1, i1);
     issue(i0, st0);
     fetch_info(2, i0);
-    if (nchunks > 1) issue(i1, st1);
+    issue(i1, st1);
     fetch_info(3, i1);
     commit(st0, lds[0]);
-    if (nchunks > 2) issue(i0, st0);
+    issue(i0, st0);
     __syncthreads();
     read_window(w0, lds[0]);
-    for (int c = 0; c < nchunks; c += 2) {
+    int c = 0;
+    for (; c + 1 < nchunks; c += 2) {
         iteration(c, st1, w0, w1, i1, i0);
-        if (c + 1 < nchunks) iteration(c + 1, st0, w1, w0, i0, i1);
+        iteration(c + 1, st0, w1, w0, i0, i1);
     }
+    if (c < nchunks) spmm_rows<LCK, T, 0>(acc, w0);        // odd table: the last window is already in registers
 
     // epilogue: lanes-along-columns -> lanes-along-rows through LDS (every
     // wave is past the last barrier, and the last window read came from the
@@ -635,7 +656,9 @@ bool spmm_tiled_ok(const DiaView &A, long long ldb, bool trans)
     const long long n_in = trans ? A.h : A.w;
     const long long x_bytes = ((SP_COLS - 1) * ldb + n_in) * 4;
     const long long a_bytes = (long long)A.nd * A.stride * 4;
-    return A.rf == 1 && x_bytes < (long long)OOB_OFFSET && a_bytes < (long long)OOB_OFFSET;
+    const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
+    return A.rf == 1 && n_in >= 4 && nchunks <= SP_MAX_CHUNKS && x_bytes < (long long)OOB_OFFSET &&
+           a_bytes < (long long)OOB_OFFSET;
 }
 
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
@@ -651,12 +674,21 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
     const int lck = trans ? A.max_len_t : A.max_len_n;
     const unsigned a_bytes = (unsigned)((long long)A.nd * A.stride * 4);
-    const dim3 grid((unsigned)(row_tiles * col_tiles)), block(64 * SP_WAVES);
+    const dim3 grid((unsigned)(row_tiles * col_tiles));
+    // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
+    // at the sizes this path is measured on; a wave issues a vector
+    // instruction only every ~6 cycles, so the SIMDs need that many waves.
+    const int rows_per_wave = g_spmm_rows_per_wave;
 #define CUVDIA_SPMM_LAUNCH(L)                                                                       \
     case L:                                                                                         \
-        hipLaunchKernelGGL(spmm_tiled_kernel<L>, grid, block, 0, stream, chunks, nchunks, vals,     \
-                           A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha,    \
-                           beta, (int)col_tiles, a_bytes);                                          \
+        if (rows_per_wave == 16)                                                                    \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 16>), grid, dim3(256), 0, stream, chunks,      \
+                               nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
+                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes);                  \
+        else                                                                                        \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8>), grid, dim3(512), 0, stream, chunks,       \
+                               nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
+                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes);                  \
         break;
     switch (lck) {
         CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
