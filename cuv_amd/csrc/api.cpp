@@ -244,7 +244,7 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
     if (batch > 0 && (lda < desc->h || ldb < desc->w)) return CUVDIA_ESHAPE;
 
     const int forced = g_path.load();
-    const bool tiled_possible = desc->rf == 1;
+    const bool tiled_possible = dd2dia_tiled_ok(desc->view, lda, ldb, batch);
     bool tiled;
     if (forced == CUVDIA_PATH_TILED) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;

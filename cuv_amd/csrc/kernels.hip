@@ -715,6 +715,12 @@ hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, 
     return hipGetLastError();
 }
 
+bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch)
+{
+    (void)lda; (void)ldb; (void)batch;
+    return C.rf == 1;
+}
+
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream)

@@ -42,6 +42,10 @@ hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, 
                                  const float *B, long long ldb, int batch,
                                  float alpha, float beta, hipStream_t stream);
 
+// Whether the tiled dd2dia can serve these operands (row_fact 1, operand
+// extents within its 32-bit buffer addressing).
+bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch);
+
 // Same contract, row_fact == 1 only: a workgroup owns 256 rows of one run
 // chunk; each lane keeps 4 rows x 8 diagonals of partial sums, the four
 // waves split the batch and are summed through LDS in wave order.
