@@ -33,6 +33,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+
+# HBM bytes per launch (fetch + write-back) measured with rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter read for a
+# 256 MiB device copy in the same run (FETCH_SIZE 0.50 KiB per KiB copied,
+# WRITE_SIZE 1.00); commands and readings: profiles/hbm_traffic_cfg1_cfg2_cfg3.md
+MEASURED_TRAFFIC_BYTES = {"up_pass": 23_060_000, "down_pass": 31_490_000, "weight_gradient": 26_260_000}
 FP32_VALU_PEAK_TFLOPS = 157.3  # published vector fp32 (packed); the kernels use no MFMA
 
 
@@ -45,6 +51,9 @@ def parse():
                     help="distinct operand sets rotated through (0: enough for > 512 MB)")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch from a Python loop instead of replaying HIP graphs")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy three times (known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
     return ap.parse_args()
@@ -137,6 +146,14 @@ def main():
 
     stream = torch.cuda.current_stream()
 
+    if args.calibrate_copy:
+        src = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device=dev)     # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # The kernels run for a few microseconds; a Python launch loop cannot feed
     # them that fast.  Launches are therefore captured into HIP graphs (one
     # graph = one rotation through the buffer sets) and the graphs replayed.
@@ -206,11 +223,11 @@ def main():
     for name, fn in (("up_pass", up), ("down_pass", down), ("weight_gradient", grad)):
         ms = timed(lambda i, fn=fn: fn(sets[0]), args.steps)
         warm[name] = ms * 1e3
-    kernel_names = {"up_pass": "spmm_tiled_kernel", "down_pass": "spmm_tiled_kernel",
+    kernel_names = {"up_pass": "spmm_tiled_kernel<7, 8>", "down_pass": "spmm_tiled_kernel<7, 8>",
                     "weight_gradient": "dd2dia_tiled_kernel"}
     dom = max(per, key=lambda k: per[k]["us"])
     roofline = dict(bound="hbm", achieved=per[dom]["gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=per[dom]["gbs"] / HBM_PEAK_GBS, traffic=None,
+                    frac=per[dom]["gbs"] / HBM_PEAK_GBS, traffic=MEASURED_TRAFFIC_BYTES.get(dom),
                     kernel=kernel_names[dom], op=dom, us_per_launch=per[dom]["us"],
                     algorithmic_bytes=per[dom]["bytes"])
 

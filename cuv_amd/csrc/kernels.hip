@@ -28,8 +28,8 @@ int g_spmm_rows_per_wave = 8;
 namespace {
 
 // Loads through this address space are issued on the scalar unit when the
-// address is wave-uniform: the chunk table is read into SGPRs and costs no
-// vector-memory or LDS bandwidth.
+// address is wave-uniform: a chunk-table entry is read into SGPRs and costs no
+// vector-memory or LDS bandwidth (used where the read sits outside a loop).
 typedef const Chunk __attribute__((address_space(4))) *sc_chunk_ptr;
 
 __device__ __forceinline__ sc_chunk_ptr scalar_ptr(const Chunk *p) { return (sc_chunk_ptr)p; }
@@ -141,8 +141,9 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 
 // -------------------------------------------------------------- tiled spmm --
 //
-// Workgroup = 64 output rows x 64 batch columns, 4 waves of 16 rows each.
-// Lane l of every wave owns batch column col0 + l and 16 running sums.  Per
+// Workgroup = 64 output rows x 64 batch columns, 64 / T waves of T rows each
+// (T = 8 by default, 16 optional; written for T = 16 below).
+// Lane l of every wave owns batch column col0 + l and T running sums.  Per
 // run chunk (<= 8 consecutive shifts starting at s0):
 //   1. the dense rows [a0, a0 + 80), a0 = row0 + s0, of the 64 columns are
 //      fetched with 16-byte buffer loads (4-byte aligned is all they need),

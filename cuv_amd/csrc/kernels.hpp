@@ -27,7 +27,7 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
 // Same contract, row_fact == 1 only: 64 output rows x 64 batch columns per
 // workgroup, dense tile staged through LDS once per run chunk, lanes own
 // batch columns and keep a sliding register window along the rows, diagonal
-// values arrive through the scalar unit.
+// values are broadcast across each 16-lane row by DPP.
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, hipStream_t stream);

@@ -283,3 +283,119 @@ def test_cfg4_reduced_multichannel(oracle, gu):
         gu.check_prod(oracle, _o_dia(oracle, wl), wl.X, None, trans, 1.0, 0.0, _lib.PATH_TILED, wl.name)
     wl = W.cfg4("dd2dia", px=64, batch=72, beta=0.9)
     gu.check_dd2dia(oracle, _o_dia(oracle, wl), wl.A, wl.B, 1.0 / 72, 0.9, _lib.PATH_TILED, wl.name)
+
+
+def test_cfg4_full_size_properties(gu):
+    """The large layer at its full shape (262144 rows, 4 x 13 x 13 = 676
+    diagonals, batch 256; about 57 GFLOP per product), where the CPU oracle
+    would take minutes.  Inputs are drawn on the device; what is checked does
+    not depend on the size:
+      * sampled output rows / diagonal slots against an fp64 evaluation of
+        the defining sum (rows at both ends, at channel boundaries, random),
+      * the generic and the tiled kernels agree on the whole result,
+      * <A*X, H> == <X, A^T*H>  and  <proj(P*Q^T), W> == <W*Q, P>  in fp64,
+      * padding slots (NaN) are neither read nor written.
+    Tolerance: 1e-5 of the summed term magnitudes per element."""
+    import torch
+    from cuv_amd import dia as D, _lib, workloads as W
+    L = _lib.lib()
+    dev = "cuda:0"
+    p = W.pattern_large(256, 4, 13)
+    n, nd, batch = p.h, len(p.offsets), 256
+    assert (n, nd) == (262144, 676) and p.stride == n
+    g = torch.Generator(device=dev)
+    g.manual_seed(0xC0FFEE + 4)
+    off = torch.tensor(np.asarray(p.offsets, np.int32), device=dev)
+    rows = torch.arange(n, dtype=torch.int32, device=dev)
+    col = rows[None, :] + off[:, None]
+    valid = (col >= 0) & (col < n)                      # (nd, n)
+    del col
+    assert int(valid.sum()) == 110616022
+
+    def new_dia(fill_valid):
+        m = D.dev_dia_matrix_f(n, n, nd, n, 1, device=dev)
+        m.set_offsets(p.offsets)
+        m.vec.copy_(torch.where(valid, fill_valid.view(nd, n), torch.full((), float("nan"), device=dev)).view(-1))
+        return m
+
+    A = new_dia(torch.randn(nd * n, generator=g, device=dev) * 0.01)
+    assert A.info()["nnz"] == 110616022
+    X = torch.rand(batch, n, generator=g, device=dev)
+    H = torch.rand(batch, n, generator=g, device=dev)
+    sample = torch.tensor(sorted(set(
+        [0, 1, 5, 6, 7, 255, 256, 1541, 1542, 65535, 65536, 65537, 131071, 131072, 196608, n - 1543, n - 1542,
+         n - 257, n - 7, n - 2, n - 1] + list(np.random.default_rng(4).integers(0, n, 27)))), device=dev)
+
+    def rows_expected(M, Bm, trans):
+        """fp64 value and term-magnitude sum of rows `sample` of op(M)*Bm."""
+        v = torch.nan_to_num(M.vec.view(nd, n))
+        if not trans:       # y[i] = sum_d v[d, i] * x[i + off_d]
+            src = sample[:, None] + off[None, :]
+            ok = (src >= 0) & (src < n)
+            a = v[:, sample].T
+        else:               # y[j] = sum_d v[d, j - off_d] * x[j - off_d]
+            src = sample[:, None] - off[None, :]
+            ok = (src >= 0) & (src < n)
+            a = v[torch.arange(nd, device=dev)[None, :], src.clamp(0, n - 1)]
+        a = (a * ok).double()
+        xs = Bm[:, src.clamp(0, n - 1)].double()      # (batch, rows, nd)
+        return torch.einsum("rd,crd->cr", a, xs), torch.einsum("rd,crd->cr", a.abs(), xs.abs())
+
+    def close(got, ref, mag, what):
+        assert torch.isfinite(got).all(), what
+        err = (got.double() - ref).abs()
+        assert bool((err <= 1e-5 * mag + 1e-30).all()), "%s: worst err/mag %.3g" % (what, float((err / (mag + 1e-30)).max()))
+
+    def run_prod(dst, M, Bm, trans, path):
+        _lib.check(L.cuvdia_set_path(path), "set_path")
+        try:
+            D.prod(dst, M, Bm, trans, "n", 1.0, 0.0)
+            assert L.cuvdia_last_path() == path
+        finally:
+            L.cuvdia_set_path(_lib.PATH_AUTO)
+
+    # forward and transposed products
+    Y = torch.full((batch, n), float("nan"), device=dev)
+    Yt = torch.full((batch, n), float("nan"), device=dev)
+    run_prod(Y, A, X, "n", _lib.PATH_TILED)
+    run_prod(Yt, A, H, "t", _lib.PATH_TILED)
+    for out, Bm, trans in ((Y, X, False), (Yt, H, True)):
+        ref, mag = rows_expected(A, Bm, trans)
+        close(out[:, sample], ref, mag, "cfg4 full %s sampled rows" % ("trans" if trans else "fwd"))
+    lhs = float((Y.double() * H.double()).sum())
+    rhs = float((X.double() * Yt.double()).sum())
+    scale = float((Y.double().abs() * H.double()).sum())
+    assert abs(lhs - rhs) <= 1e-5 * scale, ("adjoint identity", lhs, rhs, scale)
+    Yg = torch.full((batch, n), float("nan"), device=dev)
+    run_prod(Yg, A, X, "n", _lib.PATH_GENERIC)
+    assert float((Y - Yg).abs().max()) <= 1e-5 * float(Yg.abs().max()), "tiled vs generic"
+    del Yg, Yt
+
+    # weight gradient: G = proj(X * H^T) on the pattern, beta == 0 over NaN
+    G = new_dia(torch.zeros(nd * n, device=dev))
+    G.vec.fill_(float("nan"))
+    bd = D.dev_block_descriptor_f(G)
+    _lib.check(L.cuvdia_set_path(_lib.PATH_TILED), "set_path")
+    try:
+        D.densedense_to_dia(G, bd, X, H, 1.0 / batch, 0.0)
+        assert L.cuvdia_last_path() == _lib.PATH_TILED
+    finally:
+        L.cuvdia_set_path(_lib.PATH_AUTO)
+    Gv = G.vec.view(nd, n)
+    assert bool(torch.isnan(Gv[~valid]).all()), "padding slots were written"
+    assert bool(torch.isfinite(Gv[valid]).all()), "valid slots not written"
+    src = sample[:, None] + off[None, :]
+    ok = (src >= 0) & (src < n)
+    xs = X[:, sample].double()                                         # (batch, rows)
+    hs = H[:, src.clamp(0, n - 1)].double()                            # (batch, rows, nd)
+    ref = torch.einsum("cr,crd->dr", xs, hs) / batch
+    got = Gv[:, sample].double()
+    err = (got - ref).abs()[ok.T]
+    assert float(err.max()) <= 1e-5 * float(ref.abs().max()), "dd2dia sampled slots %.3g" % float(err.max())
+    # <proj(X H^T)/batch, A> == <A*H', X>/batch with H' = H: sum_valid G*A == <Y2, X>/batch, Y2 = A*H
+    Y2 = torch.full((batch, n), float("nan"), device=dev)
+    run_prod(Y2, A, H, "n", _lib.PATH_TILED)
+    lhs = float((torch.nan_to_num(Gv).double() * torch.nan_to_num(A.vec.view(nd, n)).double()).sum())
+    rhs = float((Y2.double() * X.double()).sum()) / batch
+    scale = float((Y2.double().abs() * X.double()).sum()) / batch
+    assert abs(lhs - rhs) <= 1e-5 * scale, ("gradient adjoint identity", lhs, rhs, scale)
