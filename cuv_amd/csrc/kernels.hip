@@ -465,39 +465,116 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
 
 // ------------------------------------------------------------ tiled dd2dia --
 //
-// Workgroup = 256 rows of ONE run chunk (<= 8 consecutive diagonals), 4 waves.
-// Lane l owns rows row0 + 4l .. 4l+3 and 4 x len partial sums; wave q walks
-// the batch-column groups g = q, q+4, ... (4 columns per group).  Per group
-// the wave stages, privately (no workgroup barrier), rows
-// [row0 + s0, row0 + s0 + 264) of B for the 4 columns into LDS with lanes
-// along rows; each lane then reads its 4 + len - 1 wide window with 16-byte
-// LDS reads, loads its 4 rows of A straight from global (16-byte, perfectly
-// coalesced) and issues 4 x len FMAs per column.  The staging of the next
-// group is issued before the FMAs of the current one.  The four waves'
-// partial sums meet in LDS and are added in wave order.
+// Workgroup = 256 rows of ONE run chunk, WAVES (4 or 8) waves.  Lane l owns
+// rows row0 + 4l .. 4l+3 and 4 x LC partial sums (LC = the longest chunk of
+// the table; positions past a chunk's own length are computed and dropped).
+// Wave q walks the batch-column groups g = q, q + WAVES, ... (4 columns per
+// group).  Per group the wave
+//   1. writes the group's rows [row0 + s0, row0 + s0 + 264) of B, which it
+//      fetched one step earlier with lanes along rows (4 + 1 dword buffer
+//      loads per column; rows outside B read as 0 through the buffer range
+//      check), to its private LDS buffer -- no workgroup barrier in the loop;
+//   2. requests the next group's rows of B and its own 4 rows x 4 columns of
+//      A (one 16-byte load per column when A allows it) -- columns past the
+//      batch go through an empty buffer resource and come back as zeros
+//      without touching memory, so the loop body never branches and every
+//      wait counts exactly;
+//   3. reads, per column, its 4 + LC - 1 wide window of B from LDS with
+//      16-byte reads and issues 4 x LC FMAs.
+// At the end the waves' partial sums meet in LDS and are added in wave order;
+// the result is written with lanes along rows (the values of C that beta
+// scales were fetched at kernel start).
 
 constexpr int DD_ROWS = 256;
-constexpr int DD_BG = 4;
-constexpr int DD_STAGED = 264;     // 256 + CHUNK_MAX
-constexpr int DD_PITCH = 264;
+constexpr int DD_BG = 4;           // batch columns per step
 
-template <int LC>
-__device__ __forceinline__ void dd2dia_tile(float *lds, sc_chunk_ptr ck, int row0,
-                                            float *__restrict__ C, long long stride,
-                                            const float *__restrict__ A, long long lda,
-                                            const float *__restrict__ B, long long ldb,
-                                            int h, int w, int batch, float alpha, float beta,
-                                            int a_vec)
+constexpr int DD_PITCH = 264;         // 256 + CHUNK_MAX staged rows of B per column
+
+constexpr int DD_WAVE_FLOATS = 2 * DD_BG * DD_PITCH + 4;   // two buffers + a slot idle lanes write to
+
+struct DdStage {
+    float b[DD_BG * 4 + 1];        // B: 4 x 64 rows per column, + 8 halo rows x 4 columns in one load
+    float a[DD_BG][4];             // A: this lane's 4 rows of each column
+};
+
+template <int LC, int WAVES, bool AVEC>
+__global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
+    const Chunk *__restrict__ chunks, int nchunks, float *__restrict__ C, int stride,
+    const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
+    int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
+    unsigned c_bytes)
 {
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
+    constexpr int RED_T = LC * 64 + 8;              // floats between the 4 rows a lane owns: keeps the
+                                                    // row-major read below free of bank conflicts
+    constexpr int RED_WAVE = 4 * RED_T;
+    constexpr int STAGE_FLOATS = WAVES * DD_WAVE_FLOATS;
+    constexpr int LDS_FLOATS = STAGE_FLOATS > WAVES * RED_WAVE ? STAGE_FLOATS : WAVES * RED_WAVE;
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int s0 = ck->s0;
-    const long long base = (long long)row0 + s0;
-    const bool b_interior = (base >= 0) & (base + DD_STAGED <= w);
-    const long long myrow = (long long)row0 + 4 * lane;
-    const bool a_full = (myrow + 3 < h) & (a_vec != 0);
+    const int tile = xcd_tile(blockIdx.x, gridDim.x);
+    const int rowtile = tile / nchunks;
+    const sc_chunk_ptr ck = scalar_ptr(chunks) + (tile - rowtile * nchunks);
+    const int row0 = rowtile * DD_ROWS;
+    // the whole table entry in three 16-byte scalar loads
+    typedef int int4v __attribute__((ext_vector_type(4)));
+    typedef const int4v __attribute__((address_space(4))) *sc_int4_ptr;
+    const int4v e0 = ((sc_int4_ptr)ck)[0], e1 = ((sc_int4_ptr)ck)[1], e2 = ((sc_int4_ptr)ck)[2];
+    const int s0 = e0.x;
+    const int slots[CHUNK_MAX] = {e0.z, e0.w, e1.x, e1.y, e1.z, e1.w, e2.x, e2.y};
+    const int base = row0 + s0;                     // first staged row of B
+    const int myrow = row0 + 4 * lane;
+
+    // C values this lane will combine at the end: row row0 + 64*wave' + lane
+    // of every diagonal of the chunk, wave' = wave, wave + WAVES, ... < 4
+    const int orow = row0 + lane;
+    float cpre[4 / (WAVES < 4 ? WAVES : 4)][LC];
+    constexpr int OSL = 4 / (WAVES < 4 ? WAVES : 4);
+    unsigned c_off[OSL][LC];
+    {
+        // beta == 0: C is not read (an empty resource returns zeros without touching memory)
+        const __amdgpu_buffer_rsrc_t cr = make_rsrc(C, beta != 0.f ? c_bytes : 0u);
+#pragma unroll
+        for (int u = 0; u < OSL; ++u)
+#pragma unroll
+            for (int j = 0; j < LC; ++j) {
+                const int sl = slots[j];
+                const int o = orow + 64 * (wave + WAVES * u);
+                const int in = o + s0 + j;
+                const bool ok = (wave + WAVES * u < 4) & (sl >= 0) & (o < h) & (in >= 0) & (in < w);
+                c_off[u][j] = ok ? ((unsigned)sl * (unsigned)stride + (unsigned)o) * 4u : OOB_OFFSET;
+                cpre[u][j] = buffer_load_f32(cr, c_off[u][j]);
+            }
+    }
+
+    // per-lane byte offsets inside one column; out-of-range rows use the marker
+    unsigned b_off[5];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int r = base + q * 64 + lane;
+        b_off[q] = (r >= 0 && r < w) ? (unsigned)r * 4u : OOB_OFFSET;
+    }
+    // the 8 rows past the 256 (the halo) of all 4 columns travel in one load:
+    // lane = 8 * column + row
+    const int hb = lane >> 3;
+    {
+        const int r = base + DD_ROWS + (lane & 7);
+        b_off[4] = (hb < DD_BG && r >= 0 && r < w) ? ((unsigned)r + (unsigned)hb * (unsigned)ldb) * 4u : OOB_OFFSET;
+    }
+    // where that load lands in buffer 0 / buffer 1 of this wave (idle lanes: the spare slot)
+    const int halo_at0 = hb < DD_BG ? hb * DD_PITCH + DD_ROWS + (lane & 7) : 2 * DD_BG * DD_PITCH;
+    const int halo_at1 = hb < DD_BG ? halo_at0 + DD_BG * DD_PITCH : 2 * DD_BG * DD_PITCH;
+    unsigned a_off[4];
+    if (AVEC) {
+        a_off[0] = (myrow + 3 < h) ? (unsigned)myrow * 4u : OOB_OFFSET;
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) a_off[t] = (myrow + t < h) ? (unsigned)(myrow + t) * 4u : OOB_OFFSET;
+    }
+    const unsigned lda4 = (unsigned)lda * 4u, ldb4 = (unsigned)ldb * 4u;
 
     float acc[4][LC];
 #pragma unroll
@@ -505,67 +582,52 @@ __device__ __forceinline__ void dd2dia_tile(float *lds, sc_chunk_ptr ck, int row
 #pragma unroll
         for (int j = 0; j < LC; ++j) acc[t][j] = 0.f;
 
-    float *mybuf = lds + wave * (2 * DD_BG * DD_PITCH);
-    const int ngroups = (batch + DD_BG - 1) / DD_BG;
-    float pre[DD_BG * 4 + 1];
-    const int hb = lane >> 3, hrow = DD_ROWS + (lane & 7);
+    float *mybuf = lds + wave * DD_WAVE_FLOATS;
+    const __amdgpu_buffer_rsrc_t b_all = make_rsrc(B, b_bytes);
 
-    auto issue = [&](int g) {
+    // requests group g: B rows into st.b, A rows into st.a
+    auto issue = [&](int g, DdStage &st) {
         const int b0 = g * DD_BG;
-        if (b_interior && b0 + DD_BG <= batch) {
 #pragma unroll
-            for (int i = 0; i < DD_BG; ++i)
+        for (int i = 0; i < DD_BG; ++i) {
+            const bool live = b0 + i < batch;
+            const __amdgpu_buffer_rsrc_t br = make_rsrc(B, live ? b_bytes : 0u);
+            const unsigned col = (unsigned)(b0 + i) * ldb4;
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    pre[i * 4 + q] = B[(long long)(b0 + i) * ldb + base + q * 64 + lane];
-            pre[DD_BG * 4] = (hb < DD_BG) ? B[(long long)(b0 + hb) * ldb + base + hrow] : 0.f;
-        } else {
+            for (int q = 0; q < 4; ++q)
+                st.b[i * 4 + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, b_off[q], col, 0));
+        }
+        // halo rows of column b0 + hb
+        st.b[DD_BG * 4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+            b_all, (b0 + hb < batch) ? b_off[4] : OOB_OFFSET, (unsigned)b0 * ldb4, 0));
 #pragma unroll
-            for (int i = 0; i < DD_BG; ++i)
+        for (int i = 0; i < DD_BG; ++i) {
+            const bool live = b0 + i < batch;
+            const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, live ? a_bytes : 0u);
+            const unsigned col = (unsigned)(b0 + i) * lda4;
+            if (AVEC) {
+                const float4 v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[0], col, 0));
+                st.a[i][0] = v.x; st.a[i][1] = v.y; st.a[i][2] = v.z; st.a[i][3] = v.w;
+            } else {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const long long r = base + q * 64 + lane;
-                    pre[i * 4 + q] = (b0 + i < batch && r >= 0 && r < w)
-                                         ? B[(long long)(b0 + i) * ldb + r] : 0.f;
-                }
-            const long long r = base + hrow;
-            pre[DD_BG * 4] = (hb < DD_BG && b0 + hb < batch && r >= 0 && r < w)
-                                 ? B[(long long)(b0 + hb) * ldb + r] : 0.f;
+                for (int t = 0; t < 4; ++t)
+                    st.a[i][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, a_off[t], col, 0));
+            }
         }
     };
-    auto commit = [&](float *buf) {
+    auto commit = [&](const DdStage &st, int par) {
+        float *buf = mybuf + par * (DD_BG * DD_PITCH);
 #pragma unroll
         for (int i = 0; i < DD_BG; ++i)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) buf[i * DD_PITCH + q * 64 + lane] = pre[i * 4 + q];
-        if (hb < DD_BG) buf[hb * DD_PITCH + hrow] = pre[DD_BG * 4];
+            for (int q = 0; q < 4; ++q) buf[i * DD_PITCH + q * 64 + lane] = st.b[i * 4 + q];
+        mybuf[par ? halo_at1 : halo_at0] = st.b[DD_BG * 4];
     };
-
-    int g = wave;
-    if (g < ngroups) { issue(g); commit(mybuf); }
-    for (int it = 0; g < ngroups; g += 4, ++it) {
-        float *cur = mybuf + (it & 1) * (DD_BG * DD_PITCH);
-        float *nxt = mybuf + ((it + 1) & 1) * (DD_BG * DD_PITCH);
-        const bool more = g + 4 < ngroups;
-        if (more) issue(g + 4);
-        wave_lds_fence();
+    auto compute = [&](const DdStage &st, const float *buf) {
 #pragma unroll
         for (int i = 0; i < DD_BG; ++i) {
-            const int b = g * DD_BG + i;
-            float a[4] = {0.f, 0.f, 0.f, 0.f};
-            if (b < batch) {
-                const float *ap = A + (long long)b * lda + myrow;
-                if (a_full) {
-                    const float4 v = *reinterpret_cast<const float4 *>(ap);
-                    a[0] = v.x; a[1] = v.y; a[2] = v.z; a[3] = v.w;
-                } else {
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        if (myrow + t < h) a[t] = ap[t];
-                }
-            }
             float win[WQ * 4];
-            const float4 *p4 = reinterpret_cast<const float4 *>(cur + i * DD_PITCH + 4 * lane);
+            const float4 *p4 = reinterpret_cast<const float4 *>(buf + i * DD_PITCH + 4 * lane);
 #pragma unroll
             for (int q = 0; q < WQ; ++q) {
                 const float4 v = p4[q];
@@ -575,55 +637,59 @@ __device__ __forceinline__ void dd2dia_tile(float *lds, sc_chunk_ptr ck, int row
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int j = 0; j < LC; ++j)
-                    acc[t][j] = __builtin_fmaf(a[t], win[t + j], acc[t][j]);
+                    acc[t][j] = __builtin_fmaf(st.a[i][t], win[t + j], acc[t][j]);
         }
+    };
+    // Step k works on group wave + WAVES*k out of stage set k & 1 and LDS
+    // buffer k & 1.  Entering a step its loads have been requested one step
+    // earlier; B goes to LDS, then the next group's loads are requested into
+    // the other stage set before the FMAs start, so they have a whole step to
+    // arrive.  Past the last group the requests hit the empty resource.
+    auto step = [&](int k, int par, DdStage &cur, DdStage &nxt) {
+        commit(cur, par);
+        issue(wave + WAVES * (k + 1), nxt);
         wave_lds_fence();
-        if (more) commit(nxt);
-    }
+        compute(cur, mybuf + par * (DD_BG * DD_PITCH));
+    };
 
-    // combine the four waves' partial sums in wave order
+    const int ngroups = (batch + DD_BG - 1) / DD_BG;
+    const int steps = (ngroups + WAVES - 1) / WAVES;        // same for every wave
+    DdStage st0, st1;
+    issue(wave, st0);
+    int k = 0;
+    for (; k + 1 < steps; k += 2) {
+        step(k, 0, st0, st1);
+        step(k + 1, 1, st1, st0);
+    }
+    if (k < steps) step(k, 0, st0, st1);
+
+    // combine the waves' partial sums in wave order
     __syncthreads();
-    float *red = lds;                      // [wave][4*LC][64]
+    float *red = lds;                               // [wave][t][j][64 lanes], t blocks RED_T apart
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int j = 0; j < LC; ++j)
-            red[(wave * 32 + t * LC + j) * 64 + lane] = acc[t][j];
+            red[wave * RED_WAVE + t * RED_T + j * 64 + lane] = acc[t][j];
     __syncthreads();
-    for (int j = wave; j < LC; j += 4) {
-        const int sl = ck->slot[j];
-        if (sl < 0) continue;                  // position no diagonal occupies
-        float *cd = C + (long long)sl * stride;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int ai = (t * LC + j) * 64 + lane;
-            const float total = ((red[ai] + red[32 * 64 + ai]) + red[2 * 32 * 64 + ai]) + red[3 * 32 * 64 + ai];
-            const long long o = myrow + t;
-            const long long in = o + s0 + j;
-            if (o < h && in >= 0 && in < w)
-                cd[o] = (beta == 0.f) ? alpha * total : beta * cd[o] + alpha * total;
+    for (int u = 0; u < OSL; ++u) {
+        const int ow = wave + WAVES * u;            // 64-row slice of the tile this pass writes
+        if (ow < 4) {
+            const int r = 64 * ow + lane;           // row within the tile: lane r/4 owned it as its row r%4
+            const float *src = red + (r & 3) * RED_T + (r >> 2);
+#pragma unroll
+            for (int j = 0; j < LC; ++j) {
+                float total = src[j * 64];
+#pragma unroll
+                for (int p = 1; p < WAVES; ++p) total += src[p * RED_WAVE + j * 64];
+                if (c_off[u][j] != OOB_OFFSET) {
+                    float *cd = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + c_off[u][j]);
+                    *cd = (beta == 0.f) ? alpha * total : beta * cpre[u][j] + alpha * total;
+                }
+            }
         }
     }
-}
-
-__global__ __launch_bounds__(256) void dd2dia_tiled_kernel(
-    const Chunk *__restrict__ chunks, int nchunks, float *__restrict__ C, int stride,
-    const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
-    int h, int w, int batch, float alpha, float beta, int a_vec)
-{
-    __shared__ __attribute__((aligned(16))) float lds[4 * 2 * DD_BG * DD_PITCH];
-    const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int rowtile = tile / nchunks;
-    const sc_chunk_ptr ck = scalar_ptr(chunks) + (tile - rowtile * nchunks);
-    const int row0 = rowtile * DD_ROWS;
-#define CUVDIA_DD_CASE(L) \
-    case L: dd2dia_tile<L>(lds, ck, row0, C, stride, A, lda, B, ldb, h, w, batch, alpha, beta, a_vec); break;
-    switch (ck->len) {
-        CUVDIA_DD_CASE(1) CUVDIA_DD_CASE(2) CUVDIA_DD_CASE(3) CUVDIA_DD_CASE(4)
-        CUVDIA_DD_CASE(5) CUVDIA_DD_CASE(6) CUVDIA_DD_CASE(7) CUVDIA_DD_CASE(8)
-        default: break;
-    }
-#undef CUVDIA_DD_CASE
 }
 
 }  // namespace
@@ -718,9 +784,16 @@ hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, 
 
 bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch)
 {
-    (void)lda; (void)ldb; (void)batch;
-    return C.rf == 1;
+    // buffer resources address 32-bit byte offsets below the out-of-range marker
+    const long long nb = batch > 0 ? batch : 1;
+    const long long a_bytes = ((nb - 1) * lda + C.h) * 4;
+    const long long b_bytes = ((nb - 1) * ldb + C.w) * 4;
+    const long long c_bytes = (long long)C.nd * C.stride * 4;
+    return C.rf == 1 && C.max_len_n >= 1 && a_bytes < (long long)OOB_OFFSET &&
+           b_bytes < (long long)OOB_OFFSET && c_bytes < (long long)OOB_OFFSET;
 }
+
+int g_dd2dia_waves = 4;
 
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
@@ -729,12 +802,34 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     const long long row_tiles = (C.h + DD_ROWS - 1) / DD_ROWS;
     const long long blocks = row_tiles * C.n_chunks_n;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    // 16-byte loads of A need an aligned base and leading dimension; row tiles
-    // start at multiples of 256 and lanes at multiples of 4 rows.
-    const int a_vec = (reinterpret_cast<unsigned long long>(A) % 16 == 0) && (lda % 4 == 0);
-    hipLaunchKernelGGL(dd2dia_tiled_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                       C.chunks_n_dev, C.n_chunks_n, vals, C.stride, A, lda, B, ldb,
-                       C.h, C.w, batch, alpha, beta, a_vec);
+    // 16-byte loads of A need an aligned base and leading dimension and whole
+    // groups of 4 rows; row tiles start at multiples of 256 and lanes at
+    // multiples of 4 rows.
+    const bool a_vec = (reinterpret_cast<unsigned long long>(A) % 16 == 0) && (lda % 4 == 0) && (C.h % 4 == 0);
+    const unsigned a_bytes = batch > 0 ? (unsigned)((((long long)batch - 1) * lda + C.h) * 4) : 0u;
+    const unsigned b_bytes = batch > 0 ? (unsigned)((((long long)batch - 1) * ldb + C.w) * 4) : 0u;
+    const unsigned c_bytes = (unsigned)((long long)C.nd * C.stride * 4);
+    const dim3 grid((unsigned)blocks);
+    const int waves = g_dd2dia_waves;
+#define CUVDIA_DD_ARGS C.chunks_n_dev, C.n_chunks_n, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
+                       a_bytes, b_bytes, c_bytes
+#define CUVDIA_DD_LAUNCH(L)                                                                              \
+    case L:                                                                                              \
+        if (waves == 8) {                                                                                \
+            if (a_vec) hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 8, true>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
+            else hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 8, false>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);       \
+        } else {                                                                                         \
+            if (a_vec) hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 4, true>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);  \
+            else hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 4, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);       \
+        }                                                                                                \
+        break;
+    switch (C.max_len_n) {
+        CUVDIA_DD_LAUNCH(1) CUVDIA_DD_LAUNCH(2) CUVDIA_DD_LAUNCH(3) CUVDIA_DD_LAUNCH(4)
+        CUVDIA_DD_LAUNCH(5) CUVDIA_DD_LAUNCH(6) CUVDIA_DD_LAUNCH(7) CUVDIA_DD_LAUNCH(8)
+        default: return hipErrorInvalidValue;
+    }
+#undef CUVDIA_DD_LAUNCH
+#undef CUVDIA_DD_ARGS
     return hipGetLastError();
 }
 

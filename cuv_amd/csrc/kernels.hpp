@@ -47,8 +47,8 @@ hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, 
 bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch);
 
 // Same contract, row_fact == 1 only: a workgroup owns 256 rows of one run
-// chunk; each lane keeps 4 rows x 8 diagonals of partial sums, the four
-// waves split the batch and are summed through LDS in wave order.
+// chunk; each lane keeps 4 rows x (longest chunk) diagonals of partial sums,
+// the four waves split the batch and are summed through LDS in wave order.
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream);
