@@ -174,9 +174,19 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
                       reinterpret_cast<const int *>(base),
                       reinterpret_cast<const Chunk *>(base + off_bytes), d->n_chunks_n,
                       reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t,
-                      0, 0};
-    for (const Chunk &c : cn) d->view.max_len_n = std::max(d->view.max_len_n, c.len);
-    for (const Chunk &c : ct) d->view.max_len_t = std::max(d->view.max_len_t, c.len);
+                      0, 0, 0, 0, 0, 0};
+    auto span = [](const std::vector<Chunk> &t, int &max_len, int &s_min, int &s_max) {
+        max_len = 0;
+        s_min = t.empty() ? 0 : t.front().s0;
+        s_max = s_min;
+        for (const Chunk &c : t) {
+            max_len = std::max(max_len, c.len);
+            s_min = std::min(s_min, c.s0);
+            s_max = std::max(s_max, c.s0);
+        }
+    };
+    span(cn, d->view.max_len_n, d->view.s_min_n, d->view.s_max_n);
+    span(ct, d->view.max_len_t, d->view.s_min_t, d->view.s_max_t);
     *out = d;
     return CUVDIA_OK;
 }

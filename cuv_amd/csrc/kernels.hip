@@ -287,23 +287,22 @@ __device__ __forceinline__ float4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, un
 }
 constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used here
 
-template <int LCK, int T>
-__global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
+// EDGE = false is the body for a tile whose staged rows all exist (every
+// chunk's 80 rows lie inside the dense operand and all 64 output rows exist):
+// row positions then enter the loads as a scalar offset, nothing is clamped
+// or shifted, and a chunk costs a couple of vector instructions besides its
+// FMAs.  EDGE = true handles the tiles at the operand's ends.
+template <int LCK, int T, bool EDGE>
+__device__ __forceinline__ void spmm_tile(
+    float (&lds)[2][SP_STAGE_FLOATS], int *ctab, int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
-    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes)
+    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes)
 {
     typedef SpShape<T> S;
     constexpr int SP_WAVES = S::WAVES, SP_LOADS = S::LOADS, SP_APW = S::APW, SP_CPW = S::CPW, SP_T = T;
-    __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
-    __shared__ int ctab[SP_MAX_CHUNKS * SP_CHUNK_INTS];
-
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int rowtile = tile / col_tiles;
-    const int row0 = rowtile * SP_ROWS;
-    const int col0 = (tile - rowtile * col_tiles) * SP_COLS;
     float acc[SP_T];
 #pragma unroll
     for (int t = 0; t < SP_T; ++t) acc[t] = 0.f;
@@ -313,8 +312,23 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     // Columns past the batch are replaced by the last valid one (their sums
     // are never stored).
     const int cols_here = min(SP_COLS, batch - col0);
-    const __amdgpu_buffer_rsrc_t xr =
-        make_rsrc(X + (long long)col0 * ldx, (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4));
+    const unsigned x_bytes = (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4);
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(X + (long long)col0 * ldx, x_bytes);
+
+    // beta != 0: the destination values this lane will combine at the end are
+    // requested now, so their trip from memory overlaps the whole product.
+    float ypre[SP_CPW];
+    {
+        const long long row = (long long)row0 + lane;
+        const __amdgpu_buffer_rsrc_t yr = make_rsrc(
+            Y + (long long)col0 * ldy, beta != 0.f ? (unsigned)(((long long)(cols_here - 1) * ldy + n_out) * 4) : 0u);
+#pragma unroll
+        for (int q = 0; q < SP_CPW; ++q) {
+            const int col = wave * SP_CPW + q;
+            ypre[q] = buffer_load_f32(yr, (row < n_out && col < cols_here)
+                                              ? (unsigned)(col * ldy + row) * 4u : OOB_OFFSET);
+        }
+    }
     const int grp = lane / SP_QUADS;               // column within the instruction's group (3: idle lane)
     const int quad = lane - grp * SP_QUADS;        // 16-byte piece within the column
     unsigned col_off[SP_LOADS];                    // byte offset of this lane's column per load
@@ -324,6 +338,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
         const int col = (wave + SP_WAVES * it) * SP_CPI + grp;
         const bool live = (grp < SP_CPI) & (col < SP_COLS);
         col_off[it] = live ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) : OOB_OFFSET;
+        if (!EDGE && live) col_off[it] += 16u * quad;      // the lane's piece; the chunk's first row is a scalar offset
         lds_at[it] = live ? col * SP_PITCH + 4 * quad : SP_DUMP;
     }
     // diagonal values: wave w fetches diagonals w, w + WAVES, ... of the chunk
@@ -341,18 +356,41 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     __syncthreads();
     auto fetch_info = [&](int c, SpInfo<T> &info) {
         const int *e = ctab + min(c, nchunks - 1) * SP_CHUNK_INTS;
-        info.s0 = e[0];
-        info.len = e[1];
+        // the entry is the same for every lane: keep it in scalar registers
+        info.s0 = __builtin_amdgcn_readfirstlane(e[0]);
+        info.len = __builtin_amdgcn_readfirstlane(e[1]);
 #pragma unroll
-        for (int q = 0; q < SP_APW; ++q) info.slot[q] = e[2 + wave + SP_WAVES * q];
+        for (int q = 0; q < SP_APW; ++q) info.slot[q] = __builtin_amdgcn_readfirstlane(e[2 + wave + SP_WAVES * q]);
     };
 
     // Dense rows come as 16-byte pieces.  A piece that straddles the operand's
     // first or last row is fetched from the nearest in-range position instead
     // (rows rc..rc+3) and shifted into place when it is written to LDS, so the
     // loads themselves never branch.
-    auto issue = [&](const SpInfo<T> &info, SpStage<T> &st) {
+    auto issue = [&](const SpInfo<T> &info, SpStage<T> &st, int c) {
         const int s0 = info.s0;
+        if constexpr (!EDGE) {
+            // past the table nothing is fetched: an empty resource returns zeros
+            const bool real = c < nchunks;
+            const __amdgpu_buffer_rsrc_t xq = make_rsrc(X + (long long)col0 * ldx, real ? x_bytes : 0u);
+            const unsigned soff = (unsigned)(row0 + s0) * 4u;
+#pragma unroll
+            for (int it = 0; it < SP_LOADS; ++it)
+                st.x[it] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(xq, col_off[it], soff, 0));
+            st.shift = 0;
+            st.edge = false;
+#pragma unroll
+            for (int q = 0; q < SP_APW; ++q) {
+                const int j = wave + SP_WAVES * q;
+                const int sl = info.slot[q];
+                const bool ok = real & (j < info.len) & (sl >= 0);
+                const __amdgpu_buffer_rsrc_t aq = make_rsrc(vals, ok ? a_bytes : 0u);
+                const unsigned voff = (unsigned)(ashift ? arow + s0 + j : arow) * 4u;
+                st.a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    aq, voff, (unsigned)sl * (unsigned)stride * 4u, 0));
+            }
+            return;
+        }
         const int a0 = row0 + s0;
         const int r = a0 + 4 * quad;                       // first dense row of this lane's piece
         const int rc = min(max(r, 0), n_in - 4);
@@ -375,7 +413,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
         }
     };
     auto commit = [&](const SpStage<T> &st, float *buf) {
-        if (!st.edge) {
+        if (!EDGE || !st.edge) {
 #pragma unroll
             for (int it = 0; it < SP_LOADS; ++it)
                 *reinterpret_cast<float4 *>(buf + lds_at[it]) = st.x[it];
@@ -415,7 +453,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
                          SpInfo<T> &info, SpInfo<T> &info_next) {
         commit(next, lds[(c + 1) & 1]);
         fetch_info(c + 4, info_next);
-        issue(info, next);
+        issue(info, next, c + 3);
         spmm_rows<LCK, T, 0>(acc, win_cur);
         __syncthreads();
         read_window(win_next, lds[(c + 1) & 1]);
@@ -426,20 +464,28 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     SpInfo<T> i0, i1;
     fetch_info(0, i0);
     fetch_info(1, i1);
-    issue(i0, st0);
+    issue(i0, st0, 0);
     fetch_info(2, i0);
-    issue(i1, st1);
+    issue(i1, st1, 1);
     fetch_info(3, i1);
     commit(st0, lds[0]);
-    issue(i0, st0);
+    issue(i0, st0, 2);
     __syncthreads();
     read_window(w0, lds[0]);
     int c = 0;
-    for (; c + 1 < nchunks; c += 2) {
+    if (nchunks & 1) {
+        // odd table: one chunk alone first, then the register sets trade
+        // places so the paired loop below starts in its usual state
+        iteration(0, st1, w0, w1, i1, i0);
+        { const SpStage<T> t = st0; st0 = st1; st1 = t; }
+        { const SpWindow<LCK, T> t = w0; w0 = w1; w1 = t; }
+        { const SpInfo<T> t = i0; i0 = i1; i1 = t; }
+        c = 1;
+    }
+    for (; c < nchunks; c += 2) {
         iteration(c, st1, w0, w1, i1, i0);
         iteration(c + 1, st0, w1, w0, i0, i1);
     }
-    if (c < nchunks) spmm_rows<LCK, T, 0>(acc, w0);        // odd table: the last window is already in registers
 
     // epilogue: lanes-along-columns -> lanes-along-rows through LDS (every
     // wave is past the last barrier, and the last window read came from the
@@ -457,10 +503,33 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
             if (col0 + col < batch) {
                 const float v = out[col * SP_OPITCH + lane];
                 float *y = Y + (long long)(col0 + col) * ldy + row;
-                *y = (beta == 0.f) ? alpha * v : beta * (*y) + alpha * v;
+                *y = (beta == 0.f) ? alpha * v : beta * ypre[q] + alpha * v;
             }
         }
     }
+}
+
+template <int LCK, int T>
+__global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
+    const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
+    int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
+    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes,
+    int s_min, int s_max)
+{
+    __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
+    __shared__ int ctab[SP_MAX_CHUNKS * SP_CHUNK_INTS];
+    const int tile = xcd_tile(blockIdx.x, gridDim.x);
+    const int rowtile = tile / col_tiles;
+    const int row0 = rowtile * SP_ROWS;
+    const int col0 = (tile - rowtile * col_tiles) * SP_COLS;
+    // every chunk's staged rows [row0 + s0, row0 + s0 + 80) inside the operand, all 64 output rows real
+    const bool interior = (row0 + s_min >= 0) & (row0 + s_max + 4 * SP_QUADS <= n_in) & (row0 + SP_ROWS <= n_out);
+    if (interior)
+        spmm_tile<LCK, T, false>(lds, ctab, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+                                 n_out, n_in, batch, alpha, beta, a_bytes);
+    else
+        spmm_tile<LCK, T, true>(lds, ctab, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+                                n_out, n_in, batch, alpha, beta, a_bytes);
 }
 
 // ------------------------------------------------------------ tiled dd2dia --
@@ -528,26 +597,23 @@ __global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
     const int base = row0 + s0;                     // first staged row of B
     const int myrow = row0 + 4 * lane;
 
-    // C values this lane will combine at the end: row row0 + 64*wave' + lane
-    // of every diagonal of the chunk, wave' = wave, wave + WAVES, ... < 4
-    const int orow = row0 + lane;
-    float cpre[4 / (WAVES < 4 ? WAVES : 4)][LC];
-    constexpr int OSL = 4 / (WAVES < 4 ? WAVES : 4);
-    unsigned c_off[OSL][LC];
+    // C values this lane will combine at the end: row row0 + 64*wave + lane of
+    // every diagonal of the chunk (waves 0..3; a workgroup of 8 waves leaves
+    // the output to its first four).  Byte offset of that slot, or the
+    // out-of-range marker where no matrix element sits.
+    auto c_offset = [&](int j) -> unsigned {
+        const int sl = slots[j];
+        const int o = row0 + 64 * wave + lane;
+        const int in = o + s0 + j;
+        const bool ok = (wave < 4) & (sl >= 0) & (o < h) & (in >= 0) & (in < w);
+        return ok ? ((unsigned)sl * (unsigned)stride + (unsigned)o) * 4u : OOB_OFFSET;
+    };
+    float cpre[LC];
     {
         // beta == 0: C is not read (an empty resource returns zeros without touching memory)
         const __amdgpu_buffer_rsrc_t cr = make_rsrc(C, beta != 0.f ? c_bytes : 0u);
 #pragma unroll
-        for (int u = 0; u < OSL; ++u)
-#pragma unroll
-            for (int j = 0; j < LC; ++j) {
-                const int sl = slots[j];
-                const int o = orow + 64 * (wave + WAVES * u);
-                const int in = o + s0 + j;
-                const bool ok = (wave + WAVES * u < 4) & (sl >= 0) & (o < h) & (in >= 0) & (in < w);
-                c_off[u][j] = ok ? ((unsigned)sl * (unsigned)stride + (unsigned)o) * 4u : OOB_OFFSET;
-                cpre[u][j] = buffer_load_f32(cr, c_off[u][j]);
-            }
+        for (int j = 0; j < LC; ++j) cpre[j] = buffer_load_f32(cr, c_offset(j));
     }
 
     // per-lane byte offsets inside one column; out-of-range rows use the marker
@@ -585,71 +651,91 @@ __global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
     float *mybuf = lds + wave * DD_WAVE_FLOATS;
     const __amdgpu_buffer_rsrc_t b_all = make_rsrc(B, b_bytes);
 
-    // requests group g: B rows into st.b, A rows into st.a
-    auto issue = [&](int g, DdStage &st) {
+    // requests column i of group g: B rows into st.b, A rows into st.a (the
+    // halo load, which serves all 4 columns, travels with column 0)
+    auto issue_col = [&](int g, int i, DdStage &st) {
         const int b0 = g * DD_BG;
+        const bool live = b0 + i < batch;
+        const __amdgpu_buffer_rsrc_t br = make_rsrc(B, live ? b_bytes : 0u);
+        const unsigned colb = (unsigned)(b0 + i) * ldb4;
 #pragma unroll
-        for (int i = 0; i < DD_BG; ++i) {
-            const bool live = b0 + i < batch;
-            const __amdgpu_buffer_rsrc_t br = make_rsrc(B, live ? b_bytes : 0u);
-            const unsigned col = (unsigned)(b0 + i) * ldb4;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                st.b[i * 4 + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, b_off[q], col, 0));
-        }
-        // halo rows of column b0 + hb
-        st.b[DD_BG * 4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-            b_all, (b0 + hb < batch) ? b_off[4] : OOB_OFFSET, (unsigned)b0 * ldb4, 0));
-#pragma unroll
-        for (int i = 0; i < DD_BG; ++i) {
-            const bool live = b0 + i < batch;
-            const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, live ? a_bytes : 0u);
-            const unsigned col = (unsigned)(b0 + i) * lda4;
-            if (AVEC) {
-                const float4 v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[0], col, 0));
-                st.a[i][0] = v.x; st.a[i][1] = v.y; st.a[i][2] = v.z; st.a[i][3] = v.w;
-            } else {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    st.a[i][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, a_off[t], col, 0));
-            }
-        }
-    };
-    auto commit = [&](const DdStage &st, int par) {
-        float *buf = mybuf + par * (DD_BG * DD_PITCH);
-#pragma unroll
-        for (int i = 0; i < DD_BG; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) buf[i * DD_PITCH + q * 64 + lane] = st.b[i * 4 + q];
-        mybuf[par ? halo_at1 : halo_at0] = st.b[DD_BG * 4];
-    };
-    auto compute = [&](const DdStage &st, const float *buf) {
-#pragma unroll
-        for (int i = 0; i < DD_BG; ++i) {
-            float win[WQ * 4];
-            const float4 *p4 = reinterpret_cast<const float4 *>(buf + i * DD_PITCH + 4 * lane);
-#pragma unroll
-            for (int q = 0; q < WQ; ++q) {
-                const float4 v = p4[q];
-                win[4 * q + 0] = v.x; win[4 * q + 1] = v.y; win[4 * q + 2] = v.z; win[4 * q + 3] = v.w;
-            }
+        for (int q = 0; q < 4; ++q)
+            st.b[i * 4 + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, b_off[q], colb, 0));
+        if (i == 0)
+            st.b[DD_BG * 4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                b_all, (b0 + hb < batch) ? b_off[4] : OOB_OFFSET, (unsigned)b0 * ldb4, 0));
+        const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, live ? a_bytes : 0u);
+        const unsigned cola = (unsigned)(b0 + i) * lda4;
+        if (AVEC) {
+            const float4 v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[0], cola, 0));
+            st.a[i][0] = v.x; st.a[i][1] = v.y; st.a[i][2] = v.z; st.a[i][3] = v.w;
+        } else {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int j = 0; j < LC; ++j)
-                    acc[t][j] = __builtin_fmaf(st.a[i][t], win[t + j], acc[t][j]);
+                st.a[i][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, a_off[t], cola, 0));
         }
     };
-    // Step k works on group wave + WAVES*k out of stage set k & 1 and LDS
-    // buffer k & 1.  Entering a step its loads have been requested one step
-    // earlier; B goes to LDS, then the next group's loads are requested into
-    // the other stage set before the FMAs start, so they have a whole step to
-    // arrive.  Past the last group the requests hit the empty resource.
-    auto step = [&](int k, int par, DdStage &cur, DdStage &nxt) {
-        commit(cur, par);
-        issue(wave + WAVES * (k + 1), nxt);
+    auto issue = [&](int g, DdStage &st) {
+#pragma unroll
+        for (int i = 0; i < DD_BG; ++i) issue_col(g, i, st);
+    };
+    auto commit_col = [&](const DdStage &st, int par, int i) {
+        float *buf = mybuf + par * (DD_BG * DD_PITCH);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) buf[i * DD_PITCH + q * 64 + lane] = st.b[i * 4 + q];
+        if (i == 0) mybuf[par ? halo_at1 : halo_at0] = st.b[DD_BG * 4];
         wave_lds_fence();
-        compute(cur, mybuf + par * (DD_BG * DD_PITCH));
+    };
+    auto read_window = [&](float (&win)[WQ * 4], const float *buf, int i) {
+        const float4 *p4 = reinterpret_cast<const float4 *>(buf + i * DD_PITCH + 4 * lane);
+#pragma unroll
+        for (int q = 0; q < WQ; ++q) {
+            const float4 v = p4[q];
+            win[4 * q + 0] = v.x; win[4 * q + 1] = v.y; win[4 * q + 2] = v.z; win[4 * q + 3] = v.w;
+        }
+    };
+    auto fmas = [&](const float (&a)[4], const float (&win)[WQ * 4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int j = 0; j < LC; ++j) acc[t][j] = __builtin_fmaf(a[t], win[t + j], acc[t][j]);
+    };
+    // Step k works on group wave + WAVES*k out of stage set k & 1 and LDS
+    // buffer k & 1, one column at a time: column i's rows of B go to LDS and
+    // its window is read back while the FMAs of column i - 1 run; column i of
+    // the next group is requested right after, so every load has one whole
+    // step to arrive and the requests are spread between the FMA blocks -- a
+    // wave that has to wait for room in the memory pipeline leaves the SIMD
+    // to the other wave's FMAs instead of holding its own back.  Past the last
+    // group the requests hit the empty resource.
+    auto step = [&](int k, int par, DdStage &cur, DdStage &nxt) {
+        const float *buf = mybuf + par * (DD_BG * DD_PITCH);
+        const int gn = wave + WAVES * (k + 1);
+        float w0[WQ * 4], w1[WQ * 4];
+        commit_col(cur, par, 0);
+        read_window(w0, buf, 0);
+        commit_col(cur, par, 1);
+        read_window(w1, buf, 1);
+        issue_col(gn, 0, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        fmas(cur.a[0], w0);
+        __builtin_amdgcn_sched_barrier(0);
+        commit_col(cur, par, 2);
+        read_window(w0, buf, 2);
+        issue_col(gn, 1, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        fmas(cur.a[1], w1);
+        __builtin_amdgcn_sched_barrier(0);
+        commit_col(cur, par, 3);
+        read_window(w1, buf, 3);
+        issue_col(gn, 2, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        fmas(cur.a[2], w0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_col(gn, 3, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        fmas(cur.a[3], w1);
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     const int ngroups = (batch + DD_BG - 1) / DD_BG;
@@ -672,21 +758,18 @@ __global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
         for (int j = 0; j < LC; ++j)
             red[wave * RED_WAVE + t * RED_T + j * 64 + lane] = acc[t][j];
     __syncthreads();
+    if (wave < 4) {
+        const int r = 64 * wave + lane;             // row within the tile: lane r/4 owned it as its row r%4
+        const float *src = red + (r & 3) * RED_T + (r >> 2);
 #pragma unroll
-    for (int u = 0; u < OSL; ++u) {
-        const int ow = wave + WAVES * u;            // 64-row slice of the tile this pass writes
-        if (ow < 4) {
-            const int r = 64 * ow + lane;           // row within the tile: lane r/4 owned it as its row r%4
-            const float *src = red + (r & 3) * RED_T + (r >> 2);
+        for (int j = 0; j < LC; ++j) {
+            float total = src[j * 64];
 #pragma unroll
-            for (int j = 0; j < LC; ++j) {
-                float total = src[j * 64];
-#pragma unroll
-                for (int p = 1; p < WAVES; ++p) total += src[p * RED_WAVE + j * 64];
-                if (c_off[u][j] != OOB_OFFSET) {
-                    float *cd = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + c_off[u][j]);
-                    *cd = (beta == 0.f) ? alpha * total : beta * cpre[u][j] + alpha * total;
-                }
+            for (int p = 1; p < WAVES; ++p) total += src[p * RED_WAVE + j * 64];
+            const unsigned off = c_offset(j);
+            if (off != OOB_OFFSET) {
+                float *cd = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
+                *cd = (beta == 0.f) ? alpha * total : beta * cpre[j] + alpha * total;
             }
         }
     }
@@ -741,6 +824,7 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
     const int lck = trans ? A.max_len_t : A.max_len_n;
     const unsigned a_bytes = (unsigned)((long long)A.nd * A.stride * 4);
+    const int s_min = trans ? A.s_min_t : A.s_min_n, s_max = trans ? A.s_max_t : A.s_max_n;
     const dim3 grid((unsigned)(row_tiles * col_tiles));
     // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
     // at the sizes this path is measured on; a wave issues a vector
@@ -751,11 +835,11 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
         if (rows_per_wave == 16)                                                                    \
             hipLaunchKernelGGL((spmm_tiled_kernel<L, 16>), grid, dim3(256), 0, stream, chunks,      \
                                nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
-                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes);                  \
+                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);                  \
         else                                                                                        \
             hipLaunchKernelGGL((spmm_tiled_kernel<L, 8>), grid, dim3(512), 0, stream, chunks,       \
                                nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
-                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes);                  \
+                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);                  \
         break;
     switch (lck) {
         CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)

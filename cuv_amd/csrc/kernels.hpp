@@ -16,6 +16,8 @@ struct DiaView {
     const Chunk *chunks_t_dev;   // shifts = -offsets
     int n_chunks_t;
     int max_len_n, max_len_t;    // longest chunk of each table
+    int s_min_n, s_max_n;        // smallest / largest chunk shift of each table
+    int s_min_t, s_max_t;
 };
 
 // dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch
