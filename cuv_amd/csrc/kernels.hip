@@ -24,7 +24,6 @@
 #include "kernels.hpp"
 
 namespace cuvdia {
-int g_spmm_rows_per_wave = 8;
 namespace {
 
 // Loads through this address space are issued on the scalar unit when the
@@ -142,7 +141,7 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 // -------------------------------------------------------------- tiled spmm --
 //
 // Workgroup = 64 output rows x 64 batch columns, 64 / T waves of T rows each
-// (T = 8 by default, 16 optional; written for T = 16 below).
+// (T = 8 is what the launcher uses; the text below is written for T = 16).
 // Lane l of every wave owns batch column col0 + l and T running sums.  Per
 // run chunk (<= 8 consecutive shifts starting at s0):
 //   1. the dense rows [a0, a0 + 80), a0 = row0 + s0, of the 64 columns are
@@ -168,7 +167,8 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
 // The loop is software-pipelined three chunks deep: while the FMAs of chunk c
 // run out of registers, chunk c+1 is being written to the other LDS buffer
 // (its window is read right after the barrier), chunk c+2 is in flight from
-// memory and chunk c+3 has just been requested.
+// memory and chunk c+3 has just been requested.  The chunk table itself sits
+// in vector registers (lane i <-> entry i) and is read with v_readlane.
 // The epilogue transposes the sums through LDS so the store to dst is again
 // lanes-along-rows.
 
@@ -183,8 +183,7 @@ constexpr int SP_XFLOATS = SP_COLS * SP_PITCH;
 constexpr int SP_AVALS = CHUNK_MAX * SP_ROWS;   // diagonal values per workgroup per chunk
 constexpr int SP_DUMP = SP_XFLOATS + SP_AVALS;  // where idle lanes write
 constexpr int SP_STAGE_FLOATS = SP_DUMP + 4;
-constexpr int SP_CHUNK_INTS = sizeof(Chunk) / 4;
-constexpr int SP_MAX_CHUNKS = 256;   // chunk-table entries kept in LDS
+constexpr int SP_MAX_CHUNKS = 256;   // chunk-table entries a wave can keep in registers (4 sets of 64)
 
 // Per-wave shape: T rows (8 or 16, at most one DPP row of 16 lanes), so a
 // workgroup has 64 / T waves.
@@ -292,9 +291,9 @@ constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used 
 // row positions then enter the loads as a scalar offset, nothing is clamped
 // or shifted, and a chunk costs a couple of vector instructions besides its
 // FMAs.  EDGE = true handles the tiles at the operand's ends.
-template <int LCK, int T, bool EDGE>
+template <int LCK, int T, int NTAB, bool EDGE>
 __device__ __forceinline__ void spmm_tile(
-    float (&lds)[2][SP_STAGE_FLOATS], int *ctab, int row0, int col0,
+    float (&lds)[2][SP_STAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes)
@@ -346,21 +345,38 @@ __device__ __forceinline__ void spmm_tile(
     const __amdgpu_buffer_rsrc_t ar = make_rsrc(vals, a_bytes);
     const int arow = row0 + lane;
 
-    // The chunk table sits in LDS for the whole kernel: reads of it retire in
-    // order with the other LDS traffic and can be waited for exactly.  (Scalar
-    // loads share the LDS counter but return out of order, so waiting for one
-    // drains every outstanding LDS operation; vector loads would queue behind
-    // the staging loads in flight.)
-    for (int i = threadIdx.x; i < nchunks * SP_CHUNK_INTS; i += 64 * SP_WAVES)
-        ctab[i] = reinterpret_cast<const int *>(chunks)[i];
-    __syncthreads();
-    auto fetch_info = [&](int c, SpInfo<T> &info) {
-        const int *e = ctab + min(c, nchunks - 1) * SP_CHUNK_INTS;
-        // the entry is the same for every lane: keep it in scalar registers
-        info.s0 = __builtin_amdgcn_readfirstlane(e[0]);
-        info.len = __builtin_amdgcn_readfirstlane(e[1]);
+    // The chunk table lives in vector registers, lane i of set k holding what
+    // this wave needs of entry 64*k + i (shift, length, and the table position
+    // of the diagonals it fetches); an entry is read with v_readlane into
+    // scalar registers.  Nothing in the loop waits on memory for it.
+    int tab_s0[NTAB], tab_len[NTAB], tab_slot[NTAB][SP_APW];
 #pragma unroll
-        for (int q = 0; q < SP_APW; ++q) info.slot[q] = __builtin_amdgcn_readfirstlane(e[2 + wave + SP_WAVES * q]);
+    for (int k = 0; k < NTAB; ++k) {
+        const int *e = reinterpret_cast<const int *>(chunks + min(64 * k + lane, nchunks - 1));
+        tab_s0[k] = e[0];
+        tab_len[k] = e[1];
+#pragma unroll
+        for (int q = 0; q < SP_APW; ++q) tab_slot[k][q] = e[2 + wave + SP_WAVES * q];
+    }
+    auto fetch_info = [&](int c, SpInfo<T> &info) {
+        const int cc = min(c, nchunks - 1);
+        const int l = cc & 63;
+        info.s0 = __builtin_amdgcn_readlane(tab_s0[0], l);
+        info.len = __builtin_amdgcn_readlane(tab_len[0], l);
+#pragma unroll
+        for (int q = 0; q < SP_APW; ++q) info.slot[q] = __builtin_amdgcn_readlane(tab_slot[0][q], l);
+#pragma unroll
+        for (int k = 1; k < NTAB; ++k) {
+            const bool here = (cc >> 6) == k;
+            const int s0 = __builtin_amdgcn_readlane(tab_s0[k], l), len = __builtin_amdgcn_readlane(tab_len[k], l);
+            info.s0 = here ? s0 : info.s0;
+            info.len = here ? len : info.len;
+#pragma unroll
+            for (int q = 0; q < SP_APW; ++q) {
+                const int sl = __builtin_amdgcn_readlane(tab_slot[k][q], l);
+                info.slot[q] = here ? sl : info.slot[q];
+            }
+        }
     };
 
     // Dense rows come as 16-byte pieces.  A piece that straddles the operand's
@@ -509,7 +525,7 @@ __device__ __forceinline__ void spmm_tile(
     }
 }
 
-template <int LCK, int T>
+template <int LCK, int T, int NTAB>
 __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
@@ -517,7 +533,6 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     int s_min, int s_max)
 {
     __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
-    __shared__ int ctab[SP_MAX_CHUNKS * SP_CHUNK_INTS];
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
     const int rowtile = tile / col_tiles;
     const int row0 = rowtile * SP_ROWS;
@@ -525,10 +540,10 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     // every chunk's staged rows [row0 + s0, row0 + s0 + 80) inside the operand, all 64 output rows real
     const bool interior = (row0 + s_min >= 0) & (row0 + s_max + 4 * SP_QUADS <= n_in) & (row0 + SP_ROWS <= n_out);
     if (interior)
-        spmm_tile<LCK, T, false>(lds, ctab, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+        spmm_tile<LCK, T, NTAB, false>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                  n_out, n_in, batch, alpha, beta, a_bytes);
     else
-        spmm_tile<LCK, T, true>(lds, ctab, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+        spmm_tile<LCK, T, NTAB, true>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                 n_out, n_in, batch, alpha, beta, a_bytes);
 }
 
@@ -827,19 +842,17 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const int s_min = trans ? A.s_min_t : A.s_min_n, s_max = trans ? A.s_max_t : A.s_max_n;
     const dim3 grid((unsigned)(row_tiles * col_tiles));
     // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
-    // at the sizes this path is measured on; a wave issues a vector
-    // instruction only every ~6 cycles, so the SIMDs need that many waves.
-    const int rows_per_wave = g_spmm_rows_per_wave;
+    // at the sizes this path is measured on.
 #define CUVDIA_SPMM_LAUNCH(L)                                                                       \
     case L:                                                                                         \
-        if (rows_per_wave == 16)                                                                    \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 16>), grid, dim3(256), 0, stream, chunks,      \
+        if (nchunks <= 64)                                                                          \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 1>), grid, dim3(512), 0, stream, chunks,    \
                                nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
-                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);                  \
+                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);    \
         else                                                                                        \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8>), grid, dim3(512), 0, stream, chunks,       \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 4>), grid, dim3(512), 0, stream, chunks,    \
                                nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
-                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);                  \
+                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);    \
         break;
     switch (lck) {
         CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
