@@ -137,11 +137,14 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
 
     cuvdia_desc *d = nullptr;
     std::vector<Chunk> cn, ct;
+    std::vector<Unit> un, us;
     try {
         d = new cuvdia_desc();
         d->offsets.assign(offsets_host, offsets_host + nd);
         cn = plan_chunks(offsets_host, nd, false);
         ct = plan_chunks(offsets_host, nd, true);
+        un = plan_units(cn);
+        for (int c = 0; c < (int)cn.size(); ++c) us.push_back(Unit{c, -1});
     } catch (const std::bad_alloc &) {
         delete d;
         return CUVDIA_ENOMEM;
@@ -153,13 +156,16 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     d->dev_block = nullptr;
     if ((e = hipGetDevice(&d->device)) != hipSuccess) { delete d; return hip_fail(e, "hipGetDevice"); }
 
-    // one device block: offsets (padded to 64 B) | chunks_n | chunks_t
+    // one device block: offsets (padded to 64 B) | chunks_n | chunks_t | units | one unit per chunk
     const size_t off_bytes = ((size_t)nd * sizeof(int) + 63) / 64 * 64;
     const size_t cn_bytes = cn.size() * sizeof(Chunk), ct_bytes = ct.size() * sizeof(Chunk);
-    std::vector<unsigned char> staging(off_bytes + cn_bytes + ct_bytes, 0);
+    const size_t un_bytes = un.size() * sizeof(Unit), us_bytes = us.size() * sizeof(Unit);
+    std::vector<unsigned char> staging(off_bytes + cn_bytes + ct_bytes + un_bytes + us_bytes, 0);
     std::memcpy(staging.data(), offsets_host, (size_t)nd * sizeof(int));
     std::memcpy(staging.data() + off_bytes, cn.data(), cn_bytes);
     std::memcpy(staging.data() + off_bytes + cn_bytes, ct.data(), ct_bytes);
+    std::memcpy(staging.data() + off_bytes + cn_bytes + ct_bytes, un.data(), un_bytes);
+    std::memcpy(staging.data() + off_bytes + cn_bytes + ct_bytes + un_bytes, us.data(), us_bytes);
     if ((e = hipMalloc(&d->dev_block, staging.size())) != hipSuccess) {
         delete d;
         return e == hipErrorOutOfMemory ? CUVDIA_ENOMEM : hip_fail(e, "hipMalloc(descriptor)");
@@ -174,7 +180,9 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
                       reinterpret_cast<const int *>(base),
                       reinterpret_cast<const Chunk *>(base + off_bytes), d->n_chunks_n,
                       reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t,
-                      0, 0, 0, 0, 0, 0};
+                      0, 0, 0, 0, 0, 0,
+                      reinterpret_cast<const Unit *>(base + off_bytes + cn_bytes + ct_bytes), (int)un.size(),
+                      reinterpret_cast<const Unit *>(base + off_bytes + cn_bytes + ct_bytes + un_bytes)};
     auto span = [](const std::vector<Chunk> &t, int &max_len, int &s_min, int &s_max) {
         max_len = 0;
         s_min = t.empty() ? 0 : t.front().s0;

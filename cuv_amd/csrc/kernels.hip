@@ -14,9 +14,11 @@
 //           acc = fma(a, x, acc); then dst = beta*dst + alpha*acc
 //           (dst = alpha*acc when beta == 0, dst never read).
 //           The generic kernel walks the offset table in table order instead.
-//   dd2dia  four partial sums, wave q of the workgroup owning batch columns
-//           {4*g + i : g = q (mod 4), i < 4} in ascending order, each
-//           acc = fma(a, b, acc); total = ((p0 + p1) + p2) + p3;
+//   dd2dia  a single chunk: four partial sums, wave q of the workgroup owning
+//           batch columns {4*g + i : g = q (mod 4), i < 4} in ascending order,
+//           each acc = fma(a, b, acc); total = ((p0 + p1) + p2) + p3.
+//           A chunk pair: eight sums s_q over g = q (mod 8);
+//           p_q = s_q + s_{q+4}, then total as above.
 //           C = beta*C + alpha*total.  The generic kernel sums the batch
 //           serially in ascending column order.
 #include <hip/hip_runtime.h>
@@ -549,105 +551,130 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
 
 // ------------------------------------------------------------ tiled dd2dia --
 //
-// Workgroup = 256 rows of ONE run chunk, WAVES (4 or 8) waves.  Lane l owns
-// rows row0 + 4l .. 4l+3 and 4 x LC partial sums (LC = the longest chunk of
-// the table; positions past a chunk's own length are computed and dropped).
-// Wave q walks the batch-column groups g = q, q + WAVES, ... (4 columns per
-// group).  Per group the wave
-//   1. writes the group's rows [row0 + s0, row0 + s0 + 264) of B, which it
-//      fetched one step earlier with lanes along rows (4 + 1 dword buffer
-//      loads per column; rows outside B read as 0 through the buffer range
-//      check), to its private LDS buffer -- no workgroup barrier in the loop;
-//   2. requests the next group's rows of B and its own 4 rows x 4 columns of
-//      A (one 16-byte load per column when A allows it) -- columns past the
+// Workgroup = 256 rows of ONE unit: a run chunk, or two chunks whose first
+// shifts differ by delta (a multiple of 4, at most 128) -- e.g. two rows of a
+// 2-d window.  Lane l owns rows row0 + 4l .. 4l+3 and 4 x LC partial sums per
+// chunk (LC = the longest chunk of the table; positions past a chunk's own
+// length are computed and dropped).  A single chunk is worked by 4 waves, a
+// pair by 8; wave q walks the batch-column groups g = q, q + WAVES, ...
+// (4 columns per group).  Per group and column the wave
+//   1. writes the column's rows [row0 + s0, row0 + s0 + 264 + delta) of B,
+//      fetched one step earlier with lanes along rows (dword buffer loads;
+//      rows outside B read as 0 through the buffer range check), to its
+//      private LDS buffer -- no workgroup barrier in the loop;
+//   2. reads its 4 + LC - 1 wide window of B per chunk from LDS with 16-byte
+//      reads (the second chunk's window starts delta rows further);
+//   3. requests the same column of the next group: its rows of B and its own
+//      4 rows of A (one 16-byte load when A allows it).  Columns past the
 //      batch go through an empty buffer resource and come back as zeros
 //      without touching memory, so the loop body never branches and every
 //      wait counts exactly;
-//   3. reads, per column, its 4 + LC - 1 wide window of B from LDS with
-//      16-byte reads and issues 4 x LC FMAs.
-// At the end the waves' partial sums meet in LDS and are added in wave order;
-// the result is written with lanes along rows (the values of C that beta
-// scales were fetched at kernel start).
+//   4. issues 4 x LC FMAs per chunk.  A pair needs A once and the two bands of
+//      B overlap, so it moves about 40 % fewer bytes per FMA than two singles.
+// At the end the waves' partial sums meet in LDS and are added in a fixed
+// order; the result is written with lanes along rows (the values of C that
+// beta scales were fetched at kernel start).
 
 constexpr int DD_ROWS = 256;
 constexpr int DD_BG = 4;           // batch columns per step
 
-constexpr int DD_PITCH = 264;         // 256 + CHUNK_MAX staged rows of B per column
+template <int NCH>
+struct DdShape {
+    static constexpr int NQ = NCH == 1 ? 4 : 6;                 // 64-row loads per column
+    static constexpr int PITCH = 64 * NQ + 8;                   // staged rows per column: 264 or 392
+    static constexpr int WAVES = NCH == 1 ? 4 : 8;
+    static constexpr int WAVE_FLOATS = 2 * DD_BG * PITCH + 4;   // two buffers + a slot idle lanes write to
+    static constexpr int STAGE_FLOATS = WAVES * WAVE_FLOATS;
+};
+static_assert(DdShape<2>::PITCH >= DD_ROWS + PAIR_MAX_DELTA + CHUNK_MAX, "a pair's band must fit its buffer");
 
-constexpr int DD_WAVE_FLOATS = 2 * DD_BG * DD_PITCH + 4;   // two buffers + a slot idle lanes write to
-
+template <int NCH>
 struct DdStage {
-    float b[DD_BG * 4 + 1];        // B: 4 x 64 rows per column, + 8 halo rows x 4 columns in one load
-    float a[DD_BG][4];             // A: this lane's 4 rows of each column
+    float b[DD_BG * DdShape<NCH>::NQ + 1];   // B: NQ x 64 rows per column, + the last 8 rows of all 4 columns in one load
+    float a[DD_BG][4];                        // A: this lane's 4 rows of each column
 };
 
-template <int LC, int WAVES, bool AVEC>
-__global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
-    const Chunk *__restrict__ chunks, int nchunks, float *__restrict__ C, int stride,
+template <int LC, int NCH>
+constexpr int dd_red_floats() { return 4 * 4 * (NCH * LC * 64 + 8); }
+template <int LC, int NCH>
+constexpr int dd_lds_floats()
+{
+    return DdShape<NCH>::STAGE_FLOATS > dd_red_floats<LC, NCH>() ? DdShape<NCH>::STAGE_FLOATS : dd_red_floats<LC, NCH>();
+}
+
+template <int LC, int NCH, bool AVEC>
+__device__ __forceinline__ void dd2dia_unit(
+    float *lds, int row0, const Chunk *ck1, const Chunk *ck2, float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
     int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
     unsigned c_bytes)
 {
+    typedef DdShape<NCH> S;
+    constexpr int NQ = S::NQ, PITCH = S::PITCH, WAVES = S::WAVES;
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
-    constexpr int RED_T = LC * 64 + 8;              // floats between the 4 rows a lane owns: keeps the
+    constexpr int RED_T = NCH * LC * 64 + 8;        // floats between the 4 rows a lane owns: keeps the
                                                     // row-major read below free of bank conflicts
     constexpr int RED_WAVE = 4 * RED_T;
-    constexpr int STAGE_FLOATS = WAVES * DD_WAVE_FLOATS;
-    constexpr int LDS_FLOATS = STAGE_FLOATS > WAVES * RED_WAVE ? STAGE_FLOATS : WAVES * RED_WAVE;
-    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int rowtile = tile / nchunks;
-    const sc_chunk_ptr ck = scalar_ptr(chunks) + (tile - rowtile * nchunks);
-    const int row0 = rowtile * DD_ROWS;
-    // the whole table entry in three 16-byte scalar loads
+    // each table entry in three 16-byte scalar loads
     typedef int int4v __attribute__((ext_vector_type(4)));
     typedef const int4v __attribute__((address_space(4))) *sc_int4_ptr;
-    const int4v e0 = ((sc_int4_ptr)ck)[0], e1 = ((sc_int4_ptr)ck)[1], e2 = ((sc_int4_ptr)ck)[2];
-    const int s0 = e0.x;
-    const int slots[CHUNK_MAX] = {e0.z, e0.w, e1.x, e1.y, e1.z, e1.w, e2.x, e2.y};
-    const int base = row0 + s0;                     // first staged row of B
+    int s0[NCH], slots[NCH][CHUNK_MAX];
+#pragma unroll
+    for (int n = 0; n < NCH; ++n) {
+        const sc_int4_ptr e = (sc_int4_ptr)(n == 0 ? ck1 : ck2);
+        const int4v e0 = e[0], e1 = e[1], e2 = e[2];
+        s0[n] = e0.x;
+        slots[n][0] = e0.z; slots[n][1] = e0.w; slots[n][2] = e1.x; slots[n][3] = e1.y;
+        slots[n][4] = e1.z; slots[n][5] = e1.w; slots[n][6] = e2.x; slots[n][7] = e2.y;
+    }
+    const int delta = NCH == 2 ? s0[NCH - 1] - s0[0] : 0;      // rows between the two windows
+    const int need = DD_ROWS + delta + CHUNK_MAX;               // staged rows that are ever read
+    const int base = row0 + s0[0];                              // first staged row of B
     const int myrow = row0 + 4 * lane;
 
     // C values this lane will combine at the end: row row0 + 64*wave + lane of
-    // every diagonal of the chunk (waves 0..3; a workgroup of 8 waves leaves
-    // the output to its first four).  Byte offset of that slot, or the
-    // out-of-range marker where no matrix element sits.
-    auto c_offset = [&](int j) -> unsigned {
-        const int sl = slots[j];
+    // every diagonal of the unit (waves 0..3; a pair's waves 4..7 leave the
+    // output to them).  Byte offset of that slot, or the out-of-range marker
+    // where no matrix element sits.
+    auto c_offset = [&](int n, int j) -> unsigned {
+        const int sl = slots[n][j];
         const int o = row0 + 64 * wave + lane;
-        const int in = o + s0 + j;
+        const int in = o + s0[n] + j;
         const bool ok = (wave < 4) & (sl >= 0) & (o < h) & (in >= 0) & (in < w);
         return ok ? ((unsigned)sl * (unsigned)stride + (unsigned)o) * 4u : OOB_OFFSET;
     };
-    float cpre[LC];
+    float cpre[NCH][LC];
     {
         // beta == 0: C is not read (an empty resource returns zeros without touching memory)
         const __amdgpu_buffer_rsrc_t cr = make_rsrc(C, beta != 0.f ? c_bytes : 0u);
 #pragma unroll
-        for (int j = 0; j < LC; ++j) cpre[j] = buffer_load_f32(cr, c_offset(j));
+        for (int n = 0; n < NCH; ++n)
+#pragma unroll
+            for (int j = 0; j < LC; ++j) cpre[n][j] = buffer_load_f32(cr, c_offset(n, j));
     }
 
-    // per-lane byte offsets inside one column; out-of-range rows use the marker
-    unsigned b_off[5];
+    // per-lane byte offsets inside one column; rows outside B, and staged rows
+    // no window reaches, use the out-of-range marker
+    unsigned b_off[NQ + 1];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const int r = base + q * 64 + lane;
-        b_off[q] = (r >= 0 && r < w) ? (unsigned)r * 4u : OOB_OFFSET;
+    for (int q = 0; q < NQ; ++q) {
+        const int rr = q * 64 + lane, r = base + rr;
+        b_off[q] = (rr < need && r >= 0 && r < w) ? (unsigned)r * 4u : OOB_OFFSET;
     }
-    // the 8 rows past the 256 (the halo) of all 4 columns travel in one load:
-    // lane = 8 * column + row
+    // the last 8 staged rows of all 4 columns travel in one load: lane = 8 * column + row
     const int hb = lane >> 3;
     {
-        const int r = base + DD_ROWS + (lane & 7);
-        b_off[4] = (hb < DD_BG && r >= 0 && r < w) ? ((unsigned)r + (unsigned)hb * (unsigned)ldb) * 4u : OOB_OFFSET;
+        const int rr = 64 * NQ + (lane & 7), r = base + rr;
+        b_off[NQ] = (hb < DD_BG && rr < need && r >= 0 && r < w)
+                        ? ((unsigned)r + (unsigned)hb * (unsigned)ldb) * 4u : OOB_OFFSET;
     }
     // where that load lands in buffer 0 / buffer 1 of this wave (idle lanes: the spare slot)
-    const int halo_at0 = hb < DD_BG ? hb * DD_PITCH + DD_ROWS + (lane & 7) : 2 * DD_BG * DD_PITCH;
-    const int halo_at1 = hb < DD_BG ? halo_at0 + DD_BG * DD_PITCH : 2 * DD_BG * DD_PITCH;
+    const int halo_at0 = hb < DD_BG ? hb * PITCH + 64 * NQ + (lane & 7) : 2 * DD_BG * PITCH;
+    const int halo_at1 = hb < DD_BG ? halo_at0 + DD_BG * PITCH : 2 * DD_BG * PITCH;
     unsigned a_off[4];
     if (AVEC) {
         a_off[0] = (myrow + 3 < h) ? (unsigned)myrow * 4u : OOB_OFFSET;
@@ -655,30 +682,39 @@ __global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
 #pragma unroll
         for (int t = 0; t < 4; ++t) a_off[t] = (myrow + t < h) ? (unsigned)(myrow + t) * 4u : OOB_OFFSET;
     }
-    const unsigned lda4 = (unsigned)lda * 4u, ldb4 = (unsigned)ldb * 4u;
+    // Column strides in bytes, pinned to scalar registers: they feed the loads'
+    // scalar offsets, and left alone the compiler derives them from a vector
+    // copy of ldb and then has to loop over lanes to issue each load.
+    unsigned lda4, ldb4;
+    asm("v_readfirstlane_b32 %0, %1" : "=s"(lda4) : "v"((unsigned)lda * 4u));
+    asm("v_readfirstlane_b32 %0, %1" : "=s"(ldb4) : "v"((unsigned)ldb * 4u));
 
-    float acc[4][LC];
+    float acc[NCH][4][LC];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int n = 0; n < NCH; ++n)
 #pragma unroll
-        for (int j = 0; j < LC; ++j) acc[t][j] = 0.f;
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int j = 0; j < LC; ++j) acc[n][t][j] = 0.f;
 
-    float *mybuf = lds + wave * DD_WAVE_FLOATS;
+    const int ngroups = (batch + DD_BG - 1) / DD_BG;
+    const int steps = (ngroups + WAVES - 1) / WAVES;        // same for every wave
+    float *mybuf = lds + wave * S::WAVE_FLOATS;
     const __amdgpu_buffer_rsrc_t b_all = make_rsrc(B, b_bytes);
 
     // requests column i of group g: B rows into st.b, A rows into st.a (the
-    // halo load, which serves all 4 columns, travels with column 0)
-    auto issue_col = [&](int g, int i, DdStage &st) {
-        const int b0 = g * DD_BG;
+    // load of the last 8 rows, which serves all 4 columns, travels with column 0)
+    auto issue_col = [&](int g, int i, DdStage<NCH> &st) {
+        const int b0 = __builtin_amdgcn_readfirstlane(g * DD_BG);   // wave-uniform: keeps column offsets scalar
         const bool live = b0 + i < batch;
         const __amdgpu_buffer_rsrc_t br = make_rsrc(B, live ? b_bytes : 0u);
         const unsigned colb = (unsigned)(b0 + i) * ldb4;
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-            st.b[i * 4 + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, b_off[q], colb, 0));
+        for (int q = 0; q < NQ; ++q)
+            st.b[i * NQ + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, b_off[q], colb, 0));
         if (i == 0)
-            st.b[DD_BG * 4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                b_all, (b0 + hb < batch) ? b_off[4] : OOB_OFFSET, (unsigned)b0 * ldb4, 0));
+            st.b[DD_BG * NQ] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                b_all, (b0 + hb < batch) ? b_off[NQ] : OOB_OFFSET, (unsigned)b0 * ldb4, 0));
         const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, live ? a_bytes : 0u);
         const unsigned cola = (unsigned)(b0 + i) * lda4;
         if (AVEC) {
@@ -690,59 +726,63 @@ __global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
                 st.a[i][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, a_off[t], cola, 0));
         }
     };
-    auto issue = [&](int g, DdStage &st) {
+    auto issue = [&](int g, DdStage<NCH> &st) {
 #pragma unroll
         for (int i = 0; i < DD_BG; ++i) issue_col(g, i, st);
     };
-    auto commit_col = [&](const DdStage &st, int par, int i) {
-        float *buf = mybuf + par * (DD_BG * DD_PITCH);
+    auto commit_col = [&](const DdStage<NCH> &st, int par, int i) {
+        float *buf = mybuf + par * (DD_BG * PITCH);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) buf[i * DD_PITCH + q * 64 + lane] = st.b[i * 4 + q];
-        if (i == 0) mybuf[par ? halo_at1 : halo_at0] = st.b[DD_BG * 4];
+        for (int q = 0; q < NQ; ++q) buf[i * PITCH + q * 64 + lane] = st.b[i * NQ + q];
+        if (i == 0) mybuf[par ? halo_at1 : halo_at0] = st.b[DD_BG * NQ];
         wave_lds_fence();
     };
-    auto read_window = [&](float (&win)[WQ * 4], const float *buf, int i) {
-        const float4 *p4 = reinterpret_cast<const float4 *>(buf + i * DD_PITCH + 4 * lane);
+    struct Windows { float w[NCH][WQ * 4]; };
+    auto read_windows = [&](Windows &win, const float *buf, int i) {
 #pragma unroll
-        for (int q = 0; q < WQ; ++q) {
-            const float4 v = p4[q];
-            win[4 * q + 0] = v.x; win[4 * q + 1] = v.y; win[4 * q + 2] = v.z; win[4 * q + 3] = v.w;
+        for (int n = 0; n < NCH; ++n) {
+            const float4 *p4 = reinterpret_cast<const float4 *>(buf + i * PITCH + 4 * lane + (n ? delta : 0));
+#pragma unroll
+            for (int q = 0; q < WQ; ++q) {
+                const float4 v = p4[q];
+                win.w[n][4 * q + 0] = v.x; win.w[n][4 * q + 1] = v.y; win.w[n][4 * q + 2] = v.z; win.w[n][4 * q + 3] = v.w;
+            }
         }
     };
-    auto fmas = [&](const float (&a)[4], const float (&win)[WQ * 4]) {
+    auto fmas = [&](const float (&a)[4], const Windows &win) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int n = 0; n < NCH; ++n)
 #pragma unroll
-            for (int j = 0; j < LC; ++j) acc[t][j] = __builtin_fmaf(a[t], win[t + j], acc[t][j]);
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int j = 0; j < LC; ++j) acc[n][t][j] = __builtin_fmaf(a[t], win.w[n][t + j], acc[n][t][j]);
     };
     // Step k works on group wave + WAVES*k out of stage set k & 1 and LDS
     // buffer k & 1, one column at a time: column i's rows of B go to LDS and
-    // its window is read back while the FMAs of column i - 1 run; column i of
-    // the next group is requested right after, so every load has one whole
-    // step to arrive and the requests are spread between the FMA blocks -- a
-    // wave that has to wait for room in the memory pipeline leaves the SIMD
-    // to the other wave's FMAs instead of holding its own back.  Past the last
-    // group the requests hit the empty resource.
-    auto step = [&](int k, int par, DdStage &cur, DdStage &nxt) {
-        const float *buf = mybuf + par * (DD_BG * DD_PITCH);
+    // its windows are read back while the FMAs of column i - 1 run; column i
+    // of the next group is requested right after, so every load has one whole
+    // step to arrive and the requests are spread between the FMA blocks.  Past
+    // the last group the requests hit the empty resource.
+    auto step = [&](int k, int par, DdStage<NCH> &cur, DdStage<NCH> &nxt) {
+        const float *buf = mybuf + par * (DD_BG * PITCH);
         const int gn = wave + WAVES * (k + 1);
-        float w0[WQ * 4], w1[WQ * 4];
+        Windows w0, w1;
         commit_col(cur, par, 0);
-        read_window(w0, buf, 0);
+        read_windows(w0, buf, 0);
         commit_col(cur, par, 1);
-        read_window(w1, buf, 1);
+        read_windows(w1, buf, 1);
         issue_col(gn, 0, nxt);
         __builtin_amdgcn_sched_barrier(0);
         fmas(cur.a[0], w0);
         __builtin_amdgcn_sched_barrier(0);
         commit_col(cur, par, 2);
-        read_window(w0, buf, 2);
+        read_windows(w0, buf, 2);
         issue_col(gn, 1, nxt);
         __builtin_amdgcn_sched_barrier(0);
         fmas(cur.a[1], w1);
         __builtin_amdgcn_sched_barrier(0);
         commit_col(cur, par, 3);
-        read_window(w1, buf, 3);
+        read_windows(w1, buf, 3);
         issue_col(gn, 2, nxt);
         __builtin_amdgcn_sched_barrier(0);
         fmas(cur.a[2], w0);
@@ -753,9 +793,7 @@ __global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    const int ngroups = (batch + DD_BG - 1) / DD_BG;
-    const int steps = (ngroups + WAVES - 1) / WAVES;        // same for every wave
-    DdStage st0, st1;
+    DdStage<NCH> st0, st1;
     issue(wave, st0);
     int k = 0;
     for (; k + 1 < steps; k += 2) {
@@ -764,29 +802,87 @@ __global__ __launch_bounds__(64 * WAVES) void dd2dia_tiled_kernel(
     }
     if (k < steps) step(k, 0, st0, st1);
 
-    // combine the waves' partial sums in wave order
+    // Combine the waves' partial sums.  8 waves: wave q + 4 hands its sums to
+    // wave q first (same lanes, same layout); then the four sums meet in wave
+    // order: total = ((p0 + p1) + p2) + p3 with p_q = s_q (+ s_{q+4}).
     __syncthreads();
-    float *red = lds;                               // [wave][t][j][64 lanes], t blocks RED_T apart
+    float *red = lds;                               // [wave][t][n][j][64 lanes], t blocks RED_T apart
+    if (WAVES == 8) {
+        if (wave >= 4) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+            for (int n = 0; n < NCH; ++n)
 #pragma unroll
-        for (int j = 0; j < LC; ++j)
-            red[wave * RED_WAVE + t * RED_T + j * 64 + lane] = acc[t][j];
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int j = 0; j < LC; ++j)
+                        red[(wave - 4) * RED_WAVE + t * RED_T + (n * LC + j) * 64 + lane] = acc[n][t][j];
+        }
+        __syncthreads();
+        if (wave >= 4) return;
+#pragma unroll
+        for (int n = 0; n < NCH; ++n)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int j = 0; j < LC; ++j)
+                    acc[n][t][j] += red[wave * RED_WAVE + t * RED_T + (n * LC + j) * 64 + lane];
+        // no barrier needed here: below, wave q overwrites only the block it has just read
+    }
+#pragma unroll
+    for (int n = 0; n < NCH; ++n)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int j = 0; j < LC; ++j)
+                red[wave * RED_WAVE + t * RED_T + (n * LC + j) * 64 + lane] = acc[n][t][j];
     __syncthreads();
-    if (wave < 4) {
+    {
         const int r = 64 * wave + lane;             // row within the tile: lane r/4 owned it as its row r%4
         const float *src = red + (r & 3) * RED_T + (r >> 2);
 #pragma unroll
-        for (int j = 0; j < LC; ++j) {
-            float total = src[j * 64];
+        for (int n = 0; n < NCH; ++n)
 #pragma unroll
-            for (int p = 1; p < WAVES; ++p) total += src[p * RED_WAVE + j * 64];
-            const unsigned off = c_offset(j);
-            if (off != OOB_OFFSET) {
-                float *cd = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
-                *cd = (beta == 0.f) ? alpha * total : beta * cpre[j] + alpha * total;
+            for (int j = 0; j < LC; ++j) {
+                float total = src[(n * LC + j) * 64];
+#pragma unroll
+                for (int p = 1; p < 4; ++p) total += src[p * RED_WAVE + (n * LC + j) * 64];
+                const unsigned off = c_offset(n, j);
+                if (off != OOB_OFFSET) {
+                    float *cd = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
+                    *cd = (beta == 0.f) ? alpha * total : beta * cpre[n][j] + alpha * total;
+                }
             }
-        }
+    }
+}
+
+// PAIRS = false: every unit is a single chunk, 4 waves per workgroup.
+// PAIRS = true: 8 waves per workgroup; a workgroup whose unit is a single
+// chunk retires its upper four waves at once.
+template <int LC, bool AVEC, bool PAIRS>
+__global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
+    const Chunk *__restrict__ chunks, const Unit *__restrict__ units, int nunits,
+    float *__restrict__ C, int stride,
+    const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
+    int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
+    unsigned c_bytes)
+{
+    constexpr int LDS_FLOATS = PAIRS ? (dd_lds_floats<LC, 2>() > dd_lds_floats<LC, 1>() ? dd_lds_floats<LC, 2>()
+                                                                                         : dd_lds_floats<LC, 1>())
+                                     : dd_lds_floats<LC, 1>();
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+    const int tile = xcd_tile(blockIdx.x, gridDim.x);
+    const int rowtile = tile / nunits;
+    typedef const Unit __attribute__((address_space(4))) *sc_unit_ptr;
+    const sc_unit_ptr u = (sc_unit_ptr)units + (tile - rowtile * nunits);
+    const int c1 = u->c1, c2 = u->c2;
+    const int row0 = rowtile * DD_ROWS;
+    if (PAIRS && c2 >= 0) {
+        dd2dia_unit<LC, 2, AVEC>(lds, row0, chunks + c1, chunks + c2, C, stride, A, lda, B, ldb, h, w, batch,
+                                 alpha, beta, a_bytes, b_bytes, c_bytes);
+    } else {
+        if (PAIRS && threadIdx.x >= 256) return;
+        dd2dia_unit<LC, 1, AVEC>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
+                                 alpha, beta, a_bytes, b_bytes, c_bytes);
     }
 }
 
@@ -890,15 +986,15 @@ bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch)
            b_bytes < (long long)OOB_OFFSET && c_bytes < (long long)OOB_OFFSET;
 }
 
-int g_dd2dia_waves = 4;
+// 0: pair chunks where the plan allows it; 1: every chunk on its own (tests
+// and measurements of the unpaired kernel)
+int g_dd2dia_no_pairs = 0;
 
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream)
 {
     const long long row_tiles = (C.h + DD_ROWS - 1) / DD_ROWS;
-    const long long blocks = row_tiles * C.n_chunks_n;
-    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     // 16-byte loads of A need an aligned base and leading dimension and whole
     // groups of 4 rows; row tiles start at multiples of 256 and lanes at
     // multiples of 4 rows.
@@ -906,18 +1002,25 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     const unsigned a_bytes = batch > 0 ? (unsigned)((((long long)batch - 1) * lda + C.h) * 4) : 0u;
     const unsigned b_bytes = batch > 0 ? (unsigned)((((long long)batch - 1) * ldb + C.w) * 4) : 0u;
     const unsigned c_bytes = (unsigned)((long long)C.nd * C.stride * 4);
+    // without pairs the units are the chunks themselves, in table order
+    // (pairs only with 16-byte loads of A: the dword-load variant of the pair
+    // body needs more registers than a wave has)
+    const bool use_units = C.n_units < C.n_chunks_n && a_vec && !g_dd2dia_no_pairs;
+    const bool pairs = use_units;
+    const Unit *units = use_units ? C.units_dev : C.single_units_dev;
+    const int nunits = use_units ? C.n_units : C.n_chunks_n;
+    const long long blocks = row_tiles * nunits;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks);
-    const int waves = g_dd2dia_waves;
-#define CUVDIA_DD_ARGS C.chunks_n_dev, C.n_chunks_n, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
+#define CUVDIA_DD_ARGS C.chunks_n_dev, units, nunits, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
                        a_bytes, b_bytes, c_bytes
 #define CUVDIA_DD_LAUNCH(L)                                                                              \
     case L:                                                                                              \
-        if (waves == 8) {                                                                                \
-            if (a_vec) hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 8, true>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
-            else hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 8, false>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);       \
+        if (pairs) {                                                                                     \
+            hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, true>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
         } else {                                                                                         \
-            if (a_vec) hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 4, true>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);  \
-            else hipLaunchKernelGGL((dd2dia_tiled_kernel<L, 4, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);       \
+            if (a_vec) hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);  \
+            else hipLaunchKernelGGL((dd2dia_tiled_kernel<L, false, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);       \
         }                                                                                                \
         break;
     switch (C.max_len_n) {

@@ -18,6 +18,9 @@ struct DiaView {
     int max_len_n, max_len_t;    // longest chunk of each table
     int s_min_n, s_max_n;        // smallest / largest chunk shift of each table
     int s_min_t, s_max_t;
+    const Unit *units_dev;       // units of the normal table (dense x dense^T projection)
+    int n_units;
+    const Unit *single_units_dev;   // one unit per chunk of the normal table, in table order
 };
 
 // dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch

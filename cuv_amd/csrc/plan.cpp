@@ -37,6 +37,26 @@ std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed)
     return out;
 }
 
+std::vector<Unit> plan_units(const std::vector<Chunk> &chunks)
+{
+    std::vector<Unit> out;
+    const int n = (int)chunks.size();
+    int c = 0;
+    while (c < n) {
+        if (c + 1 < n) {
+            const long long delta = (long long)chunks[c + 1].s0 - chunks[c].s0;
+            if (delta > 0 && delta <= PAIR_MAX_DELTA && delta % 4 == 0) {
+                out.push_back(Unit{c, c + 1});
+                c += 2;
+                continue;
+            }
+        }
+        out.push_back(Unit{c, -1});
+        c += 1;
+    }
+    return out;
+}
+
 long long count_valid(const int *offsets, int nd, int h, int w, int rf)
 {
     long long total = 0;

@@ -28,6 +28,19 @@ static_assert(sizeof(Chunk) == 48, "Chunk layout is part of the device table");
 // length carry slot -1.
 std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed);
 
+// A unit of work of the tiled dense x dense^T projection: one chunk, or two
+// chunks of the normal table whose first shifts differ by a multiple of 4 of
+// at most PAIR_MAX_DELTA rows.  A wave serves both chunks of a pair from one
+// staged band of the second operand and one copy of the first operand's rows.
+constexpr int PAIR_MAX_DELTA = 128;
+struct Unit {
+    int c1;                 // chunk index
+    int c2;                 // second chunk index, or -1
+};
+// Greedy over the table in shift order: chunk c pairs with c + 1 when their
+// shifts allow it.
+std::vector<Unit> plan_units(const std::vector<Chunk> &chunks);
+
 // Number of matrix elements stored (slots the reference host loops touch):
 // sum over diagonals of min(h - rf*max(0,-k), rf*(w - max(0,k))), clamped at 0
 // (src/cuv/matrix_ops/spmv.cu:183-189).

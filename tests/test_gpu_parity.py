@@ -104,6 +104,11 @@ SHAPES = [
     (130, 130, [1], 1, 1),
     (64, 64, [0], 1, 64),
     (700, 650, [d * 25 + e for d in range(-2, 3) for e in range(-2, 3)], 1, 96),
+    # chunk pairs of the dense x dense^T projection (first shifts a multiple of 4, at most 128, apart)
+    (512, 512, [dy * 128 + dx for dy in range(-1, 2) for dx in range(-3, 4)], 1, 40),
+    (300, 300, list(range(-8, -1)) + list(range(0, 8)) + [100, 101], 1, 7),
+    (260, 1000, [-200, -199, -198, -72, -71, 56, 57, 58, 59, 700], 1, 131),
+    (1024, 768, [dy * 64 + dx for dy in range(-2, 3) for dx in range(0, 8)], 1, 1),
 ]
 
 
