@@ -54,9 +54,71 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--workload", default="step",
+                    help="'step' (default): cfg1 + cfg2 + cfg3, the configuration the metric is quoted on; "
+                         "'cfg4': the large layer (262144 rows, 676 diagonals, batch 256), each product timed "
+                         "on its own -- an auxiliary line, no CPU leg (the oracle needs minutes for it)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
     return ap.parse_args()
+
+
+def bench_cfg4(args, torch, D, W, dev):
+    """The large layer: 256x256 map, 4 channels, 13x13 window per channel pair (676 diagonals), batch 256,
+    inputs drawn on the device.  The working set (about 1.8 GB) is far beyond every cache, so no buffer
+    rotation is needed.  Parity at this size is covered by tests/test_gpu_parity.py."""
+    import numpy as np
+    p = W.pattern_large(256, 4, 13)
+    n, nd, batch = p.h, len(p.offsets), 256
+    g = torch.Generator(device=dev)
+    g.manual_seed(0xC0FFEE + 4)
+    nnz = p.nnz
+
+    def dia():
+        m = D.dev_dia_matrix_f(n, n, nd, n, 1, device=dev)
+        m.set_offsets(p.offsets)
+        m.vec.copy_(torch.randn(nd * n, generator=g, device=dev) * 0.01)
+        return m
+    A, G = dia(), dia()
+    X = torch.rand(batch, n, generator=g, device=dev)
+    H = torch.rand(batch, n, generator=g, device=dev)
+    Y = torch.empty(batch, n, device=dev)
+    bd = D.dev_block_descriptor_f(G)
+    A.desc
+    ops = {
+        "forward": (lambda: D.prod(Y, A, X, "n", "n", 1.0, 0.0, sync=False), W.spmm_bytes(p, batch, "n", 0.0)),
+        "transposed": (lambda: D.prod(Y, A, H, "t", "n", 1.0, 0.0, sync=False), W.spmm_bytes(p, batch, "t", 0.0)),
+        "weight_gradient": (lambda: D.densedense_to_dia(G, bd, X, H, 1.0 / batch, 0.0, sync=False),
+                            W.dd2dia_bytes(p, batch, 0.0)),
+    }
+    flops = 2 * nnz * batch
+    steps = min(args.steps, 50)
+    res = {}
+    stream = torch.cuda.current_stream()
+    for name, (fn, nbytes) in ops.items():
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        res[name] = dict(ms=ms, bytes=nbytes, flops=flops, gbs=nbytes / (ms * 1e-3) / 1e9,
+                         frac_hbm=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, tflops=flops / (ms * 1e-3) / 1e12,
+                         frac_fp32_valu=flops / (ms * 1e-3) / 1e12 / FP32_VALU_PEAK_TFLOPS)
+    tot_ms = sum(r["ms"] for r in res.values())
+    tot_bytes = sum(r["bytes"] for r in res.values())
+    print(json.dumps(dict(
+        metric="achieved HBM GB/s, DIA SpMM (both transposes) + densedense_to_dia, large layer", unit="GB/s",
+        value=tot_bytes / (tot_ms * 1e-3) / 1e9, n_gpus=1, steps=steps, warmup=3, ms_per_step=tot_ms,
+        higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
+        config=dict(workload="cfg4: 262144x262144 DIA, 676 diagonals (4 channels x 13x13 window on a 256x256 map), "
+                             "batch 256; forward, transposed and gradient products each timed alone",
+                    rows=n, diagonals=nd, batch=batch, nnz=nnz),
+        ops=res, note="bound by the fp32 vector rate (57 FLOP per algorithmic byte), not by HBM")))
 
 
 def main():
@@ -76,6 +138,9 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     L = _lib.lib()
+
+    if args.workload == "cfg4":
+        return bench_cfg4(args, torch, D, W, dev)
 
     w1, w2, w3 = W.cfg1(), W.cfg2(), W.cfg3()
     p = w1.pattern

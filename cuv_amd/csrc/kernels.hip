@@ -288,11 +288,12 @@ __device__ __forceinline__ float4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, un
 }
 constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used here
 
-// EDGE = false is the body for a tile whose staged rows all exist (every
-// chunk's 80 rows lie inside the dense operand and all 64 output rows exist):
-// row positions then enter the loads as a scalar offset, nothing is clamped
-// or shifted, and a chunk costs a couple of vector instructions besides its
-// FMAs.  EDGE = true handles the tiles at the operand's ends.
+// EDGE = false is the body for a tile all of whose 64 output rows exist and
+// none of whose chunks straddles an end of the dense operand (each chunk's 80
+// staged rows lie inside it, or wholly outside): row positions then enter the
+// loads as a scalar offset, nothing is clamped or shifted, and a chunk costs a
+// couple of vector instructions besides its FMAs.  EDGE = true handles the
+// tiles at the operand's ends.
 template <int LCK, int T, int NTAB, bool EDGE>
 __device__ __forceinline__ void spmm_tile(
     float (&lds)[2][SP_STAGE_FLOATS], int row0, int col0,
@@ -388,10 +389,12 @@ __device__ __forceinline__ void spmm_tile(
     auto issue = [&](const SpInfo<T> &info, SpStage<T> &st, int c) {
         const int s0 = info.s0;
         if constexpr (!EDGE) {
-            // past the table nothing is fetched: an empty resource returns zeros
-            const bool real = c < nchunks;
+            // past the table, and for a chunk whose rows lie outside the operand,
+            // nothing is fetched: an empty resource returns zeros
+            const int a0 = row0 + s0;
+            const bool real = (c < nchunks) & (a0 >= 0) & (a0 + 4 * SP_QUADS <= n_in);
             const __amdgpu_buffer_rsrc_t xq = make_rsrc(X + (long long)col0 * ldx, real ? x_bytes : 0u);
-            const unsigned soff = (unsigned)(row0 + s0) * 4u;
+            const unsigned soff = real ? (unsigned)a0 * 4u : 0u;
 #pragma unroll
             for (int it = 0; it < SP_LOADS; ++it)
                 st.x[it] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(xq, col_off[it], soff, 0));
@@ -539,9 +542,22 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     const int rowtile = tile / col_tiles;
     const int row0 = rowtile * SP_ROWS;
     const int col0 = (tile - rowtile * col_tiles) * SP_COLS;
-    // every chunk's staged rows [row0 + s0, row0 + s0 + 80) inside the operand, all 64 output rows real
-    const bool interior = (row0 + s_min >= 0) & (row0 + s_max + 4 * SP_QUADS <= n_in) & (row0 + SP_ROWS <= n_out);
-    if (interior)
+    // The lean body serves a tile all of whose 64 output rows exist and none of
+    // whose chunks straddles an end of the operand: each chunk's staged rows
+    // [row0 + s0, row0 + s0 + 80) lie either inside it or wholly outside (such
+    // a chunk contributes nothing and is skipped through an empty resource).
+    bool lean = row0 + SP_ROWS <= n_out;
+    if (!((row0 + s_min >= 0) & (row0 + s_max + 4 * SP_QUADS <= n_in))) {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int k = 0; k < NTAB; ++k) {
+            const int a0 = row0 + chunks[min(64 * k + lane, nchunks - 1)].s0;
+            const bool inside = (a0 >= 0) & (a0 + 4 * SP_QUADS <= n_in);
+            const bool outside = (a0 + 4 * SP_QUADS <= 0) | (a0 >= n_in);
+            lean &= __builtin_amdgcn_ballot_w64(!(inside | outside)) == 0;
+        }
+    }
+    if (lean)
         spmm_tile<LCK, T, NTAB, false>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                  n_out, n_in, batch, alpha, beta, a_bytes);
     else
