@@ -91,6 +91,8 @@ def bench_cfg4(args, torch, D, W, dev):
         "weight_gradient": (lambda: D.densedense_to_dia(G, bd, X, H, 1.0 / batch, 0.0, sync=False),
                             W.dd2dia_bytes(p, batch, 0.0)),
     }
+    avg = torch.empty(nd, device=dev)
+    aux_ops = {"avg_diagonals": (lambda: D.avg_diagonals(avg, A, sync=False), 4 * nnz + 8 * nd)}
     flops = 2 * nnz * batch
     steps = min(args.steps, 50)
     res = {}
@@ -111,6 +113,20 @@ def bench_cfg4(args, torch, D, W, dev):
                          frac_fp32_valu=flops / (ms * 1e-3) / 1e12 / FP32_VALU_PEAK_TFLOPS)
     tot_ms = sum(r["ms"] for r in res.values())
     tot_bytes = sum(r["bytes"] for r in res.values())
+    aux = {}
+    for name, (fn, nbytes) in aux_ops.items():
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        aux[name] = dict(ms=ms, bytes=nbytes, gbs=nbytes / (ms * 1e-3) / 1e9,
+                         frac_hbm=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
     print(json.dumps(dict(
         metric="achieved HBM GB/s, DIA SpMM (both transposes) + densedense_to_dia, large layer", unit="GB/s",
         value=tot_bytes / (tot_ms * 1e-3) / 1e9, n_gpus=1, steps=steps, warmup=3, ms_per_step=tot_ms,
@@ -118,7 +134,7 @@ def bench_cfg4(args, torch, D, W, dev):
         config=dict(workload="cfg4: 262144x262144 DIA, 676 diagonals (4 channels x 13x13 window on a 256x256 map), "
                              "batch 256; forward, transposed and gradient products each timed alone",
                     rows=n, diagonals=nd, batch=batch, nnz=nnz),
-        ops=res, note="bound by the fp32 vector rate (57 FLOP per algorithmic byte), not by HBM")))
+        ops=res, aux=aux, note="bound by the fp32 vector rate (57 FLOP per algorithmic byte), not by HBM")))
 
 
 def main():

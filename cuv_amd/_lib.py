@@ -49,6 +49,7 @@ def lib():
     L.cuvdia_desc_info.argtypes = [c_vp, ip, ip, ctypes.POINTER(c_ll)]
     L.cuvdia_spmm_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp]
     L.cuvdia_dd2dia_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_f, c_f, c_vp]
+    L.cuvdia_avg_diagonals_f32.argtypes = [c_vp, c_vp, c_vp, c_vp]
     L.cuvdia_spmm_offsets_f32.argtypes = [c_vp, ip, c_int, c_int, c_int, c_int, c_int, c_vp, c_ll,
                                           c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp]
     L.cuvdia_dd2dia_offsets_f32.argtypes = [c_vp, ip, c_int, c_int, c_int, c_int, c_int, c_vp, c_ll,

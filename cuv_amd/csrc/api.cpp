@@ -350,6 +350,14 @@ int cuvdia_cache_clear(void)
     return rc;
 }
 
+int cuvdia_avg_diagonals_f32(const cuvdia_desc *desc, const float *A_vals, float *dst, void *stream)
+{
+    if (!desc || !A_vals || !dst) return CUVDIA_EINVAL;
+    if (desc->rf != 1) return CUVDIA_EUNSUPPORTED;      // src/cuv/matrix_ops/diagonals.cu:28
+    const hipError_t e = launch_avg_diagonals(desc->view, A_vals, dst, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "avg_diagonals kernel launch");
+}
+
 int cuvdia_spmm_offsets_f32(const float *A_vals, const int *offsets_host, int nd, int stride,
                             int h, int w, int row_fact, const float *B, long long ldb,
                             float *dst, long long ldd, int batch, char transA,

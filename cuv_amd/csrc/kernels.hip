@@ -140,6 +140,44 @@ __global__ __launch_bounds__(256) void dd2dia_generic_kernel(
     *dst = (beta == 0.f) ? alpha * s : beta * (*dst) + alpha * s;
 }
 
+// Mean of every stored diagonal over its valid slots (row_fact == 1):
+// dst[d] = sum_{n < N_d} vals[d*stride + i_start + n] / N_d
+// (src/cuv/matrix_ops/diagonals.cu:24-51).  One workgroup of 1024 threads per
+// diagonal.  Summation order: thread t keeps 8 running sums, sum u taking the
+// elements n = 8192*k + 1024*u + t in ascending k; the thread adds them in
+// ascending u; the 1024 thread sums are folded in LDS, s[t] += s[t + w] for
+// w = 512, 256, .., 1.  A diagonal with no valid slot yields 0.
+constexpr int AVG_THREADS = 1024;
+__global__ __launch_bounds__(AVG_THREADS) void avg_diagonals_kernel(
+    const int *__restrict__ offsets, const float *__restrict__ vals, int stride, int h, int w,
+    float *__restrict__ dst)
+{
+    __shared__ float part[AVG_THREADS];
+    const int d = blockIdx.x, t = threadIdx.x;
+    const long long k = offsets[d];
+    const long long i_start = k < 0 ? -k : 0, j_start = k > 0 ? k : 0;
+    const long long N = min((long long)h - i_start, (long long)w - j_start);
+    const float *x = vals + (long long)d * stride + i_start;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (long long base = 0; base < N; base += 8 * AVG_THREADS) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const long long n = base + AVG_THREADS * u + t;
+            acc[u] += n < N ? x[n] : 0.f;
+        }
+    }
+    float sum = acc[0];
+#pragma unroll
+    for (int u = 1; u < 8; ++u) sum += acc[u];
+    part[t] = sum;
+    __syncthreads();
+    for (int wdt = AVG_THREADS / 2; wdt >= 1; wdt >>= 1) {
+        if (t < wdt) part[t] += part[t + wdt];
+        __syncthreads();
+    }
+    if (t == 0) dst[d] = N > 0 ? part[0] / (float)N : 0.f;
+}
+
 // -------------------------------------------------------------- tiled spmm --
 //
 // Workgroup = 64 output rows x 64 batch columns, 64 / T waves of T rows each
@@ -986,6 +1024,18 @@ hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, 
         hipLaunchKernelGGL(dd2dia_generic_kernel, dim3(gx, (unsigned)slab), dim3(256), 0, stream,
                            C.offsets_dev + done, vals + (long long)done * C.stride, C.stride,
                            C.h, C.w, C.rf, A, lda, B, ldb, batch, alpha, beta);
+        done += slab;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_avg_diagonals(const DiaView &A, const float *vals, float *dst, hipStream_t stream)
+{
+    int done = 0;
+    while (done < A.nd) {
+        const int slab = A.nd - done < 65535 ? A.nd - done : 65535;
+        hipLaunchKernelGGL(avg_diagonals_kernel, dim3((unsigned)slab), dim3(AVG_THREADS), 0, stream,
+                           A.offsets_dev + done, vals + (long long)done * A.stride, A.stride, A.h, A.w, dst + done);
         done += slab;
     }
     return hipGetLastError();

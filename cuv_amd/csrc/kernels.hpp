@@ -58,4 +58,7 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream);
 
+// dst[d] = mean of diagonal d over its valid slots (row_fact == 1), dst on the device.
+hipError_t launch_avg_diagonals(const DiaView &A, const float *vals, float *dst, hipStream_t stream);
+
 }  // namespace cuvdia

@@ -141,6 +141,22 @@ def densedense_to_dia(C, bd, A, B, factAB=1.0, factC=0.0, sync=True):
     return C
 
 
+def avg_diagonals(dst, A, sync=True):
+    """dst[d] = mean of diagonal d of A over its valid slots
+    (src/cuv/matrix_ops/diagonals.cu:24-51); dst: float32 CUDA tensor of num_dia entries."""
+    if A.row_fact != 1:
+        raise RuntimeError("dia.row_fact( )==1")
+    if not (isinstance(dst, torch.Tensor) and dst.is_cuda and dst.dtype == torch.float32 and dst.is_contiguous()
+            and dst.numel() == A.num_dia):
+        raise RuntimeError("dia.num_dia( )==dst.size( )")
+    with torch.cuda.device(dst.device):
+        _lib.check(_lib.lib().cuvdia_avg_diagonals_f32(A.desc, A.vec.data_ptr(), dst.data_ptr(), _stream_ptr()),
+                   "cuvdia_avg_diagonals_f32")
+        if sync:
+            torch.cuda.current_stream().synchronize()
+    return dst
+
+
 def to_device_colmajor(a, device="cuda:0"):
     """numpy (rows, batch) array -> torch (batch, rows) contiguous CUDA tensor
     holding the same column-major matrix."""

@@ -110,6 +110,18 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals_device,
                       const float *B_device, long long ldb, int batch,
                       float alpha, float beta, void *stream);
 
+/* dst[d] = mean of stored diagonal d over its valid (non-padding) slots, for
+ * every table position d; dst is a device array of num_dia floats.  Replaces
+ * avg_diagonals<float,dev_memory_space> (src/cuv/matrix_ops/diagonals.cu:14-22,
+ * declared in src/cuv/matrix_ops/diagonals.hpp:12) with the semantics of the
+ * host version (diagonals.cu:24-51: the mean over the N_d = min(h - max(0,-k),
+ * w - max(0,k)) valid slots, padding never read; the reference's device
+ * version averages over the padded stride instead).  row_fact must be 1
+ * (diagonals.cu:28), else CUVDIA_EUNSUPPORTED; a diagonal without valid slots
+ * yields 0. */
+int cuvdia_avg_diagonals_f32(const cuvdia_desc *desc, const float *A_vals_device,
+                             float *dst_device, void *stream);
+
 /* The same two operations taking the offset table from HOST memory on every
  * call, for callers that hold only a dia_matrix (the reference signatures
  * carry no descriptor for prod).  A descriptor is created on first sight of

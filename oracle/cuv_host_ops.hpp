@@ -86,6 +86,17 @@ inline void densedense_to_dia_literal(dia_matrix<float, host_memory_space> &C,
     cuvAssert(rc == 0);
 }
 
+// Mean of every stored diagonal over its valid slots
+// (src/cuv/matrix_ops/diagonals.cu:24-51).
+inline void avg_diagonals(tensor<float, host_memory_space> &dst, const dia_matrix<float, host_memory_space> &dia)
+{
+    cuvAssert(dia.row_fact() == 1);
+    cuvAssert(dia.num_dia() == dst.size());
+    const int rc = oracle_avg_diagonals_f32((int)dia.h(), (int)dia.w(), dia.num_dia(), (int)dia.stride(),
+                                            dia.host_offsets().data(), dia.vec().ptr(), dst.ptr());
+    cuvAssert(rc == 0);
+}
+
 // Dense C = factC*C + factAB*op(A)*op(B), fp64 accumulation: stands in for the
 // CBLAS sgemm the reference cross-checks against (src/cuv/matrix_ops/matrix_ops.cu:177-304).
 inline void prod(tensor<float, host_memory_space, column_major> &dst,

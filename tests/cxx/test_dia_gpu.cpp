@@ -125,6 +125,36 @@ TEST_CASE(dd2s_cmp_dev_host)
     MAT_CMP(f.C, C2, 0.01f);
 }
 
+// src/tests/dia_mat.cpp:130-140 sets this fixture up (the call itself is
+// commented out there); sequence() data makes every mean a closed form.
+TEST_CASE(avg_diagonals_dev)
+{
+    dia_matrix<float, host_memory_space> w(32, 16, 7, 32, 1);
+    std::vector<int> off;
+    for (int i = -3; i <= 3; ++i) off.push_back(i);
+    w.set_offsets(off);
+    sequence(w.vec());
+    dia_matrix<float, dev_memory_space> wd(32, 16, 7, 32, 1);
+    convert(wd, w);
+    tensor<float, dev_memory_space> avg(7);
+    tensor<float, host_memory_space> avg_h(7), avg_ref(7);
+    avg_diagonals(avg, wd);
+    avg_diagonals(avg_ref, w);
+    convert(avg_h, avg);
+    for (int d = 0; d < 7; ++d) {
+        const int k = off[d], i0 = std::max(0, -k), j0 = std::max(0, k);
+        const int n = std::min(32 - i0, 16 - j0);
+        const float exact = 32.f * d + i0 + 0.5f * (n - 1);      // mean of 32 d + i, i = i0 .. i0 + n - 1
+        CHECK(close_pct(avg_h[d], exact, 0.001f));
+        CHECK(close_pct(avg_h[d], avg_ref[d], 0.001f));
+    }
+    dia_matrix<float, dev_memory_space> steep(36, 19, 7, 36, 4);
+    steep.set_offsets(off);
+    CHECK_THROWS(avg_diagonals(avg, steep));
+    tensor<float, dev_memory_space> wrong(5);
+    CHECK_THROWS(avg_diagonals(wrong, wd));
+}
+
 TEST_CASE(spmv_uninit)
 {
     dia_matrix<float, host_memory_space> w(32, 16, 3, 32, 1);

@@ -404,3 +404,60 @@ def test_cfg4_full_size_properties(gu):
     rhs = float((Y2.double() * X.double()).sum()) / batch
     scale = float((Y2.double().abs() * X.double()).sum()) / batch
     assert abs(lhs - rhs) <= 1e-5 * scale, ("gradient adjoint identity", lhs, rhs, scale)
+
+
+# ------------------------------------------------------------ avg_diagonals ---
+@pytest.mark.parametrize("h,w,offs", [
+    (32, 16, [-3, -2, -1, 0, 1, 2, 3]),
+    (1000, 700, [0, 5, -999, 699, -400, 12]),
+    (16384, 16384, [dy * 128 + dx for dy in range(-3, 4) for dx in range(-3, 4)]),
+    (40, 40, [39, -39, 0, 100, -100]),                # single-slot and empty diagonals
+])
+def test_avg_diagonals(oracle, gu, h, w, offs):
+    """Mean of each diagonal over its valid slots against the host loop
+    (serial fp32 sum); the device sums in a different order, so the bound is
+    1e-5 of the mean magnitude sum.  Padding holds NaN and must not be read."""
+    import torch
+    from cuv_amd import dia as D
+    rng = np.random.default_rng(h + w)
+    A = _rand_dia(oracle, rng, h, w, offs, 1, pad=np.nan)
+    valid = oracle.valid_mask(A).reshape(len(offs), -1)
+    n_valid = valid.sum(axis=1)
+    ref = oracle.avg_diagonals(A)
+    vals = np.nan_to_num(A.vals.reshape(len(offs), -1))
+    exact = np.where(n_valid > 0, vals.astype(np.float64).sum(axis=1) / np.maximum(n_valid, 1), 0.0)
+    mag = np.where(n_valid > 0, np.abs(vals).astype(np.float64).sum(axis=1) / np.maximum(n_valid, 1), 0.0)
+    dev = gu.make_dev_dia(A)
+    out = torch.full((len(offs),), float("nan"), dtype=torch.float32, device="cuda:0")
+    D.avg_diagonals(out, dev)
+    got = out.cpu().numpy().astype(np.float64)
+    assert np.isfinite(got).all()
+    live = n_valid > 0
+    assert np.all(np.abs(got[live] - ref[live]) <= 1e-5 * mag[live] + 1e-30)
+    assert np.all(np.abs(got[live] - exact[live]) <= 1e-5 * mag[live] + 1e-30)
+    assert np.all(got[~live] == 0.0)                  # the reference divides by zero there
+    # sequence() data: every mean is a closed form (src/tests/dia_mat.cpp:130-140 fixture)
+    S = oracle.Dia(h, w, offs, A.stride, 1)
+    small = h * len(offs) < 2 ** 22
+    if small:
+        S.vals[:] = np.arange(S.vals.size, dtype=np.float32)
+        D.avg_diagonals(out, gu.make_dev_dia(S))
+        got = out.cpu().numpy()
+        for d, k in enumerate(offs):
+            i0, j0 = max(0, -k), max(0, k)
+            n = min(h - i0, w - j0)
+            if n > 0:
+                assert abs(got[d] - (S.stride * d + i0 + (n - 1) / 2)) <= 1e-6 * (S.stride * d + i0 + n)
+
+
+def test_avg_diagonals_errors(oracle, gu):
+    import torch
+    from cuv_amd import dia as D
+    A = D.dev_dia_matrix_f(36, 19, 3, 36, 4)
+    A.set_offsets([0, 1, -1])
+    with pytest.raises(RuntimeError):
+        D.avg_diagonals(torch.zeros(3, device="cuda:0"), A)
+    B = D.dev_dia_matrix_f(32, 16, 3, 32, 1)
+    B.set_offsets([0, 1, -1])
+    with pytest.raises(RuntimeError):
+        D.avg_diagonals(torch.zeros(4, device="cuda:0"), B)
