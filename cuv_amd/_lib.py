@@ -44,6 +44,7 @@ def lib():
     L.cuvdia_set_path.argtypes = [c_int]
     L.cuvdia_last_path.restype = c_int
     L.cuvdia_plan_chunks.argtypes = [ip, c_int, c_int, ip, ip, ip, c_int]
+    L.cuvdia_plan_units.argtypes = [ip, c_int, ip, ip, c_int]
     L.cuvdia_desc_create.argtypes = [ctypes.POINTER(c_vp), ip, c_int, c_int, c_int, c_int, c_int]
     L.cuvdia_desc_destroy.argtypes = [c_vp]
     L.cuvdia_desc_info.argtypes = [c_vp, ip, ip, ctypes.POINTER(c_ll)]

@@ -119,6 +119,25 @@ int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
     return n;
 }
 
+int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap)
+{
+    if (!offsets_host || nd < 1) return CUVDIA_EINVAL;
+    std::vector<Unit> un;
+    try {
+        un = plan_units(plan_chunks(offsets_host, nd, false));
+    } catch (const std::bad_alloc &) {
+        return CUVDIA_ENOMEM;
+    }
+    const int n = (int)un.size();
+    if (n <= cap && c1 && c2) {
+        for (int u = 0; u < n; ++u) {
+            c1[u] = un[u].c1;
+            c2[u] = un[u].c2;
+        }
+    }
+    return n;
+}
+
 int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
                        int h, int w, int stride, int row_fact)
 {

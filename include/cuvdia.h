@@ -81,6 +81,16 @@ int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t,
 int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
                        int *s0, int *len, int *slot, int cap);
 
+/* Pure host function: the work units the tiled dense x dense^T projection
+ * walks.  A unit is one chunk of the normal (transposed == 0) chunk table, or
+ * two chunks adjacent in that table whose first shifts differ by a positive
+ * multiple of 4 of at most 128 rows (two rows of a 2-d window): a wave serves
+ * both from one staged band of the second operand.  c1[u] is the unit's chunk
+ * index, c2[u] its second chunk or -1.  Returns the number of units (also when
+ * it exceeds cap; then nothing is written), or a negative error.  The role of
+ * the block list built in src/cuv/matrix_ops/densedense_to_sparse.cu:123-171. */
+int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap);
+
 /* dst = beta*dst + alpha*op(A)*B for a batch of dense columns.
  * Replaces prod<float,dev_memory_space,column_major>(dst, dia A, B, transA,
  * 'n', factAB, factC) (src/cuv/matrix_ops/spmv.cu:221-247), the spmv it

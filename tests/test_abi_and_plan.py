@@ -121,3 +121,36 @@ def test_plan_rejects_bad_arguments():
     assert L.cuvdia_plan_chunks(None, 3, 0, None, None, None, 0) == _lib.EINVAL
     offs = np.array([1], np.int32)
     assert L.cuvdia_plan_chunks(offs.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), 0, 0, None, None, None, 0) == _lib.EINVAL
+
+
+def _units(offs):
+    from cuv_amd import _lib
+    L = _lib.lib()
+    ip = ctypes.POINTER(ctypes.c_int)
+    offs = np.ascontiguousarray(offs, np.int32)
+    n = L.cuvdia_plan_units(offs.ctypes.data_as(ip), offs.size, None, None, 0)
+    assert n >= 1
+    c1, c2 = np.zeros(n, np.int32), np.zeros(n, np.int32)
+    assert L.cuvdia_plan_units(offs.ctypes.data_as(ip), offs.size, c1.ctypes.data_as(ip), c2.ctypes.data_as(ip), n) == n
+    return list(zip(c1.tolist(), c2.tolist()))
+
+
+def test_units_pair_window_rows():
+    # 7x7 window on a 128-wide map: 7 chunks with first shifts 128 apart -> 3 pairs and a single
+    offs = [dy * 128 + dx for dy in range(-3, 4) for dx in range(-3, 4)]
+    assert _units(offs) == [(0, 1), (2, 3), (4, 5), (6, -1)]
+    # every chunk appears exactly once, in order
+    for o in ([0], list(range(-20, 21)), [5, -7, 0, 39, -39], [dy * 64 + dx for dy in range(5) for dx in range(8)]):
+        got = _units(o)
+        flat = [c for u in got for c in u if c >= 0]
+        assert flat == list(range(len(_plan(o, False)[0])))
+
+
+def test_units_pairing_rule():
+    # first shifts 8 apart (multiple of 4, <= 128): a pair; 7 apart or 132 apart: singles
+    assert _units(list(range(-8, -1)) + list(range(0, 8))) == [(0, 1)]
+    assert _units(list(range(0, 13))) == [(0, -1), (1, -1)]                 # one run of 13 -> chunks 7 + 6, shifts 7 apart
+    assert _units([0, 1, 132, 133]) == [(0, -1), (1, -1)]
+    assert _units([0, 1, 128, 129, 256]) == [(0, 1), (2, -1)]
+    from cuv_amd import _lib
+    assert _lib.lib().cuvdia_plan_units(None, 3, None, None, 0) == _lib.EINVAL
