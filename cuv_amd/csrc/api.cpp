@@ -47,6 +47,20 @@ int hip_fail(hipError_t e, const char *what)
     return CUVDIA_EHIP;
 }
 
+// A descriptor's tables live on the device that was current when it was
+// created; launching with it from another device would hand the kernels
+// pointers they cannot reach.
+int check_device(const cuvdia_desc *desc)
+{
+    int device = -1;
+    const hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return CUVDIA_ENODEVICE;
+    }
+    return device == desc->device ? CUVDIA_OK : CUVDIA_EINVAL;
+}
+
 int validate_shape(const int *offsets, int nd, int h, int w, int stride, int rf)
 {
     if (!offsets || nd < 1 || h < 1 || w < 1 || rf < 1 || stride < 1) return CUVDIA_EINVAL;
@@ -252,9 +266,10 @@ int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals, const float *B
     const int n_out = trans ? desc->w : desc->h;
     const int n_in = trans ? desc->h : desc->w;
     if (ldb < n_in || ldd < n_out) return CUVDIA_ESHAPE;
+    if (const int rc = check_device(desc)) return rc;
 
     const int forced = g_path.load();
-    const bool tiled_possible = spmm_tiled_ok(desc->view, ldb, trans);
+    const bool tiled_possible = spmm_tiled_ok(desc->view, ldb, ldd, trans);
     bool tiled;
     if (forced == CUVDIA_PATH_TILED) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
@@ -279,6 +294,7 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
     if (!desc || !C_vals || batch < 0) return CUVDIA_EINVAL;
     if (batch > 0 && (!A || !B)) return CUVDIA_EINVAL;
     if (batch > 0 && (lda < desc->h || ldb < desc->w)) return CUVDIA_ESHAPE;
+    if (const int rc = check_device(desc)) return rc;
 
     const int forced = g_path.load();
     const bool tiled_possible = dd2dia_tiled_ok(desc->view, lda, ldb, batch);
@@ -313,6 +329,10 @@ std::mutex g_cache_mutex;
 std::list<CacheEntry> g_cache;              // most recently used first
 constexpr size_t CACHE_CAPACITY = 32;
 
+// Caller holds g_cache_mutex, and keeps holding it until the launch that uses
+// the descriptor has been enqueued: an eviction by another thread (which
+// waits for the device before freeing) can then never pull a table from
+// under a launch in progress.
 int cached_desc(const int *offsets, int nd, int stride, int h, int w, int rf, cuvdia_desc **out)
 {
     *out = nullptr;
@@ -323,7 +343,6 @@ int cached_desc(const int *offsets, int nd, int stride, int h, int w, int rf, cu
         (void)hipGetLastError();
         return CUVDIA_ENODEVICE;
     }
-    std::lock_guard<std::mutex> lock(g_cache_mutex);
     for (auto it = g_cache.begin(); it != g_cache.end(); ++it) {
         if (it->h == h && it->w == w && it->stride == stride && it->rf == rf &&
             it->device == device && (int)it->offsets.size() == nd &&
@@ -373,6 +392,7 @@ int cuvdia_avg_diagonals_f32(const cuvdia_desc *desc, const float *A_vals, float
 {
     if (!desc || !A_vals || !dst) return CUVDIA_EINVAL;
     if (desc->rf != 1) return CUVDIA_EUNSUPPORTED;      // src/cuv/matrix_ops/diagonals.cu:28
+    if (const int rc = check_device(desc)) return rc;
     const hipError_t e = launch_avg_diagonals(desc->view, A_vals, dst, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "avg_diagonals kernel launch");
 }
@@ -382,6 +402,7 @@ int cuvdia_spmm_offsets_f32(const float *A_vals, const int *offsets_host, int nd
                             float *dst, long long ldd, int batch, char transA,
                             float alpha, float beta, void *stream)
 {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
     cuvdia_desc *d = nullptr;
     const int rc = cached_desc(offsets_host, nd, stride, h, w, row_fact, &d);
     if (rc) return rc;
@@ -393,6 +414,7 @@ int cuvdia_dd2dia_offsets_f32(float *C_vals, const int *offsets_host, int nd, in
                               const float *B, long long ldb, int batch,
                               float alpha, float beta, void *stream)
 {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
     cuvdia_desc *d = nullptr;
     const int rc = cached_desc(offsets_host, nd, stride, h, w, row_fact, &d);
     if (rc) return rc;

@@ -965,15 +965,16 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
     return hipGetLastError();
 }
 
-bool spmm_tiled_ok(const DiaView &A, long long ldb, bool trans)
+bool spmm_tiled_ok(const DiaView &A, long long ldb, long long ldd, bool trans)
 {
     // buffer resources address 32-bit byte offsets below the out-of-range marker
-    const long long n_in = trans ? A.h : A.w;
+    const long long n_in = trans ? A.h : A.w, n_out = trans ? A.w : A.h;
     const long long x_bytes = ((SP_COLS - 1) * ldb + n_in) * 4;
+    const long long y_bytes = ((SP_COLS - 1) * ldd + n_out) * 4;
     const long long a_bytes = (long long)A.nd * A.stride * 4;
     const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
     return A.rf == 1 && n_in >= 4 && nchunks <= SP_MAX_CHUNKS && x_bytes < (long long)OOB_OFFSET &&
-           a_bytes < (long long)OOB_OFFSET;
+           y_bytes < (long long)OOB_OFFSET && a_bytes < (long long)OOB_OFFSET;
 }
 
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,

@@ -39,7 +39,7 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
 
 // Whether the tiled SpMM can serve these operands (row_fact 1, operand extents
 // within its 32-bit buffer addressing).
-bool spmm_tiled_ok(const DiaView &A, long long ldb, bool trans);
+bool spmm_tiled_ok(const DiaView &A, long long ldb, long long ldd, bool trans);
 
 // C_d[i] = beta*C_d[i] + alpha*sum_c A[i,c]*B[k_d + i/rf, c] on valid slots.
 // One thread per slot, serial over the batch; honours row_fact.

@@ -24,7 +24,10 @@
  *     "results visible on return" behaviour (spmv.cu:99,
  *     densedense_to_sparse.cu:295);
  *   - no entry point allocates device memory except cuvdia_desc_create and
- *     the first use of a new offset table by the *_offsets_* forms.
+ *     the first use of a new offset table by the *_offsets_* forms;
+ *   - a descriptor belongs to the device that was current when it was
+ *     created; a compute call made while another device is current returns
+ *     CUVDIA_EINVAL.  The *_offsets_* forms keep one descriptor per device.
  */
 #ifndef CUVDIA_H
 #define CUVDIA_H
