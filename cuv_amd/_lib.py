@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libcuvdia.so")
 
 OK = 0
 EINVAL, ESHAPE, EHIP, ENOMEM, EUNSUPPORTED, ENODEVICE = -1, -2, -3, -4, -5, -6
+ACT_NONE, ACT_SIGMOID = 0, 1
 PATH_AUTO, PATH_GENERIC, PATH_TILED = 0, 1, 2
 
 _lib = None
@@ -49,6 +50,8 @@ def lib():
     L.cuvdia_desc_destroy.argtypes = [c_vp]
     L.cuvdia_desc_info.argtypes = [c_vp, ip, ip, ctypes.POINTER(c_ll)]
     L.cuvdia_spmm_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp]
+    L.cuvdia_spmm_bias_act_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp, c_int,
+                                           c_vp]
     L.cuvdia_dd2dia_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_f, c_f, c_vp]
     L.cuvdia_avg_diagonals_f32.argtypes = [c_vp, c_vp, c_vp, c_vp]
     L.cuvdia_spmm_offsets_f32.argtypes = [c_vp, ip, c_int, c_int, c_int, c_int, c_int, c_vp, c_ll,

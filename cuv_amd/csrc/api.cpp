@@ -253,10 +253,12 @@ int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t, long
     return CUVDIA_OK;
 }
 
-int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
-                    float *dst, long long ldd, int batch, char transA,
-                    float alpha, float beta, void *stream)
+int cuvdia_spmm_bias_act_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
+                             float *dst, long long ldd, int batch, char transA,
+                             float alpha, float beta, const float *bias, int act, void *stream)
 {
+    if (act != CUVDIA_ACT_NONE && act != CUVDIA_ACT_SIGMOID) return CUVDIA_EINVAL;
+    const SpEpilogue ep{bias, act};
     if (!desc || !A_vals || batch < 0) return CUVDIA_EINVAL;
     // make_spmv_header.pl:121-123: anything but 'n' / 't' is an error
     if (transA != 'n' && transA != 't') return CUVDIA_EINVAL;
@@ -281,10 +283,18 @@ int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals, const float *B
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const hipError_t e = tiled
-        ? launch_spmm_tiled(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, s)
-        : launch_spmm_generic(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, s);
+        ? launch_spmm_tiled(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s)
+        : launch_spmm_generic(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s);
     t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "spmm kernel launch");
+}
+
+int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
+                    float *dst, long long ldd, int batch, char transA,
+                    float alpha, float beta, void *stream)
+{
+    return cuvdia_spmm_bias_act_f32(desc, A_vals, B, ldb, dst, ldd, batch, transA, alpha, beta, nullptr,
+                                    CUVDIA_ACT_NONE, stream);
 }
 
 int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, long long lda,

@@ -57,6 +57,14 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Last step of an SpMM result element: optional per-row bias, optional
+// logistic sigmoid 1/(1+exp(-v)) (src/cuv/tensor_ops/functors.hpp:122).
+__device__ __forceinline__ float sp_finish(float v, float bias, int act)
+{
+    v += bias;
+    return act == 1 ? 1.f / (1.f + expf(-v)) : v;
+}
+
 // ------------------------------------------------------------------ generic --
 
 template <int CB>
@@ -64,7 +72,7 @@ __global__ __launch_bounds__(256) void spmm_generic_kernel(
     const int *__restrict__ offsets, int nd, const float *__restrict__ vals, int stride,
     int h, int w, int rf, const float *__restrict__ X, long long ldx,
     float *__restrict__ Y, long long ldy, int n_out, int batch, int trans,
-    float alpha, float beta)
+    float alpha, float beta, SpEpilogue ep)
 {
     const long long o = (long long)blockIdx.x * 256 + threadIdx.x;
     const int c0 = blockIdx.y * CB;
@@ -112,7 +120,8 @@ __global__ __launch_bounds__(256) void spmm_generic_kernel(
     for (int c = 0; c < CB; ++c) {
         if (c0 + c < batch) {
             float *y = Y + (long long)(c0 + c) * ldy + o;
-            *y = (beta == 0.f) ? alpha * acc[c] : beta * (*y) + alpha * acc[c];
+            const float v = (beta == 0.f) ? alpha * acc[c] : beta * (*y) + alpha * acc[c];
+            *y = sp_finish(v, ep.bias ? ep.bias[o] : 0.f, ep.act);
         }
     }
 }
@@ -332,12 +341,12 @@ constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used 
 // loads as a scalar offset, nothing is clamped or shifted, and a chunk costs a
 // couple of vector instructions besides its FMAs.  EDGE = true handles the
 // tiles at the operand's ends.
-template <int LCK, int T, int NTAB, bool EDGE>
+template <int LCK, int T, int NTAB, bool EDGE, bool EP>
 __device__ __forceinline__ void spmm_tile(
     float (&lds)[2][SP_STAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
-    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes)
+    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, SpEpilogue ep)
 {
     typedef SpShape<T> S;
     constexpr int SP_WAVES = S::WAVES, SP_LOADS = S::LOADS, SP_APW = S::APW, SP_CPW = S::CPW, SP_T = T;
@@ -556,24 +565,27 @@ __device__ __forceinline__ void spmm_tile(
     __syncthreads();
     const long long row = (long long)row0 + lane;
     if (row < n_out) {
+        const float bias = (EP && ep.bias) ? ep.bias[row] : 0.f;
 #pragma unroll
         for (int q = 0; q < SP_CPW; ++q) {
             const int col = wave * SP_CPW + q;
             if (col0 + col < batch) {
                 const float v = out[col * SP_OPITCH + lane];
                 float *y = Y + (long long)(col0 + col) * ldy + row;
-                *y = (beta == 0.f) ? alpha * v : beta * ypre[q] + alpha * v;
+                const float r = (beta == 0.f) ? alpha * v : beta * ypre[q] + alpha * v;
+                *y = EP ? sp_finish(r, bias, ep.act) : r;
             }
         }
     }
 }
 
-template <int LCK, int T, int NTAB>
+// EP = false: the plain product (no bias, no activation); EP = true applies `ep`.
+template <int LCK, int T, int NTAB, bool EP>
 __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes,
-    int s_min, int s_max)
+    int s_min, int s_max, SpEpilogue ep)
 {
     __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
@@ -596,11 +608,11 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
         }
     }
     if (lean)
-        spmm_tile<LCK, T, NTAB, false>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
-                                 n_out, n_in, batch, alpha, beta, a_bytes);
+        spmm_tile<LCK, T, NTAB, false, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+                                 n_out, n_in, batch, alpha, beta, a_bytes, ep);
     else
-        spmm_tile<LCK, T, NTAB, true>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
-                                n_out, n_in, batch, alpha, beta, a_bytes);
+        spmm_tile<LCK, T, NTAB, true, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+                                n_out, n_in, batch, alpha, beta, a_bytes, ep);
 }
 
 // ------------------------------------------------------------ tiled dd2dia --
@@ -946,7 +958,7 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
 
 hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float *B, long long ldb,
                                float *dst, long long ldd, int batch, bool trans,
-                               float alpha, float beta, hipStream_t stream)
+                               float alpha, float beta, SpEpilogue ep, hipStream_t stream)
 {
     const int n_out = trans ? A.w : A.h;
     constexpr int CB = 4;
@@ -959,7 +971,7 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
         hipLaunchKernelGGL(spmm_generic_kernel<CB>, grid, dim3(256), 0, stream,
                            A.offsets_dev, A.nd, vals, A.stride, A.h, A.w, A.rf,
                            B + (long long)done * ldb, ldb, dst + (long long)done * ldd, ldd,
-                           n_out, slab, trans ? 1 : 0, alpha, beta);
+                           n_out, slab, trans ? 1 : 0, alpha, beta, ep);
         done += slab;
     }
     return hipGetLastError();
@@ -979,7 +991,7 @@ bool spmm_tiled_ok(const DiaView &A, long long ldb, long long ldd, bool trans)
 
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
-                             float alpha, float beta, hipStream_t stream)
+                             float alpha, float beta, SpEpilogue ep, hipStream_t stream)
 {
     const int n_out = trans ? A.w : A.h;
     const int n_in = trans ? A.h : A.w;
@@ -994,23 +1006,27 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const dim3 grid((unsigned)(row_tiles * col_tiles));
     // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
     // at the sizes this path is measured on.
-#define CUVDIA_SPMM_LAUNCH(L)                                                                       \
-    case L:                                                                                         \
-        if (nchunks <= 64)                                                                          \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 1>), grid, dim3(512), 0, stream, chunks,    \
-                               nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
-                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);    \
-        else                                                                                        \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 4>), grid, dim3(512), 0, stream, chunks,    \
-                               nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out,     \
-                               n_in, batch, alpha, beta, (int)col_tiles, a_bytes, s_min, s_max);    \
+#define CUVDIA_SPMM_ARGS chunks, nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha, \
+                         beta, (int)col_tiles, a_bytes, s_min, s_max, ep
+#define CUVDIA_SPMM_LAUNCH(L)                                                                                   \
+    case L:                                                                                                     \
+        if (nchunks <= 64 && !fused)                                                                            \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 1, false>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS); \
+        else if (nchunks <= 64)                                                                                 \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 1, true>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS);  \
+        else if (!fused)                                                                                        \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 4, false>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS); \
+        else                                                                                                    \
+            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 4, true>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS);  \
         break;
+    const bool fused = ep.bias != nullptr || ep.act != 0;
     switch (lck) {
         CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
         CUVDIA_SPMM_LAUNCH(5) CUVDIA_SPMM_LAUNCH(6) CUVDIA_SPMM_LAUNCH(7) CUVDIA_SPMM_LAUNCH(8)
         default: return hipErrorInvalidValue;
     }
 #undef CUVDIA_SPMM_LAUNCH
+#undef CUVDIA_SPMM_ARGS
     return hipGetLastError();
 }
 

@@ -23,11 +23,19 @@ struct DiaView {
     const Unit *single_units_dev;   // one unit per chunk of the normal table, in table order
 };
 
+// What the SpMM kernels do to a result element before storing it:
+// v = beta*dst + alpha*sum; v += bias[row] (bias != nullptr); v = 1/(1+exp(-v))
+// (act == 1).  The default, {nullptr, 0}, stores the plain product.
+struct SpEpilogue {
+    const float *bias;   // one value per output row, on the device, or nullptr
+    int act;             // 0: none, 1: logistic sigmoid
+};
+
 // dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch
 // columns per thread; honours row_fact.
 hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float *B, long long ldb,
                                float *dst, long long ldd, int batch, bool trans,
-                               float alpha, float beta, hipStream_t stream);
+                               float alpha, float beta, SpEpilogue ep, hipStream_t stream);
 
 // Same contract, row_fact == 1 only: 64 output rows x 64 batch columns per
 // workgroup, dense tile staged through LDS once per run chunk, lanes own
@@ -35,7 +43,7 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
 // values are broadcast across each 16-lane row by DPP.
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
-                             float alpha, float beta, hipStream_t stream);
+                             float alpha, float beta, SpEpilogue ep, hipStream_t stream);
 
 // Whether the tiled SpMM can serve these operands (row_fact 1, operand extents
 // within its 32-bit buffer addressing).

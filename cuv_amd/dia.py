@@ -125,6 +125,28 @@ def prod(dst, A, B, transA="n", transB="n", factAB=1.0, factC=0.0, sync=True):
     return dst
 
 
+def prod_bias_act(dst, A, B, transA="n", factAB=1.0, factC=0.0, bias=None, act=_lib.ACT_NONE, sync=True):
+    """dst = act(factC*dst + factAB*op(A)*B + bias[row]): prod, matrix_plus_col and the SIGM functor of an
+    RBM/MLP layer update in one launch (examples/rbm/base.py:48-54,127-136)."""
+    if transA not in ("n", "t"):
+        raise RuntimeError("transA must be 'n' or 't'")
+    n_out, n_in = (A.w, A.h) if transA == "t" else (A.h, A.w)
+    bb, ldb = _check_dense(B, n_in, "B")
+    bd, ldd = _check_dense(dst, n_out, "dst")
+    if bb != bd:
+        raise RuntimeError("dst.shape()[1] == B.shape()[1]")
+    if bias is not None and not (isinstance(bias, torch.Tensor) and bias.is_cuda and bias.dtype == torch.float32
+                                 and bias.is_contiguous() and bias.numel() == n_out):
+        raise RuntimeError("A.shape()[0] == v.size()")
+    with torch.cuda.device(dst.device):
+        _lib.check(_lib.lib().cuvdia_spmm_bias_act_f32(
+            A.desc, A.vec.data_ptr(), B.data_ptr(), ldb, dst.data_ptr(), ldd, bb, transA.encode(), factAB, factC,
+            bias.data_ptr() if bias is not None else None, act, _stream_ptr()), "cuvdia_spmm_bias_act_f32")
+        if sync:
+            torch.cuda.current_stream().synchronize()
+    return dst
+
+
 def densedense_to_dia(C, bd, A, B, factAB=1.0, factC=0.0, sync=True):
     """C = factC*C + factAB*proj(A*B') on C's stored diagonals
     (src/cuv/matrix_ops/densedense_to_sparse.hpp:107-129)."""

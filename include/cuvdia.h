@@ -49,6 +49,10 @@ extern "C" {
 #define CUVDIA_PATH_GENERIC  1  /* one-thread-per-output kernels, any row_fact    */
 #define CUVDIA_PATH_TILED    2  /* LDS-staged, register-blocked kernels (rf == 1) */
 
+/* Activation applied by cuvdia_spmm_bias_act_f32. */
+#define CUVDIA_ACT_NONE      0
+#define CUVDIA_ACT_SIGMOID   1  /* 1 / (1 + exp(-x)), src/cuv/tensor_ops/functors.hpp:122 */
+
 /* Opaque description of one diagonal pattern: shape, offset table, and the
  * device-resident run table the tiled kernels walk.  Replaces the contents of
  * dev_block_descriptor (src/cuv/matrix_ops/densedense_to_sparse.hpp:69-105,
@@ -109,6 +113,21 @@ int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals_device,
                     const float *B_device, long long ldb,
                     float *dst_device, long long ldd, int batch,
                     char transA, float alpha, float beta, void *stream);
+
+/* The same product with the two element-wise passes an RBM/MLP layer runs on
+ * its result fused into the store:
+ *   dst = act(beta*dst + alpha*op(A)*B + bias[row])
+ * i.e. prod (above), then matrix_plus_col(dst, bias)
+ * (src/cuv/matrix_ops/matrix_ops.hpp:307), then apply_scalar_functor(dst, SIGM)
+ * (src/cuv/tensor_ops/functors.hpp:122) as in examples/rbm/base.py:48-54,127-136.
+ * bias: device array with one float per output row, or NULL for none;
+ * act: CUVDIA_ACT_NONE or CUVDIA_ACT_SIGMOID.  With bias == NULL and
+ * CUVDIA_ACT_NONE this is cuvdia_spmm_f32.  batch == 0 is a no-op. */
+int cuvdia_spmm_bias_act_f32(const cuvdia_desc *desc, const float *A_vals_device,
+                             const float *B_device, long long ldb,
+                             float *dst_device, long long ldd, int batch,
+                             char transA, float alpha, float beta,
+                             const float *bias_device, int act, void *stream);
 
 /* C = beta*C + alpha*proj(A*B') restricted to the stored diagonals of C:
  *   C_d[i] = beta*C_d[i] + alpha * sum_c A[i,c] * B[offsets[d] + i/row_fact, c]

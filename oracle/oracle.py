@@ -201,6 +201,20 @@ def filter_offsets(px, py, fs, input_maps, output_maps):
     return out
 
 
+def prod_bias_act(dia, B, dst=None, trans="n", alpha=1.0, beta=0.0, bias=None, sigmoid=False):
+    """The reference's sequence for a layer update, each step in fp32 as the
+    host path does it: prod (spmv.cu:145-220), matrix_plus_col
+    (matrix_ops.hpp:307: A(i, j) += v(i)), apply_scalar_functor SIGM
+    (functors.hpp:122: 1 / (1 + expf(-t)))."""
+    out = prod(dia, B, dst, trans, alpha, beta)
+    if bias is not None:
+        out = (out + np.asarray(bias, np.float32)[:, None]).astype(np.float32)
+    if sigmoid:
+        one = np.float32(1)
+        out = (one / (one + np.exp(-out, dtype=np.float32))).astype(np.float32)
+    return np.asfortranarray(out)
+
+
 def avg_diagonals(dia):
     out = np.zeros(dia.nd, np.float32)
     lib().oracle_avg_diagonals_f32(dia.h, dia.w, dia.nd, dia.stride,

@@ -461,3 +461,53 @@ def test_avg_diagonals_errors(oracle, gu):
     B.set_offsets([0, 1, -1])
     with pytest.raises(RuntimeError):
         D.avg_diagonals(torch.zeros(4, device="cuda:0"), B)
+
+
+# ----------------------------------------------- prod + bias + sigmoid, fused ---
+@pytest.mark.parametrize("trans", ["n", "t"])
+@pytest.mark.parametrize("h,w,offs,batch", [
+    (32, 16, [-3, -2, -1, 0, 1, 2, 3], 6),
+    (700, 650, [d * 25 + e for d in range(-2, 3) for e in range(-2, 3)], 96),
+    (1024, 1024, [dy * 32 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 128),
+])
+def test_prod_bias_sigmoid(oracle, gu, h, w, offs, batch, trans):
+    """dst = sigmoid(beta*dst + alpha*op(A)*B + bias) in one launch against the
+    reference's three host steps (prod, matrix_plus_col, SIGM functor).
+    Tolerance: the pre-activation is within 1e-5 of its term-magnitude sum, the
+    logistic function has slope <= 1/4 and expf differs by a few ulp between
+    the two sides: |gpu - ref| <= 0.25e-5 * mag + 4e-7."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(h + 3 * w + batch)
+    A = _rand_dia(oracle, rng, h, w, offs, 1)
+    n_in, n_out = (h, w) if trans == "t" else (w, h)
+    B = np.asfortranarray(rng.uniform(-1, 1, (n_in, batch)).astype(np.float32))
+    dst0 = np.asfortranarray(rng.uniform(-1, 1, (n_out, batch)).astype(np.float32))
+    bias = rng.uniform(-2, 2, n_out).astype(np.float32)
+    dev = gu.make_dev_dia(A)
+    Bd = D.to_device_colmajor(B)
+    bd = torch.from_numpy(bias).cuda()
+    for path in (_lib.PATH_GENERIC, _lib.PATH_TILED):
+        for (alpha, beta, use_bias, act) in ((1.0, 0.0, True, True), (0.5, -1.5, True, True),
+                                             (1.0, 0.0, True, False), (2.0, 0.25, False, True)):
+            dd = D.to_device_colmajor(dst0) if beta != 0 else torch.full((batch, n_out), float("nan"), device="cuda:0")
+            _lib.check(L.cuvdia_set_path(path), "set_path")
+            try:
+                D.prod_bias_act(dd, dev, Bd, trans, alpha, beta, bd if use_bias else None,
+                                _lib.ACT_SIGMOID if act else _lib.ACT_NONE)
+                assert L.cuvdia_last_path() == path
+            finally:
+                L.cuvdia_set_path(_lib.PATH_AUTO)
+            got = D.to_host_colmajor(dd).astype(np.float64)
+            ref = oracle.prod_bias_act(A, B, dst0 if beta != 0 else None, trans, alpha, beta,
+                                       bias if use_bias else None, act).astype(np.float64)
+            mag = oracle.prod_mag(A, B, dst0 if beta != 0 else None, trans, alpha, beta)
+            if use_bias:
+                mag = mag + np.abs(bias)[:, None]
+            assert np.isfinite(got).all()
+            tol = (0.25e-5 * mag + 4e-7) if act else (1e-5 * mag + 1e-30)
+            assert np.all(np.abs(got - ref) <= tol), (path, alpha, beta, use_bias, act,
+                                                      float((np.abs(got - ref) / tol).max()))
+            if act:
+                assert got.min() >= 0.0 and got.max() <= 1.0
