@@ -18,7 +18,7 @@ namespace cuv {
 inline void avg_diagonals(tensor<float, dev_memory_space> &dst, const dia_matrix<float, dev_memory_space> &dia)
 {
     cuvAssert(dia.row_fact() == 1);
-    cuvAssert(dia.num_dia() == dst.size());
+    cuvAssert((size_t)dia.num_dia() == (size_t)dst.size());
     cuvAssert(dst.ptr());
     cuvAssert(dia.vec_ptr());
     checkDiaCall(cuvdia_avg_diagonals_f32(dia.descriptor(), dia.vec().ptr(), dst.ptr(), NULL),

@@ -91,7 +91,7 @@ inline void densedense_to_dia_literal(dia_matrix<float, host_memory_space> &C,
 inline void avg_diagonals(tensor<float, host_memory_space> &dst, const dia_matrix<float, host_memory_space> &dia)
 {
     cuvAssert(dia.row_fact() == 1);
-    cuvAssert(dia.num_dia() == dst.size());
+    cuvAssert((size_t)dia.num_dia() == (size_t)dst.size());
     const int rc = oracle_avg_diagonals_f32((int)dia.h(), (int)dia.w(), dia.num_dia(), (int)dia.stride(),
                                             dia.host_offsets().data(), dia.vec().ptr(), dst.ptr());
     cuvAssert(rc == 0);
