@@ -36,15 +36,26 @@ typedef const Chunk __attribute__((address_space(4))) *sc_chunk_ptr;
 __device__ __forceinline__ sc_chunk_ptr scalar_ptr(const Chunk *p) { return (sc_chunk_ptr)p; }
 
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and each
-// XCD has its own L2.  Remap so that every XCD works on one contiguous span of
+// XCD has its own L2.  Remap so that every XCD works on contiguous spans of
 // tiles: neighbouring row tiles share dense-operand rows (the halo and the
-// bands +-px apart), which then hit in that XCD's L2.
+// bands +-px apart), which then hit in that XCD's L2.  The tiles are dealt out
+// in groups of 8 spans of XCD_SPAN, one span per XCD and group, so that work
+// which varies along the rows (chunks falling outside the operand) still
+// spreads evenly; the last, partial group is split into 8 near-equal spans.
+constexpr int XCD_SPAN = 64;
 __device__ __forceinline__ int xcd_tile(int bid, int nblk)
 {
-    constexpr int XCDS = 8;
-    const int q = nblk / XCDS, r = nblk % XCDS;
-    const int xcd = bid % XCDS, slot = bid / XCDS;
-    return xcd * q + (xcd < r ? xcd : r) + slot;
+    constexpr int XCDS = 8, GROUP = XCDS * XCD_SPAN;
+    const int full = nblk / GROUP * GROUP;           // tiles in whole groups
+    if (bid < full) {
+        const int g = bid / GROUP, in = bid - g * GROUP;
+        const int xcd = in % XCDS, slot = in / XCDS;
+        return g * GROUP + xcd * XCD_SPAN + slot;
+    }
+    const int rest = nblk - full, b = bid - full;
+    const int q = rest / XCDS, r = rest % XCDS;
+    const int xcd = b % XCDS, slot = b / XCDS;
+    return full + xcd * q + (xcd < r ? xcd : r) + slot;
 }
 
 // Orders this wave's LDS writes before its later LDS reads (and the reverse)
@@ -597,19 +608,34 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     // [row0 + s0, row0 + s0 + 80) lie either inside it or wholly outside (such
     // a chunk contributes nothing and is skipped through an empty resource).
     bool lean = row0 + SP_ROWS <= n_out;
+    int c_lo = 0, c_hi = nchunks;                   // the chunks whose rows lie inside the operand: a contiguous
+                                                    // range, the table being sorted by shift
     if (!((row0 + s_min >= 0) & (row0 + s_max + 4 * SP_QUADS <= n_in))) {
         const int lane = threadIdx.x & 63;
+        c_lo = nchunks;
+        c_hi = 0;
 #pragma unroll
         for (int k = 0; k < NTAB; ++k) {
-            const int a0 = row0 + chunks[min(64 * k + lane, nchunks - 1)].s0;
+            const int idx = 64 * k + lane;
+            const int a0 = row0 + chunks[min(idx, nchunks - 1)].s0;
             const bool inside = (a0 >= 0) & (a0 + 4 * SP_QUADS <= n_in);
             const bool outside = (a0 + 4 * SP_QUADS <= 0) | (a0 >= n_in);
             lean &= __builtin_amdgcn_ballot_w64(!(inside | outside)) == 0;
+            const unsigned long long m = __builtin_amdgcn_ballot_w64(inside & (idx < nchunks));
+            if (m) {
+                c_lo = min(c_lo, 64 * k + (int)__builtin_ctzll(m));
+                c_hi = max(c_hi, 64 * k + 64 - (int)__builtin_clzll(m));
+            }
+        }
+        if (c_hi <= c_lo) {                          // nothing inside: one (outside) chunk keeps the pipeline fed
+            c_lo = 0;
+            c_hi = 1;
         }
     }
     if (lean)
-        spmm_tile<LCK, T, NTAB, false, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
-                                 n_out, n_in, batch, alpha, beta, a_bytes, ep);
+        // only the chunks inside the operand are walked; the others would add zeros
+        spmm_tile<LCK, T, NTAB, false, EP>(lds, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
+                                           Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
     else
         spmm_tile<LCK, T, NTAB, true, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                 n_out, n_in, batch, alpha, beta, a_bytes, ep);
@@ -700,6 +726,10 @@ __device__ __forceinline__ void dd2dia_unit(
     const int delta = NCH == 2 ? s0[NCH - 1] - s0[0] : 0;      // rows between the two windows
     const int need = DD_ROWS + delta + CHUNK_MAX;               // staged rows that are ever read
     const int base = row0 + s0[0];                              // first staged row of B
+    // Every slot of the unit pairs row i with row i + s0 + j of B: with the
+    // whole band outside B the unit stores no matrix element, and there is
+    // nothing to compute or to write (the whole workgroup leaves together).
+    if (base + need <= 0 || base >= w) return;
     const int myrow = row0 + 4 * lane;
 
     // C values this lane will combine at the end: row row0 + 64*wave + lane of
