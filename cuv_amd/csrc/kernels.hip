@@ -28,13 +28,6 @@
 namespace cuvdia {
 namespace {
 
-// Loads through this address space are issued on the scalar unit when the
-// address is wave-uniform: a chunk-table entry is read into SGPRs and costs no
-// vector-memory or LDS bandwidth (used where the read sits outside a loop).
-typedef const Chunk __attribute__((address_space(4))) *sc_chunk_ptr;
-
-__device__ __forceinline__ sc_chunk_ptr scalar_ptr(const Chunk *p) { return (sc_chunk_ptr)p; }
-
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and each
 // XCD has its own L2.  Remap so that every XCD works on contiguous spans of
 // tiles: neighbouring row tiles share dense-operand rows (the halo and the
@@ -200,37 +193,33 @@ __global__ __launch_bounds__(AVG_THREADS) void avg_diagonals_kernel(
 
 // -------------------------------------------------------------- tiled spmm --
 //
-// Workgroup = 64 output rows x 64 batch columns, 64 / T waves of T rows each
-// (T = 8 is what the launcher uses; the text below is written for T = 16).
+// Workgroup = 64 output rows x 64 batch columns, 8 waves of T = 8 rows each.
 // Lane l of every wave owns batch column col0 + l and T running sums.  Per
 // run chunk (<= 8 consecutive shifts starting at s0):
-//   1. the dense rows [a0, a0 + 80), a0 = row0 + s0, of the 64 columns are
-//      fetched with 16-byte buffer loads (4-byte aligned is all they need),
-//      20 lanes per column and 3 columns per instruction, so every cache line
-//      of a column is requested by one instruction only, and written to LDS
-//      with 16-byte stores, columns 84 floats apart: LDS row i of a column
-//      holds dense row a0 + i.  Each wave also fetches two of the
-//      chunk's eight diagonals for all 64 rows (one 256-byte row segment per
-//      instruction) and parks them in LDS.  Rows outside the operand and
-//      diagonal slots outside the matrix become zeros (an out-of-range buffer
-//      offset reads as 0; pieces straddling the operand's first or last row
-//      are shifted into place on the way to LDS), so the arithmetic below
-//      needs no guards and never sees padding;
-//   2. each lane reads its column's window of 16 + LCK - 1 values with
-//      16-byte LDS reads (pitch/4 is odd, so the 64 lanes spread over all
-//      banks).  Every chunk is processed as LCK diagonals, LCK = the longest
-//      chunk of the table; shorter chunks carry zeros;
-//   3. for each diagonal j the wave reads A_j[16 rows] into one VGPR (lane & 15
-//      selects the row) and issues 16 FMAs whose first operand is that VGPR
-//      broadcast within each 16-lane row by DPP (row_newbcast:t):
+//   1. the dense rows a0 .., a0 = row0 + s0, that the chunk touches are staged
+//      in LDS for the 64 columns, LDS row i of a column holding dense row
+//      a0 + i, together with the chunk's diagonals for the 64 rows (wave w
+//      fetches diagonal w, one 256-byte row segment).  Rows outside the
+//      operand and diagonal slots outside the matrix become zeros (an
+//      out-of-range buffer offset reads as 0), so the arithmetic below needs
+//      no guards and never sees padding;
+//   2. each lane reads its column's window of T + LCK - 1 values with 16-byte
+//      LDS reads (the column pitch / 4 is odd, so the 64 lanes spread over
+//      all banks).  Every chunk is processed as LCK diagonals, LCK = the
+//      longest chunk of the table; shorter chunks carry zeros;
+//   3. for each diagonal j the wave reads A_j[its T rows] into one VGPR (lane
+//      & (T-1) selects the row) and issues T FMAs whose first operand is that
+//      VGPR broadcast within each 16-lane row by DPP (row_newbcast:t):
 //          acc[t] = fma(A_j[row t], win[t + j], acc[t]).
-// The loop is software-pipelined three chunks deep: while the FMAs of chunk c
-// run out of registers, chunk c+1 is being written to the other LDS buffer
-// (its window is read right after the barrier), chunk c+2 is in flight from
-// memory and chunk c+3 has just been requested.  The chunk table itself sits
-// in vector registers (lane i <-> entry i) and is read with v_readlane.
-// The epilogue transposes the sums through LDS so the store to dst is again
-// lanes-along-rows.
+// There are two bodies.  Tiles all of whose rows exist and none of whose
+// chunks straddles an end of the dense operand -- all but a few of a large
+// matrix -- take the lean body (spmm_tile_lean): its loads write LDS directly,
+// so staging costs the waves 4 instructions per chunk.  The tiles at the
+// operand's ends take spmm_tile_edge, which stages through registers because
+// it has to clamp and shift what it fetches.  Both are software-pipelined
+// three chunks deep, keep the chunk table in vector registers (lane i <->
+// entry i, read with v_readlane), and transpose the sums through LDS at the
+// end so the store to dst is lanes-along-rows.
 
 constexpr int SP_ROWS = 64;        // output rows per workgroup
 constexpr int SP_COLS = 64;        // batch columns per workgroup (one per lane)
@@ -346,14 +335,16 @@ __device__ __forceinline__ float4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, un
 }
 constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used here
 
-// EDGE = false is the body for a tile all of whose 64 output rows exist and
-// none of whose chunks straddles an end of the dense operand (each chunk's 80
-// staged rows lie inside it, or wholly outside): row positions then enter the
-// loads as a scalar offset, nothing is clamped or shifted, and a chunk costs a
-// couple of vector instructions besides its FMAs.  EDGE = true handles the
-// tiles at the operand's ends.
-template <int LCK, int T, int NTAB, bool EDGE, bool EP>
-__device__ __forceinline__ void spmm_tile(
+// The body for tiles at the operand's ends.  The dense rows [a0, a0 + 80) of
+// the 64 columns are fetched with 16-byte buffer loads into registers (20
+// lanes per column and 3 columns per instruction) and written to LDS with
+// 16-byte stores, columns 84 floats apart; a piece that straddles the
+// operand's first or last row is fetched from the nearest in-range position
+// and shifted into place on the way.  While the FMAs of chunk c run, chunk
+// c+1 is being written to the other LDS buffer (its window is read right after
+// the barrier), chunk c+2 is in flight and chunk c+3 has just been requested.
+template <int LCK, int T, int NTAB, bool EP>
+__device__ __forceinline__ void spmm_tile_edge(
     float (&lds)[2][SP_STAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
@@ -398,7 +389,6 @@ __device__ __forceinline__ void spmm_tile(
         const int col = (wave + SP_WAVES * it) * SP_CPI + grp;
         const bool live = (grp < SP_CPI) & (col < SP_COLS);
         col_off[it] = live ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) : OOB_OFFSET;
-        if (!EDGE && live) col_off[it] += 16u * quad;      // the lane's piece; the chunk's first row is a scalar offset
         lds_at[it] = live ? col * SP_PITCH + 4 * quad : SP_DUMP;
     }
     // diagonal values: wave w fetches diagonals w, w + WAVES, ... of the chunk
@@ -446,30 +436,6 @@ __device__ __forceinline__ void spmm_tile(
     // loads themselves never branch.
     auto issue = [&](const SpInfo<T> &info, SpStage<T> &st, int c) {
         const int s0 = info.s0;
-        if constexpr (!EDGE) {
-            // past the table, and for a chunk whose rows lie outside the operand,
-            // nothing is fetched: an empty resource returns zeros
-            const int a0 = row0 + s0;
-            const bool real = (c < nchunks) & (a0 >= 0) & (a0 + 4 * SP_QUADS <= n_in);
-            const __amdgpu_buffer_rsrc_t xq = make_rsrc(X + (long long)col0 * ldx, real ? x_bytes : 0u);
-            const unsigned soff = real ? (unsigned)a0 * 4u : 0u;
-#pragma unroll
-            for (int it = 0; it < SP_LOADS; ++it)
-                st.x[it] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(xq, col_off[it], soff, 0));
-            st.shift = 0;
-            st.edge = false;
-#pragma unroll
-            for (int q = 0; q < SP_APW; ++q) {
-                const int j = wave + SP_WAVES * q;
-                const int sl = info.slot[q];
-                const bool ok = real & (j < info.len) & (sl >= 0);
-                const __amdgpu_buffer_rsrc_t aq = make_rsrc(vals, ok ? a_bytes : 0u);
-                const unsigned voff = (unsigned)(ashift ? arow + s0 + j : arow) * 4u;
-                st.a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    aq, voff, (unsigned)sl * (unsigned)stride * 4u, 0));
-            }
-            return;
-        }
         const int a0 = row0 + s0;
         const int r = a0 + 4 * quad;                       // first dense row of this lane's piece
         const int rc = min(max(r, 0), n_in - 4);
@@ -492,7 +458,7 @@ __device__ __forceinline__ void spmm_tile(
         }
     };
     auto commit = [&](const SpStage<T> &st, float *buf) {
-        if (!EDGE || !st.edge) {
+        if (!st.edge) {
 #pragma unroll
             for (int it = 0; it < SP_LOADS; ++it)
                 *reinterpret_cast<float4 *>(buf + lds_at[it]) = st.x[it];
@@ -577,13 +543,209 @@ __device__ __forceinline__ void spmm_tile(
     const long long row = (long long)row0 + lane;
     if (row < n_out) {
         const float bias = (EP && ep.bias) ? ep.bias[row] : 0.f;
+        float v[SP_CPW];
+#pragma unroll
+        for (int q = 0; q < SP_CPW; ++q) v[q] = out[(wave * SP_CPW + q) * SP_OPITCH + lane];   // all reads before the first store
 #pragma unroll
         for (int q = 0; q < SP_CPW; ++q) {
             const int col = wave * SP_CPW + q;
             if (col0 + col < batch) {
-                const float v = out[col * SP_OPITCH + lane];
                 float *y = Y + (long long)(col0 + col) * ldy + row;
-                const float r = (beta == 0.f) ? alpha * v : beta * ypre[q] + alpha * v;
+                const float r = (beta == 0.f) ? alpha * v[q] : beta * ypre[q] + alpha * v[q];
+                *y = EP ? sp_finish(r, bias, ep.act) : r;
+            }
+        }
+    }
+}
+
+// Loads that deliver straight into LDS (no vector register in between): lane i
+// of the wave writes its 16 (4) bytes at lds_byte_addr + 16*i (4*i); an
+// out-of-range lane writes zeros, an inactive lane writes nothing.  They are
+// vector-memory operations and complete in order with the wave's other loads
+// (s_waitcnt vmcnt).  Written in assembly so that the waits below can be
+// placed by hand: the loop keeps two chunks of them in flight across
+// barriers, which no automatic placement allows.
+typedef int sp_int4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ sp_int4 raw_rsrc(const void *base, unsigned bytes)
+{
+    const unsigned long long b = reinterpret_cast<unsigned long long>(base);
+    return sp_int4{(int)(unsigned)b, (int)((unsigned)(b >> 32) & 0xffffu), (int)bytes, 0x00020000};
+}
+__device__ __forceinline__ void lds_load_b128(sp_int4 rsrc, unsigned lds_byte_addr, unsigned voff, unsigned soff)
+{
+    asm volatile("s_mov_b32 m0, %0\n\t"
+                 "s_nop 0\n\t"
+                 "buffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+__device__ __forceinline__ void lds_load_b32(sp_int4 rsrc, unsigned lds_byte_addr, unsigned voff, unsigned soff)
+{
+    asm volatile("s_mov_b32 m0, %0\n\t"
+                 "s_nop 0\n\t"
+                 "buffer_load_dword %1, %2, %3 offen lds"
+                 :: "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+
+// The lean body (see spmm_tile) with the staging done by loads that write LDS
+// directly.  A chunk stages 76 rows (19 16-byte pieces) of each of the 64
+// columns, column after column without gaps: piece p = 19 * column + quad
+// lives at byte 16 * p of the stage buffer, so load instruction i (lane l
+// fetching piece 64 * i + l) fills bytes [1024 * i, 1024 * i + 1024) and 19
+// instructions, every lane busy, stage the chunk.  Columns are then 76 floats
+// apart, which keeps the 16-byte window reads (one lane per column) free of
+// bank conflicts.  Wave w issues instructions w, w + 8 and w + 16 (where that
+// is past the last one it asks for nothing and zeros drop into a spare
+// kilobyte, so every wave has the same number of loads in flight) and diagonal
+// w of the chunk: 4 loads per wave and chunk, none through registers, no LDS
+// write instruction.  Three LDS buffers: chunk k lives in buffer k % 3; while
+// the FMAs of chunk c run, window(c+1) is being read, chunk c+2 is landing and
+// chunk c+3 has just been requested.
+constexpr int SP_DQUADS = 19;                       // pieces per column staged by the direct loads (76 rows)
+constexpr int SP_DPITCH = 4 * SP_DQUADS;            // floats between staged columns
+constexpr int SP_DAVALS = SP_COLS * SP_DPITCH;      // diagonal values sit behind the dense rows
+constexpr int SP_DSPARE = SP_DAVALS + SP_AVALS;     // 256 floats that idle load slots fill with zeros
+constexpr int SP_DSTAGE_FLOATS = SP_DSPARE + 256;
+static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + CHUNK_MAX - 1 <= SP_DPITCH, "staging layout");
+
+template <int LCK, int NTAB, bool EP>
+__device__ __forceinline__ void spmm_tile_lean(
+    float (&lds)[3][SP_DSTAGE_FLOATS], int row0, int col0,
+    const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
+    int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
+    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, SpEpilogue ep)
+{
+    constexpr int T = 8, WAVES = 8, CPW = SP_COLS / WAVES;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.f;
+    const int cols_here = min(SP_COLS, batch - col0);
+    const unsigned x_bytes = (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4);
+    const float *xbase = X + (long long)col0 * ldx;
+
+    float ypre[CPW];
+    {
+        const long long row = (long long)row0 + lane;
+        const __amdgpu_buffer_rsrc_t yr = make_rsrc(
+            Y + (long long)col0 * ldy, beta != 0.f ? (unsigned)(((long long)(cols_here - 1) * ldy + n_out) * 4) : 0u);
+#pragma unroll
+        for (int q = 0; q < CPW; ++q) {
+            const int col = wave * CPW + q;
+            ypre[q] = buffer_load_f32(yr, (row < n_out && col < cols_here)
+                                              ? (unsigned)(col * ldy + row) * 4u : OOB_OFFSET);
+        }
+    }
+
+    // this lane's pieces in the three load instructions the wave issues
+    unsigned x_off[3];
+    unsigned x_lds[3];                      // byte offset inside a stage buffer that the instruction fills
+#pragma unroll
+    for (int it = 0; it < 3; ++it) {
+        const int i = wave + WAVES * it;
+        const int piece = 64 * i + lane;
+        const int col = piece / SP_DQUADS, quad = piece - col * SP_DQUADS;
+        const bool live = i < SP_DQUADS;     // SP_COLS * SP_DQUADS / 64 instructions stage a chunk
+        x_off[it] = live ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) + 16u * quad : OOB_OFFSET;
+        x_lds[it] = live ? 1024u * i : SP_DSPARE * 4u;
+    }
+    const int arow = row0 + lane;
+
+    int tab_s0[NTAB], tab_len[NTAB], tab_slot[NTAB];
+#pragma unroll
+    for (int k = 0; k < NTAB; ++k) {
+        const int *e = reinterpret_cast<const int *>(chunks + min(64 * k + lane, nchunks - 1));
+        tab_s0[k] = e[0];
+        tab_len[k] = e[1];
+        tab_slot[k] = e[2 + wave];
+    }
+    const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
+    constexpr unsigned BUF_BYTES = SP_DSTAGE_FLOATS * 4u;
+
+    // requests chunk c into the buffer at byte address `buf`: 4 loads
+    auto issue = [&](int c, unsigned buf) {
+        const int cc = min(c, nchunks - 1);
+        const int l = cc & 63;
+        int s0 = __builtin_amdgcn_readlane(tab_s0[0], l), len = __builtin_amdgcn_readlane(tab_len[0], l);
+        int sl = __builtin_amdgcn_readlane(tab_slot[0], l);
+#pragma unroll
+        for (int k = 1; k < NTAB; ++k) {
+            const bool here = (cc >> 6) == k;
+            const int s0k = __builtin_amdgcn_readlane(tab_s0[k], l), lenk = __builtin_amdgcn_readlane(tab_len[k], l);
+            const int slk = __builtin_amdgcn_readlane(tab_slot[k], l);
+            s0 = here ? s0k : s0;
+            len = here ? lenk : len;
+            sl = here ? slk : sl;
+        }
+        const int a0 = row0 + s0;
+        // past the table, and for a chunk whose rows lie outside the operand,
+        // nothing is fetched: an empty resource delivers zeros
+        const bool real = (c < nchunks) & (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
+        const sp_int4 xq = raw_rsrc(xbase, real ? x_bytes : 0u);
+        const unsigned soff = real ? (unsigned)a0 * 4u : 0u;
+#pragma unroll
+        for (int it = 0; it < 3; ++it)
+            lds_load_b128(xq, buf + x_lds[it], x_off[it], soff);
+        const bool ok = real & (wave < len) & (sl >= 0);
+        const sp_int4 aq = raw_rsrc(vals, ok ? a_bytes : 0u);
+        const unsigned voff = (unsigned)(ashift ? arow + s0 + wave : arow) * 4u;
+        lds_load_b32(aq, buf + (unsigned)(SP_DAVALS + wave * SP_ROWS) * 4u, voff,
+                     ok ? (unsigned)sl * (unsigned)stride * 4u : 0u);
+    };
+    auto read_window = [&](SpWindow<LCK, T> &win, int b) {
+        const float *buf = lds[b];
+        spmm_read_window<LCK, T>(win, buf + lane * SP_DPITCH + wave * T, buf + SP_DAVALS + wave * T + (lane & (T - 1)));
+    };
+
+    SpWindow<LCK, T> w0, w1;
+    issue(0, lds0);
+    issue(1, lds0 + BUF_BYTES);
+    issue(2, lds0 + 2 * BUF_BYTES);
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");     // chunks 0 and 1 (and the destination values) are in
+    __syncthreads();
+    read_window(w0, 0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();                                     // every wave has its window(0): buffer 0 may be reused
+    // iteration c: buffers b (chunk c), b1 (chunk c+1), b2 (chunk c+2)
+    auto iteration = [&](int c, int b, int b1, SpWindow<LCK, T> &cur, SpWindow<LCK, T> &nxt) {
+        read_window(nxt, b1);
+        const bool more = c + 3 < nchunks;
+        if (more) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES);    // over chunk c, whose window every wave holds
+        spmm_rows<LCK, T, 0>(acc, cur);
+        // chunk c+2 must be in: everything but the 4 loads just issued
+        if (more) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+    int c = 0, b = 0, b1 = 1, b2 = 2;
+    if (nchunks & 1) {
+        iteration(0, b, b1, w0, w1);
+        { const SpWindow<LCK, T> t = w0; w0 = w1; w1 = t; }
+        { const int t = b; b = b1; b1 = b2; b2 = t; }
+        c = 1;
+    }
+    for (; c < nchunks; c += 2) {
+        iteration(c, b, b1, w0, w1);
+        iteration(c + 1, b1, b2, w1, w0);
+        { const int t0 = b, t1 = b1; b = b2; b1 = t0; b2 = t1; }
+    }
+    // (the last barrier came after every window read, and no load is in flight)
+    float *out = &lds[0][0];
+#pragma unroll
+    for (int t = 0; t < T; ++t) out[lane * SP_OPITCH + wave * T + t] = acc[t];
+    __syncthreads();
+    const long long row = (long long)row0 + lane;
+    if (row < n_out) {
+        const float bias = (EP && ep.bias) ? ep.bias[row] : 0.f;
+        float v[CPW];
+#pragma unroll
+        for (int q = 0; q < CPW; ++q) v[q] = out[(wave * CPW + q) * SP_OPITCH + lane];   // all reads before the first store
+#pragma unroll
+        for (int q = 0; q < CPW; ++q) {
+            const int col = wave * CPW + q;
+            if (col0 + col < batch) {
+                float *y = Y + (long long)(col0 + col) * ldy + row;
+                const float r = (beta == 0.f) ? alpha * v[q] : beta * ypre[q] + alpha * v[q];
                 *y = EP ? sp_finish(r, bias, ep.act) : r;
             }
         }
@@ -598,7 +760,9 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes,
     int s_min, int s_max, SpEpilogue ep)
 {
-    __shared__ __attribute__((aligned(16))) float lds[2][SP_STAGE_FLOATS];
+    static_assert(3 * SP_DSTAGE_FLOATS >= 2 * SP_STAGE_FLOATS, "the two bodies share one LDS block");
+    __shared__ __attribute__((aligned(16))) float lds3[3][SP_DSTAGE_FLOATS];
+    float (&lds)[2][SP_STAGE_FLOATS] = *reinterpret_cast<float (*)[2][SP_STAGE_FLOATS]>(&lds3[0][0]);
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
     const int rowtile = tile / col_tiles;
     const int row0 = rowtile * SP_ROWS;
@@ -610,7 +774,8 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     bool lean = row0 + SP_ROWS <= n_out;
     int c_lo = 0, c_hi = nchunks;                   // the chunks whose rows lie inside the operand: a contiguous
                                                     // range, the table being sorted by shift
-    if (!((row0 + s_min >= 0) & (row0 + s_max + 4 * SP_QUADS <= n_in))) {
+    constexpr int STAGED = 4 * SP_DQUADS;           // rows the lean body stages per chunk
+    if (!((row0 + s_min >= 0) & (row0 + s_max + STAGED <= n_in))) {
         const int lane = threadIdx.x & 63;
         c_lo = nchunks;
         c_hi = 0;
@@ -618,8 +783,8 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
         for (int k = 0; k < NTAB; ++k) {
             const int idx = 64 * k + lane;
             const int a0 = row0 + chunks[min(idx, nchunks - 1)].s0;
-            const bool inside = (a0 >= 0) & (a0 + 4 * SP_QUADS <= n_in);
-            const bool outside = (a0 + 4 * SP_QUADS <= 0) | (a0 >= n_in);
+            const bool inside = (a0 >= 0) & (a0 + STAGED <= n_in);
+            const bool outside = (a0 + STAGED <= 0) | (a0 >= n_in);
             lean &= __builtin_amdgcn_ballot_w64(!(inside | outside)) == 0;
             const unsigned long long m = __builtin_amdgcn_ballot_w64(inside & (idx < nchunks));
             if (m) {
@@ -634,11 +799,11 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     }
     if (lean)
         // only the chunks inside the operand are walked; the others would add zeros
-        spmm_tile<LCK, T, NTAB, false, EP>(lds, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
-                                           Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
+        spmm_tile_lean<LCK, NTAB, EP>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
+                                      Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
     else
-        spmm_tile<LCK, T, NTAB, true, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
-                                n_out, n_in, batch, alpha, beta, a_bytes, ep);
+        spmm_tile_edge<LCK, T, NTAB, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+                                         n_out, n_in, batch, alpha, beta, a_bytes, ep);
 }
 
 // ------------------------------------------------------------ tiled dd2dia --
