@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libcuvdia.so")
 
 OK = 0
 EINVAL, ESHAPE, EHIP, ENOMEM, EUNSUPPORTED, ENODEVICE = -1, -2, -3, -4, -5, -6
-ACT_NONE, ACT_SIGMOID = 0, 1
+ACT_NONE, ACT_SIGMOID, ACT_SIGMOID_SAMPLE = 0, 1, 2
 PATH_AUTO, PATH_GENERIC, PATH_TILED = 0, 1, 2
 
 _lib = None
@@ -52,6 +52,9 @@ def lib():
     L.cuvdia_spmm_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp]
     L.cuvdia_spmm_bias_act_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp, c_int,
                                            c_vp]
+    L.cuvdia_spmm_layer_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp, c_int,
+                                        ctypes.c_ulonglong, c_vp]
+    L.cuvdia_learn_step_weight_decay_f32.argtypes = [c_vp, c_vp, c_ll, c_f, c_f, c_vp]
     L.cuvdia_dd2dia_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_f, c_f, c_vp]
     L.cuvdia_avg_diagonals_f32.argtypes = [c_vp, c_vp, c_vp, c_vp]
     L.cuvdia_spmm_offsets_f32.argtypes = [c_vp, ip, c_int, c_int, c_int, c_int, c_int, c_vp, c_ll,
@@ -60,7 +63,9 @@ def lib():
                                             c_vp, c_ll, c_int, c_f, c_f, c_vp]
     for name in ("cuvdia_set_path", "cuvdia_plan_chunks", "cuvdia_desc_create", "cuvdia_desc_destroy",
                  "cuvdia_desc_info", "cuvdia_spmm_f32", "cuvdia_dd2dia_f32", "cuvdia_spmm_offsets_f32",
-                 "cuvdia_dd2dia_offsets_f32", "cuvdia_cache_clear"):
+                 "cuvdia_dd2dia_offsets_f32", "cuvdia_cache_clear", "cuvdia_spmm_bias_act_f32",
+                 "cuvdia_spmm_layer_f32", "cuvdia_learn_step_weight_decay_f32", "cuvdia_avg_diagonals_f32",
+                 "cuvdia_plan_units"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

@@ -61,6 +61,19 @@ int check_device(const cuvdia_desc *desc)
     return device == desc->device ? CUVDIA_OK : CUVDIA_EINVAL;
 }
 
+// For the entry points that take no descriptor: a device must be there.
+int require_device()
+{
+    int ndev = 0;
+    const hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev < 1) {
+        t_hip_error = std::string("hipGetDeviceCount: ") + hipGetErrorString(e);
+        (void)hipGetLastError();
+        return CUVDIA_ENODEVICE;
+    }
+    return CUVDIA_OK;
+}
+
 int validate_shape(const int *offsets, int nd, int h, int w, int stride, int rf)
 {
     if (!offsets || nd < 1 || h < 1 || w < 1 || rf < 1 || stride < 1) return CUVDIA_EINVAL;
@@ -253,12 +266,13 @@ int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t, long
     return CUVDIA_OK;
 }
 
-int cuvdia_spmm_bias_act_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
-                             float *dst, long long ldd, int batch, char transA,
-                             float alpha, float beta, const float *bias, int act, void *stream)
+int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
+                          float *dst, long long ldd, int batch, char transA,
+                          float alpha, float beta, const float *bias, int act,
+                          unsigned long long seed, void *stream)
 {
-    if (act != CUVDIA_ACT_NONE && act != CUVDIA_ACT_SIGMOID) return CUVDIA_EINVAL;
-    const SpEpilogue ep{bias, act};
+    if (act != CUVDIA_ACT_NONE && act != CUVDIA_ACT_SIGMOID && act != CUVDIA_ACT_SIGMOID_SAMPLE) return CUVDIA_EINVAL;
+    const SpEpilogue ep{bias, act, (unsigned)(seed & 0xffffffffull), (unsigned)(seed >> 32)};
     if (!desc || !A_vals || batch < 0) return CUVDIA_EINVAL;
     // make_spmv_header.pl:121-123: anything but 'n' / 't' is an error
     if (transA != 'n' && transA != 't') return CUVDIA_EINVAL;
@@ -287,6 +301,27 @@ int cuvdia_spmm_bias_act_f32(const cuvdia_desc *desc, const float *A_vals, const
         : launch_spmm_generic(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s);
     t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "spmm kernel launch");
+}
+
+int cuvdia_spmm_bias_act_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
+                             float *dst, long long ldd, int batch, char transA,
+                             float alpha, float beta, const float *bias, int act, void *stream)
+{
+    if (act == CUVDIA_ACT_SIGMOID_SAMPLE) return CUVDIA_EINVAL;      // sampling takes a seed: cuvdia_spmm_layer_f32
+    return cuvdia_spmm_layer_f32(desc, A_vals, B, ldb, dst, ldd, batch, transA, alpha, beta, bias, act, 0ull, stream);
+}
+
+int cuvdia_learn_step_weight_decay_f32(float *W, const float *dW, long long n, float learnrate, float decay,
+                                       void *stream)
+{
+    if (n < 0) return CUVDIA_EINVAL;
+    if (n == 0) return CUVDIA_OK;
+    if (!W || !dW) return CUVDIA_EINVAL;             // src/cuv/tensor_ops/rprop.cu:342-343
+    if (const int rc = require_device()) return rc;
+    // src/cuv/tensor_ops/rprop.cu:345: alpha = -learnrate, beta = 1 - learnrate*decay, both in fp32
+    const float alpha = -learnrate, beta = 1.f - learnrate * decay;
+    const hipError_t e = launch_axpby(W, dW, n, alpha, beta, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "learn_step_weight_decay kernel launch");
 }
 
 int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,

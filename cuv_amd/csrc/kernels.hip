@@ -61,12 +61,42 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy
+// as 1, 2, 3", SC'11): a counter-based generator, 4 x 32 random bits per
+// 128-bit counter and 64-bit key, no state.  The result element (row, col)
+// draws word col & 3 of the block with counter (row, col >> 2, 0, 0) and key
+// (seed_lo, seed_hi), so a sample depends on the seed and the element's
+// position only -- not on which kernel, tile or lane produced it.
+struct SpRand4 { unsigned w[4]; };
+__device__ __forceinline__ SpRand4 sp_philox(unsigned row, unsigned colblock, unsigned k0, unsigned k1)
+{
+    unsigned c0 = row, c1 = colblock, c2 = 0u, c3 = 0u;
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const unsigned hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const unsigned hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        c0 = hi1 ^ c1 ^ k0;
+        c1 = lo1;
+        c2 = hi0 ^ c3 ^ k1;
+        c3 = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return SpRand4{{c0, c1, c2, c3}};
+}
+// 24 random bits -> a uniform variate in [0, 1), exactly representable
+__device__ __forceinline__ float sp_uniform(unsigned word) { return (float)(word >> 8) * 0x1p-24f; }
+
 // Last step of an SpMM result element: optional per-row bias, optional
-// logistic sigmoid 1/(1+exp(-v)) (src/cuv/tensor_ops/functors.hpp:122).
-__device__ __forceinline__ float sp_finish(float v, float bias, int act)
+// logistic sigmoid 1/(1+exp(-v)) (src/cuv/tensor_ops/functors.hpp:122),
+// optional Bernoulli sample of that probability, v > u
+// (src/cuv/random/random.cu:86-91).
+__device__ __forceinline__ float sp_finish(float v, float bias, int act, unsigned word = 0u)
 {
     v += bias;
-    return act == 1 ? 1.f / (1.f + expf(-v)) : v;
+    if (act == 0) return v;
+    const float p = 1.f / (1.f + expf(-v));
+    return act == 2 ? (p > sp_uniform(word) ? 1.f : 0.f) : p;
 }
 
 // ------------------------------------------------------------------ generic --
@@ -125,7 +155,9 @@ __global__ __launch_bounds__(256) void spmm_generic_kernel(
         if (c0 + c < batch) {
             float *y = Y + (long long)(c0 + c) * ldy + o;
             const float v = (beta == 0.f) ? alpha * acc[c] : beta * (*y) + alpha * acc[c];
-            *y = sp_finish(v, ep.bias ? ep.bias[o] : 0.f, ep.act);
+            const unsigned col = (unsigned)(c0 + c);
+            const unsigned word = ep.act == 2 ? sp_philox((unsigned)o, col >> 2, ep.seed_lo, ep.seed_hi).w[col & 3u] : 0u;
+            *y = sp_finish(v, ep.bias ? ep.bias[o] : 0.f, ep.act, word);
         }
     }
 }
@@ -189,6 +221,42 @@ __global__ __launch_bounds__(AVG_THREADS) void avg_diagonals_kernel(
         __syncthreads();
     }
     if (t == 0) dst[d] = N > 0 ? part[0] / (float)N : 0.f;
+}
+
+// W[i] = alpha*dW[i] + beta*W[i]: the weight update that follows the
+// gradient (src/cuv/tensor_ops/rprop.cu:148-156).  Purely HBM-bound: 8 bytes
+// read and 4 written per element, 16-byte accesses once both arrays are
+// 16-byte aligned (the first elements up to that point, and the tail, go one
+// by one).
+constexpr int AXPBY_THREADS = 256;
+__global__ __launch_bounds__(AXPBY_THREADS) void axpby_kernel(
+    float *__restrict__ W, const float *__restrict__ dW, long long n, float alpha, float beta, int head, int vec)
+{
+    const long long tid = (long long)blockIdx.x * AXPBY_THREADS + threadIdx.x;
+    const long long nthreads = (long long)gridDim.x * AXPBY_THREADS;
+    if (!vec) {                                      // the arrays are misaligned against each other
+        for (long long i = tid; i < n; i += nthreads) W[i] = alpha * dW[i] + beta * W[i];
+        return;
+    }
+    // `head` (< 4) elements precede the first 16-byte boundary of both arrays
+    const long long nvec = (n - head) / 4;
+    float4 *W4 = reinterpret_cast<float4 *>(W + head);
+    const float4 *D4 = reinterpret_cast<const float4 *>(dW + head);
+    for (long long i = tid; i < nvec; i += nthreads) {
+        const float4 d = D4[i];
+        float4 w = W4[i];
+        w.x = alpha * d.x + beta * w.x;
+        w.y = alpha * d.y + beta * w.y;
+        w.z = alpha * d.z + beta * w.z;
+        w.w = alpha * d.w + beta * w.w;
+        W4[i] = w;
+    }
+    const long long rest = n - head - 4 * nvec;      // < 4
+    if (tid < head) W[tid] = alpha * dW[tid] + beta * W[tid];
+    if (tid < rest) {
+        const long long i = head + 4 * nvec + tid;
+        W[i] = alpha * dW[i] + beta * W[i];
+    }
 }
 
 // -------------------------------------------------------------- tiled spmm --
@@ -546,13 +614,20 @@ __device__ __forceinline__ void spmm_tile_edge(
         float v[SP_CPW];
 #pragma unroll
         for (int q = 0; q < SP_CPW; ++q) v[q] = out[(wave * SP_CPW + q) * SP_OPITCH + lane];   // all reads before the first store
+        // the lane's 8 columns are two aligned blocks of 4: two generator calls
+        SpRand4 rnd[SP_CPW / 4] = {};
+        if (EP && ep.act == 2) {
+#pragma unroll
+            for (int k = 0; k < SP_CPW / 4; ++k)
+                rnd[k] = sp_philox((unsigned)row, (unsigned)(col0 + wave * SP_CPW) / 4u + k, ep.seed_lo, ep.seed_hi);
+        }
 #pragma unroll
         for (int q = 0; q < SP_CPW; ++q) {
             const int col = wave * SP_CPW + q;
             if (col0 + col < batch) {
                 float *y = Y + (long long)(col0 + col) * ldy + row;
                 const float r = (beta == 0.f) ? alpha * v[q] : beta * ypre[q] + alpha * v[q];
-                *y = EP ? sp_finish(r, bias, ep.act) : r;
+                *y = EP ? sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]) : r;
             }
         }
     }
@@ -740,13 +815,20 @@ __device__ __forceinline__ void spmm_tile_lean(
         float v[CPW];
 #pragma unroll
         for (int q = 0; q < CPW; ++q) v[q] = out[(wave * CPW + q) * SP_OPITCH + lane];   // all reads before the first store
+        // the lane's 8 columns are two aligned blocks of 4: two generator calls
+        SpRand4 rnd[CPW / 4] = {};
+        if (EP && ep.act == 2) {
+#pragma unroll
+            for (int k = 0; k < CPW / 4; ++k)
+                rnd[k] = sp_philox((unsigned)row, (unsigned)(col0 + wave * CPW) / 4u + k, ep.seed_lo, ep.seed_hi);
+        }
 #pragma unroll
         for (int q = 0; q < CPW; ++q) {
             const int col = wave * CPW + q;
             if (col0 + col < batch) {
                 float *y = Y + (long long)(col0 + col) * ldy + row;
                 const float r = (beta == 0.f) ? alpha * v[q] : beta * ypre[q] + alpha * v[q];
-                *y = EP ? sp_finish(r, bias, ep.act) : r;
+                *y = EP ? sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]) : r;
             }
         }
     }
@@ -1250,6 +1332,21 @@ hipError_t launch_avg_diagonals(const DiaView &A, const float *vals, float *dst,
                            A.offsets_dev + done, vals + (long long)done * A.stride, A.stride, A.h, A.w, dst + done);
         done += slab;
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_axpby(float *W, const float *dW, long long n, float alpha, float beta, hipStream_t stream)
+{
+    if (n <= 0) return hipSuccess;
+    const unsigned long long wa = reinterpret_cast<unsigned long long>(W), da = reinterpret_cast<unsigned long long>(dW);
+    const bool vec = (wa & 15u) == (da & 15u) && (wa & 3u) == 0 && n >= 8;
+    const long long head = vec ? (long long)(((16u - (wa & 15u)) & 15u) / 4u) : 0;
+    const long long items = vec ? (n - head) / 4 : n;
+    long long blocks = (items + AXPBY_THREADS - 1) / AXPBY_THREADS;
+    if (blocks > 256 * 16) blocks = 256 * 16;         // 16 workgroups per CU, grid-stride beyond that
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(axpby_kernel, dim3((unsigned)blocks), dim3(AXPBY_THREADS), 0, stream, W, dW, n, alpha, beta,
+                       (int)head, (int)vec);
     return hipGetLastError();
 }
 

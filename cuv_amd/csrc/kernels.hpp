@@ -25,10 +25,13 @@ struct DiaView {
 
 // What the SpMM kernels do to a result element before storing it:
 // v = beta*dst + alpha*sum; v += bias[row] (bias != nullptr); v = 1/(1+exp(-v))
-// (act == 1).  The default, {nullptr, 0}, stores the plain product.
+// (act >= 1); v = v > u(row, col) ? 1 : 0 (act == 2), u being the uniform
+// variate in [0, 1) that sp_uniform() derives from (seed, row, col) with
+// Philox4x32-10.  The default, {nullptr, 0, 0, 0}, stores the plain product.
 struct SpEpilogue {
     const float *bias;   // one value per output row, on the device, or nullptr
-    int act;             // 0: none, 1: logistic sigmoid
+    int act;             // 0: none, 1: logistic sigmoid, 2: sigmoid, then a Bernoulli sample of it
+    unsigned seed_lo, seed_hi;
 };
 
 // dst = beta*dst + alpha*op(A)*B.  One thread per output row, a few batch
@@ -44,6 +47,9 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, SpEpilogue ep, hipStream_t stream);
+
+// W[i] = alpha*dW[i] + beta*W[i], i < n.
+hipError_t launch_axpby(float *W, const float *dW, long long n, float alpha, float beta, hipStream_t stream);
 
 // Whether the tiled SpMM can serve these operands (row_fact 1, operand extents
 // within its 32-bit buffer addressing).

@@ -125,9 +125,11 @@ def prod(dst, A, B, transA="n", transB="n", factAB=1.0, factC=0.0, sync=True):
     return dst
 
 
-def prod_bias_act(dst, A, B, transA="n", factAB=1.0, factC=0.0, bias=None, act=_lib.ACT_NONE, sync=True):
+def prod_bias_act(dst, A, B, transA="n", factAB=1.0, factC=0.0, bias=None, act=_lib.ACT_NONE, seed=0, sync=True):
     """dst = act(factC*dst + factAB*op(A)*B + bias[row]): prod, matrix_plus_col and the SIGM functor of an
-    RBM/MLP layer update in one launch (examples/rbm/base.py:48-54,127-136)."""
+    RBM/MLP layer update in one launch (examples/rbm/base.py:48-54,127-136).  act = ACT_SIGMOID_SAMPLE also
+    replaces each probability by a Bernoulli sample of it (rnd_binarize, src/cuv/random/random.cu:139-142),
+    drawn from Philox4x32-10 keyed by `seed` and the element's (row, column)."""
     if transA not in ("n", "t"):
         raise RuntimeError("transA must be 'n' or 't'")
     n_out, n_in = (A.w, A.h) if transA == "t" else (A.h, A.w)
@@ -139,9 +141,10 @@ def prod_bias_act(dst, A, B, transA="n", factAB=1.0, factC=0.0, bias=None, act=_
                                  and bias.is_contiguous() and bias.numel() == n_out):
         raise RuntimeError("A.shape()[0] == v.size()")
     with torch.cuda.device(dst.device):
-        _lib.check(_lib.lib().cuvdia_spmm_bias_act_f32(
+        _lib.check(_lib.lib().cuvdia_spmm_layer_f32(
             A.desc, A.vec.data_ptr(), B.data_ptr(), ldb, dst.data_ptr(), ldd, bb, transA.encode(), factAB, factC,
-            bias.data_ptr() if bias is not None else None, act, _stream_ptr()), "cuvdia_spmm_bias_act_f32")
+            bias.data_ptr() if bias is not None else None, act, int(seed) & 0xFFFFFFFFFFFFFFFF, _stream_ptr()),
+            "cuvdia_spmm_layer_f32")
         if sync:
             torch.cuda.current_stream().synchronize()
     return dst
@@ -177,6 +180,25 @@ def avg_diagonals(dst, A, sync=True):
         if sync:
             torch.cuda.current_stream().synchronize()
     return dst
+
+
+def learn_step_weight_decay(W, dW, learnrate, decay=0.0, sync=True):
+    """W = -learnrate*dW + (1 - learnrate*decay)*W (src/cuv/tensor_ops/rprop.cu:341-346).  W, dW: dev_dia_matrix_f
+    (the whole value vector is updated, as the reference's call on dia.vec() does) or float32 CUDA tensors."""
+    w = W.vec if isinstance(W, dev_dia_matrix_f) else W
+    d = dW.vec if isinstance(dW, dev_dia_matrix_f) else dW
+    for t in (w, d):
+        if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+            raise RuntimeError("W.ptr() / dW.ptr(): contiguous float32 CUDA tensors")
+    if w.numel() != d.numel():
+        raise RuntimeError("W.size() == dW.size()")
+    with torch.cuda.device(w.device):
+        _lib.check(_lib.lib().cuvdia_learn_step_weight_decay_f32(w.data_ptr(), d.data_ptr(), w.numel(),
+                                                                 learnrate, decay, _stream_ptr()),
+                   "cuvdia_learn_step_weight_decay_f32")
+        if sync:
+            torch.cuda.current_stream().synchronize()
+    return W
 
 
 def to_device_colmajor(a, device="cuda:0"):

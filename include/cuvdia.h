@@ -52,6 +52,7 @@ extern "C" {
 /* Activation applied by cuvdia_spmm_bias_act_f32. */
 #define CUVDIA_ACT_NONE      0
 #define CUVDIA_ACT_SIGMOID   1  /* 1 / (1 + exp(-x)), src/cuv/tensor_ops/functors.hpp:122 */
+#define CUVDIA_ACT_SIGMOID_SAMPLE 2  /* the sigmoid, then a Bernoulli sample of it (cuvdia_spmm_layer_f32 only) */
 
 /* Opaque description of one diagonal pattern: shape, offset table, and the
  * device-resident run table the tiled kernels walk.  Replaces the contents of
@@ -128,6 +129,40 @@ int cuvdia_spmm_bias_act_f32(const cuvdia_desc *desc, const float *A_vals_device
                              float *dst_device, long long ldd, int batch,
                              char transA, float alpha, float beta,
                              const float *bias_device, int act, void *stream);
+
+/* The layer update with a Bernoulli sample of the result:
+ *   p = 1/(1+exp(-(beta*dst + alpha*op(A)*B + bias[row]))),
+ *   dst = p > u(row, col) ? 1 : 0                    (act == CUVDIA_ACT_SIGMOID_SAMPLE)
+ * -- prod, matrix_plus_col, SIGM and rnd_binarize (src/cuv/random/random.cu:86-91,
+ * 139-142: f > uniform) of examples/rbm/base.py:48-54,94-99,127-136 in one
+ * launch.  The reference draws u from cuRAND's per-thread XORWOW states (a
+ * closed third-party generator whose stream depends on the launch shape);
+ * here u(row, col) = (w >> 8) * 2^-24 with w = word (col & 3) of
+ * Philox4x32-10 (Salmon et al., SC'11) at counter (row, col >> 2, 0, 0) and
+ * key (seed & 0xffffffff, seed >> 32): a function of the seed and the
+ * element's position in dst only, so results do not depend on the kernel
+ * family or the tiling.  row, col index dst (0-based).  With CUVDIA_ACT_NONE or
+ * CUVDIA_ACT_SIGMOID this is cuvdia_spmm_bias_act_f32 and the seed is unused.
+ * No counterpart with this signature exists in the reference. */
+int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals_device,
+                          const float *B_device, long long ldb,
+                          float *dst_device, long long ldd, int batch,
+                          char transA, float alpha, float beta,
+                          const float *bias_device, int act,
+                          unsigned long long seed, void *stream);
+
+/* W[i] = -learnrate*dW[i] + (1 - learnrate*decay)*W[i] for i < n: replaces
+ * learn_step_weight_decay<float,dev_memory_space>
+ * (src/cuv/tensor_ops/rprop.cu:148-156,324-346, declared in
+ * src/cuv/tensor_ops/rprop.hpp:127-128; the reference ignores sparsedecay,
+ * rprop.cu:153-154).  For a DIA weight matrix W and dW are the value vectors
+ * (num_dia*stride floats, padding included, as the reference's call on
+ * dia.vec() does).  W and dW must not overlap.  n == 0 is a no-op.
+ * When dW is itself a projected product, cuvdia_dd2dia_f32 with
+ * alpha = -learnrate*scale and beta = 1 - learnrate*decay applies the same
+ * update without materialising dW. */
+int cuvdia_learn_step_weight_decay_f32(float *W_device, const float *dW_device, long long n,
+                                       float learnrate, float decay, void *stream);
 
 /* C = beta*C + alpha*proj(A*B') restricted to the stored diagonals of C:
  *   C_d[i] = beta*C_d[i] + alpha * sum_c A[i,c] * B[offsets[d] + i/row_fact, c]

@@ -97,6 +97,22 @@ inline void avg_diagonals(tensor<float, host_memory_space> &dst, const dia_matri
     cuvAssert(rc == 0);
 }
 
+// W = -learnrate*dW + (1 - learnrate*decay)*W, element by element in fp32
+// (src/cuv/tensor_ops/rprop.cu:331-346).
+template <class L>
+inline void learn_step_weight_decay(tensor<float, host_memory_space, L> &W, const tensor<float, host_memory_space, L> &dW,
+                                    const float &learnrate, const float &decay = 0.0f, const float &sparsedecay = 0.0f)
+{
+    (void)sparsedecay;
+    cuvAssert(dW.ptr());
+    cuvAssert(W.ptr());
+    cuvAssert(W.size() == dW.size());
+    const float alpha = -learnrate, beta = 1.f - learnrate * decay;
+    float *w = W.ptr();
+    const float *d = dW.ptr();
+    for (size_t i = 0; i < (size_t)W.size(); ++i) w[i] = alpha * d[i] + beta * w[i];
+}
+
 // Dense C = factC*C + factAB*op(A)*op(B), fp64 accumulation: stands in for the
 // CBLAS sgemm the reference cross-checks against (src/cuv/matrix_ops/matrix_ops.cu:177-304).
 inline void prod(tensor<float, host_memory_space, column_major> &dst,

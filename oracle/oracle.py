@@ -215,6 +215,55 @@ def prod_bias_act(dia, B, dst=None, trans="n", alpha=1.0, beta=0.0, bias=None, s
     return np.asfortranarray(out)
 
 
+def philox4x32_10(counter, key):
+    """Philox4x32-10 of Salmon, Moraes, Dror and Shaw ("Parallel random numbers: as easy as 1, 2, 3", SC'11;
+    Random123 1.x, philox.h): counter (..., 4) and key (..., 2) uint32 arrays -> (..., 4) uint32.  The
+    algorithm lives in no reference file (the reference samples with cuRAND's XORWOW states,
+    src/cuv/random/random.cu:86-91); it is pinned by the known-answer vectors Random123 publishes."""
+    c = [np.asarray(counter[..., i], dtype=np.uint64) for i in range(4)]
+    k0 = np.asarray(key[..., 0], dtype=np.uint64)
+    k1 = np.asarray(key[..., 1], dtype=np.uint64)
+    m0, m1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+    mask = np.uint64(0xFFFFFFFF)
+    sh = np.uint64(32)
+    for _ in range(10):
+        p0 = m0 * c[0]
+        p1 = m1 * c[2]
+        c = [(p1 >> sh) ^ c[1] ^ k0, p1 & mask, (p0 >> sh) ^ c[3] ^ k1, p0 & mask]
+        k0 = (k0 + np.uint64(0x9E3779B9)) & mask
+        k1 = (k1 + np.uint64(0xBB67AE85)) & mask
+    return np.stack(c, axis=-1).astype(np.uint32)
+
+
+def sample_uniform(n_rows, n_cols, seed):
+    """u(row, col) in [0, 1): 24 bits of word (col & 3) of the Philox block at counter (row, col >> 2, 0, 0),
+    key (seed & 0xffffffff, seed >> 32) -- the draw the fused layer update documents in its header."""
+    rows, cols = np.meshgrid(np.arange(n_rows, dtype=np.uint32), np.arange(n_cols, dtype=np.uint32), indexing="ij")
+    ctr = np.stack([rows, cols >> 2, np.zeros_like(rows), np.zeros_like(rows)], axis=-1)
+    key = np.empty(rows.shape + (2,), np.uint32)
+    key[..., 0] = seed & 0xFFFFFFFF
+    key[..., 1] = (seed >> 32) & 0xFFFFFFFF
+    words = philox4x32_10(ctr, key)
+    w = np.take_along_axis(words, (cols & 3)[..., None].astype(np.int64), axis=-1)[..., 0]
+    return ((w >> 8).astype(np.float32) * np.float32(2.0 ** -24)).astype(np.float32)
+
+
+def rnd_binarize(p, u):
+    """src/cuv/random/random.cu:86-91: f > uniform, as 0 / 1 floats."""
+    return np.asfortranarray((np.asarray(p, np.float32) > np.asarray(u, np.float32)).astype(np.float32))
+
+
+def learn_step_weight_decay(W, dW, learnrate, decay=0.0):
+    """src/cuv/tensor_ops/rprop.cu:331-346: W[i] = alpha*dW[i] + beta*W[i] with alpha = -learnrate and
+    beta = 1 - learnrate*decay, every operation rounded to fp32 (sparsedecay is ignored there too)."""
+    lr, dc = np.float32(learnrate), np.float32(decay)
+    alpha = np.float32(-lr)
+    beta = np.float32(np.float32(1) - np.float32(lr * dc))
+    W = np.asarray(W, np.float32)
+    dW = np.asarray(dW, np.float32)
+    return (np.float32(alpha) * dW).astype(np.float32) + (np.float32(beta) * W).astype(np.float32)
+
+
 def avg_diagonals(dia):
     out = np.zeros(dia.nd, np.float32)
     lib().oracle_avg_diagonals_f32(dia.h, dia.w, dia.nd, dia.stride,

@@ -155,6 +155,33 @@ TEST_CASE(avg_diagonals_dev)
     CHECK_THROWS(avg_diagonals(wrong, wd));
 }
 
+// The weight update of examples/rbm/base.py:71 on a DIA layer's value vector:
+// with learnrate 0.5, decay 0.25 and sequence() data (W = i, dW = i) every
+// product is exact: W' = -0.5 i + 0.875 i = 0.375 i.
+TEST_CASE(learn_step_weight_decay_dev)
+{
+    dia_matrix<float, host_memory_space> w(32, 16, 7, 32, 1), dw(32, 16, 7, 32, 1);
+    std::vector<int> off;
+    for (int i = -3; i <= 3; ++i) off.push_back(i);
+    w.set_offsets(off);
+    dw.set_offsets(off);
+    sequence(w.vec());
+    sequence(dw.vec());
+    dia_matrix<float, dev_memory_space> wd(32, 16, 7, 32, 1), dwd(32, 16, 7, 32, 1);
+    convert(wd, w);
+    convert(dwd, dw);
+    learn_step_weight_decay(wd.vec(), dwd.vec(), 0.5f, 0.25f);
+    learn_step_weight_decay(w.vec(), dw.vec(), 0.5f, 0.25f);
+    dia_matrix<float, host_memory_space> back(32, 16, 7, 32, 1);
+    convert(back, wd);
+    for (unsigned i = 0; i < w.vec().size(); ++i) {
+        CHECK(back.vec()[i] == 0.375f * i);
+        CHECK(back.vec()[i] == w.vec()[i]);
+    }
+    tensor<float, dev_memory_space> shorter(5);
+    CHECK_THROWS(learn_step_weight_decay(wd.vec(), shorter, 0.5f));
+}
+
 TEST_CASE(spmv_uninit)
 {
     dia_matrix<float, host_memory_space> w(32, 16, 3, 32, 1);

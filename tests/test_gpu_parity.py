@@ -511,3 +511,136 @@ def test_prod_bias_sigmoid(oracle, gu, h, w, offs, batch, trans):
                                                       float((np.abs(got - ref) / tol).max()))
             if act:
                 assert got.min() >= 0.0 and got.max() <= 1.0
+
+
+# ------------------------------------- prod + bias + sigmoid + Bernoulli sample ---
+@pytest.mark.parametrize("trans", ["n", "t"])
+@pytest.mark.parametrize("h,w,offs,batch", [
+    (32, 16, [-3, -2, -1, 0, 1, 2, 3], 6),
+    (700, 650, [d * 25 + e for d in range(-2, 3) for e in range(-2, 3)], 96),
+    (1024, 1024, [dy * 32 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 130),
+])
+def test_prod_bias_sigmoid_sample(oracle, gu, h, w, offs, batch, trans):
+    """The fused layer update with sampling: dst = (p > u) with p the sigmoid of
+    the biased product and u(row, col) the documented Philox4x32-10 draw.  The
+    oracle applies rnd_binarize's rule (f > uniform) to its own p and the same
+    u.  Both kernel families must give the oracle's bits wherever the two
+    sides' p cannot straddle u (|p_ref - u| above the tolerance of the
+    non-sampled test); elsewhere either value is right.  The seed must matter
+    and the sample mean must follow the mean probability."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(7 * h + w + batch)
+    A = _rand_dia(oracle, rng, h, w, offs, 1)
+    n_in, n_out = (h, w) if trans == "t" else (w, h)
+    B = np.asfortranarray(rng.uniform(-1, 1, (n_in, batch)).astype(np.float32))
+    bias = rng.uniform(-1, 1, n_out).astype(np.float32)
+    dev = gu.make_dev_dia(A)
+    Bd = D.to_device_colmajor(B)
+    bd = torch.from_numpy(bias).cuda()
+    p_ref = oracle.prod_bias_act(A, B, None, trans, 1.0, 0.0, bias, True)
+    mag = oracle.prod_mag(A, B, None, trans, 1.0, 0.0) + np.abs(bias)[:, None]
+    tol = 0.25e-5 * mag + 4e-7
+    results = {}
+    for seed in (0, 0x9E3779B97F4A7C15):
+        u = oracle.sample_uniform(n_out, batch, seed)
+        ref = oracle.rnd_binarize(p_ref, u)
+        decided = np.abs(p_ref.astype(np.float64) - u) > tol
+        assert decided.mean() > 0.999
+        for path in (_lib.PATH_GENERIC, _lib.PATH_TILED):
+            dd = torch.full((batch, n_out), float("nan"), device="cuda:0")
+            _lib.check(L.cuvdia_set_path(path), "set_path")
+            try:
+                D.prod_bias_act(dd, dev, Bd, trans, 1.0, 0.0, bd, _lib.ACT_SIGMOID_SAMPLE, seed=seed)
+                assert L.cuvdia_last_path() == path
+            finally:
+                L.cuvdia_set_path(_lib.PATH_AUTO)
+            got = D.to_host_colmajor(dd)
+            assert np.all((got == 0.0) | (got == 1.0))
+            assert np.array_equal(got[decided], ref[decided]), (path, seed, int((got != ref)[decided].sum()))
+            results[(seed, path)] = got
+        assert abs(float(ref.mean()) - float(p_ref.mean())) < 4.0 / np.sqrt(ref.size) + 1e-3
+    assert not np.array_equal(results[(0, _lib.PATH_TILED)], results[(0x9E3779B97F4A7C15, _lib.PATH_TILED)])
+    # the plain entry point takes no seed and refuses the sampling activation
+    dd = torch.zeros((batch, n_out), device="cuda:0")
+    rc = L.cuvdia_spmm_bias_act_f32(dev.desc, dev.vec.data_ptr(), Bd.data_ptr(), n_in, dd.data_ptr(), n_out, batch,
+                                    trans.encode(), 1.0, 0.0, None, _lib.ACT_SIGMOID_SAMPLE, None)
+    assert rc == _lib.EINVAL
+
+
+# ------------------------------------------------ learn_step_weight_decay ---
+@pytest.mark.parametrize("n,shift_w,shift_d", [(1, 0, 0), (7, 0, 0), (4096, 0, 0), (100003, 1, 1), (100003, 3, 2),
+                                               (49 * 16384, 0, 0)])
+def test_learn_step_weight_decay(oracle, n, shift_w, shift_d):
+    """W = -lr*dW + (1 - lr*decay)*W (rprop.cu:341-346) against the fp32 host
+    restatement; the GPU contracts alpha*dW + (beta*W) into one FMA, which
+    moves a result by at most one rounding of the product: tolerance
+    1e-6 * (|alpha*dW| + |beta*W|).  Aligned, equally misaligned and mutually
+    misaligned arrays; elements around the arrays must stay untouched."""
+    import torch
+    from cuv_amd import dia as D
+    rng = np.random.default_rng(n + shift_w)
+    W = rng.normal(0, 0.01, n).astype(np.float32)
+    dW = rng.normal(0, 1.0, n).astype(np.float32)
+    lr, decay = 0.05, 0.002
+    ref = oracle.learn_step_weight_decay(W, dW, lr, decay)
+    bufw = torch.full((n + 16,), 123.0, device="cuda:0")
+    bufd = torch.full((n + 16,), -7.0, device="cuda:0")
+    wv = bufw[4 + shift_w:4 + shift_w + n]
+    dv = bufd[4 + shift_d:4 + shift_d + n]
+    wv.copy_(torch.from_numpy(W))
+    dv.copy_(torch.from_numpy(dW))
+    D.learn_step_weight_decay(wv, dv, lr, decay)
+    got = wv.cpu().numpy()
+    tol = 1e-6 * (np.abs(lr * dW.astype(np.float64)) + np.abs(W.astype(np.float64))) + 1e-30
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= tol), float((np.abs(got - ref) / tol).max())
+    host = bufw.cpu().numpy()
+    assert np.all(host[:4 + shift_w] == 123.0) and np.all(host[4 + shift_w + n:] == 123.0)
+    assert np.array_equal(dv.cpu().numpy(), dW)
+
+
+def test_weight_update_fused_into_the_projection(oracle, gu):
+    """examples/rbm/base.py:71-81: w_tmp = proj(v0*h0') ; w_tmp = -1/b*proj(v1*h1') + 1/b*w_tmp ;
+    W = -lr*w_tmp + (1 - lr*cost)*W.  The same update in two projection calls
+    and no w_tmp: W = (1 - lr*cost)*W + (-lr/b)*proj(v0*h0') ; W = W + (lr/b)*proj(v1*h1').
+    Both sequences round differently; they must agree within 1e-5 of the
+    magnitudes involved."""
+    import torch
+    from cuv_amd import dia as D
+    rng = np.random.default_rng(99)
+    h = w = 1024
+    offs = [dy * 32 + dx for dy in range(-3, 4) for dx in range(-3, 4)]
+    b = 64
+    W0 = _rand_dia(oracle, rng, h, w, offs, 1)
+    v0 = np.asfortranarray((rng.uniform(0, 1, (h, b)) < 0.5).astype(np.float32))
+    h0 = np.asfortranarray(rng.uniform(0, 1, (w, b)).astype(np.float32))
+    v1 = np.asfortranarray(rng.uniform(0, 1, (h, b)).astype(np.float32))
+    h1 = np.asfortranarray(rng.uniform(0, 1, (w, b)).astype(np.float32))
+    lr, cost = 0.1, 0.01
+    v0d, h0d, v1d, h1d = (D.to_device_colmajor(x) for x in (v0, h0, v1, h1))
+    # the reference's three steps, on the device
+    Wa = gu.make_dev_dia(W0)
+    tmp = gu.make_dev_dia(W0)
+    bd = D.dev_block_descriptor_f(tmp)
+    D.densedense_to_dia(tmp, bd, v0d, h0d, 1.0, 0.0)
+    D.densedense_to_dia(tmp, bd, v1d, h1d, -1.0 / b, 1.0 / b)
+    D.learn_step_weight_decay(Wa, tmp, lr, cost)
+    # fused
+    Wb = gu.make_dev_dia(W0)
+    bdb = D.dev_block_descriptor_f(Wb)
+    D.densedense_to_dia(Wb, bdb, v0d, h0d, -lr / b, 1.0 - lr * cost)
+    D.densedense_to_dia(Wb, bdb, v1d, h1d, lr / b, 1.0)
+    a = Wa.vec.cpu().numpy().astype(np.float64)
+    c = Wb.vec.cpu().numpy().astype(np.float64)
+    mask = oracle.valid_mask(W0).reshape(-1)
+    g0 = np.abs(oracle.dd2dia_f64(W0, v0, h0, 1.0, 0.0)).reshape(-1)
+    g1 = np.abs(oracle.dd2dia_f64(W0, v1, h1, 1.0, 0.0)).reshape(-1)
+    mag = np.abs(W0.vals.astype(np.float64)) + lr / b * (g0 + g1)
+    assert np.all(np.abs(a - c)[mask] <= 1e-5 * mag[mask] + 1e-30), float((np.abs(a - c)[mask] / (1e-5 * mag[mask] + 1e-30)).max())
+    # and against the oracle's three host steps
+    t = oracle.dd2dia(W0, v0, h0, 1.0, 0.0)
+    T = oracle.Dia(h, w, offs, vals=t)
+    t = oracle.dd2dia(T, v1, h1, -1.0 / b, 1.0 / b)
+    ref = oracle.learn_step_weight_decay(W0.vals, t.reshape(-1), lr, cost).astype(np.float64)
+    assert np.all(np.abs(a - ref)[mask] <= 1e-5 * mag[mask] + 1e-30)

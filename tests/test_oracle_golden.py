@@ -279,3 +279,44 @@ def test_workload_counts_match_published_table():
     q = W.pattern_large()
     assert q.nd == 676 and q.nnz == 110616022
     assert W.spmm_bytes(q, 256, "n", 0.0) == 979337704
+
+
+# ----------------------------------------------------------- Philox sampling ---
+def test_philox_known_answers(oracle):
+    """Random123's published known-answer vectors for philox4x32-10 (kat_vectors:
+    counter, key -> output)."""
+    kat = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+           ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+            (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kat:
+        got = oracle.philox4x32_10(np.array(ctr, np.uint32), np.array(key, np.uint32))
+        assert [int(x) for x in got] == list(want)
+
+
+def test_sample_uniform_indexing(oracle):
+    """u(row, col) takes word col & 3 of the block at counter (row, col >> 2, 0, 0)
+    -- checked element by element against single-block calls -- lies in [0, 1),
+    is a multiple of 2^-24 and is uniform enough for a 4-sigma test."""
+    seed = 0x0123456789ABCDEF
+    u = oracle.sample_uniform(9, 11, seed)
+    key = np.array([seed & 0xFFFFFFFF, seed >> 32], np.uint32)
+    for r in range(9):
+        for c in range(11):
+            blk = oracle.philox4x32_10(np.array([r, c >> 2, 0, 0], np.uint32), key)
+            assert u[r, c] == np.float32(int(blk[c & 3]) >> 8) * np.float32(2.0 ** -24)
+    big = oracle.sample_uniform(256, 256, 42)
+    assert big.min() >= 0.0 and big.max() < 1.0
+    assert np.all(big * 2 ** 24 == np.round(big * 2 ** 24))
+    assert abs(float(big.mean()) - 0.5) < 4 * (1 / np.sqrt(12)) / 256
+    assert np.array_equal(oracle.rnd_binarize(np.array([[0.5, 0.5]]), np.array([[0.25, 0.5]])), [[1.0, 0.0]])
+
+
+def test_learn_step_weight_decay_closed_form(oracle):
+    """rprop.cu:345: alpha = -learnrate, beta = 1 - learnrate*decay.  With
+    learnrate 0.5, decay 0.25, W = 8 i, dW = 2 i every product is exact:
+    W' = -i + 0.875 * 8 i = 6 i."""
+    i = np.arange(1000, dtype=np.float32)
+    got = oracle.learn_step_weight_decay(8 * i, 2 * i, 0.5, 0.25)
+    assert got.dtype == np.float32 and np.array_equal(got, 6 * i)
+    assert np.array_equal(oracle.learn_step_weight_decay(i, i, 0.0, 3.0), i)
