@@ -57,7 +57,9 @@ def parse():
     ap.add_argument("--workload", default="step",
                     help="'step' (default): cfg1 + cfg2 + cfg3, the configuration the metric is quoted on; "
                          "'cfg4': the large layer (262144 rows, 676 diagonals, batch 256), each product timed "
-                         "on its own -- an auxiliary line, no CPU leg (the oracle needs minutes for it)")
+                         "on its own -- an auxiliary line, no CPU leg (the oracle needs minutes for it); "
+                         "'layer': the steps either side of the products at cfg1's shape (fused bias + sigmoid "
+                         "(+ sample) against separate passes, the weight-decay step) -- an auxiliary line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
     return ap.parse_args()
@@ -137,6 +139,74 @@ def bench_cfg4(args, torch, D, W, dev):
         ops=res, aux=aux, note="bound by the fp32 vector rate (57 FLOP per algorithmic byte), not by HBM")))
 
 
+def bench_layer(args, torch, D, W, dev):
+    """What the fused layer update saves at cfg1's shape: the up-pass alone, with bias + sigmoid (+ Bernoulli
+    sample) in its store, and as the reference's separate passes over the activations (here torch's
+    element-wise kernels); and the weight-decay step on the value vector.  Warm timings from HIP graphs of 20
+    launches; parity of these operations is covered by tests/test_gpu_parity.py."""
+    from cuv_amd import _lib
+    w1 = W.cfg1()
+    p = w1.pattern
+    n, nd, batch = p.h, len(p.offsets), w1.batch
+    A = D.dev_dia_matrix_f(p.h, p.w, nd, p.stride, 1, device=dev)
+    A.set_offsets(p.offsets)
+    A.push(w1.vals)
+    G = D.dev_dia_matrix_f(p.h, p.w, nd, p.stride, 1, device=dev)
+    G.set_offsets(p.offsets)
+    G.push(w1.vals)
+    V = D.to_device_colmajor(w1.X)
+    H = torch.empty(batch, n, device=dev)
+    bias = torch.randn(n, device=dev)
+    A.desc
+
+    def timed(fn, n_rep=300):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(20):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n_rep // 20):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (n_rep // 20 * 20) * 1e3
+
+    def separate(sample):
+        D.prod(H, A, V, "n", "n", 1.0, 0.0, sync=False)
+        H.add_(bias)
+        torch.sigmoid_(H)
+        if sample:
+            H.copy_(torch.bernoulli(H))
+    step_bytes = 3 * 4 * nd * p.stride
+    us = {
+        "prod": timed(lambda: D.prod(H, A, V, "n", "n", 1.0, 0.0, sync=False)),
+        "prod_bias_sigmoid_fused": timed(lambda: D.prod_bias_act(H, A, V, "n", 1.0, 0.0, bias, _lib.ACT_SIGMOID,
+                                                                 sync=False)),
+        "prod_bias_sigmoid_sample_fused": timed(lambda: D.prod_bias_act(H, A, V, "n", 1.0, 0.0, bias,
+                                                                        _lib.ACT_SIGMOID_SAMPLE, seed=1, sync=False)),
+        "prod_then_bias_then_sigmoid": timed(lambda: separate(False)),
+        "prod_then_bias_then_sigmoid_then_sample": timed(lambda: separate(True)),
+        "learn_step_weight_decay": timed(lambda: D.learn_step_weight_decay(A, G, 0.01, 0.001, sync=False)),
+    }
+    lw = us["learn_step_weight_decay"]
+    print(json.dumps(dict(
+        metric="microseconds per launch, layer-update steps around the DIA products", unit="us",
+        value=us["prod_bias_sigmoid_fused"], n_gpus=1, steps=300, warmup=20, ms_per_step=us["prod_bias_sigmoid_fused"] * 1e-3,
+        higher_is_better=False, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
+        config=dict(workload="cfg1 shape (16384x16384 DIA, 49 diagonals, batch 128): up-pass with its bias, "
+                             "sigmoid and sampling fused or as separate passes; weight-decay step on the value vector",
+                    rows=n, diagonals=nd, batch=batch),
+        us=us, learn_step=dict(bytes=step_bytes, gbs=step_bytes / (lw * 1e-6) / 1e9,
+                               frac_hbm=step_bytes / (lw * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                               note="warm: the 6.4 MB working set stays in cache between launches"))))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -157,6 +227,8 @@ def main():
 
     if args.workload == "cfg4":
         return bench_cfg4(args, torch, D, W, dev)
+    if args.workload == "layer":
+        return bench_layer(args, torch, D, W, dev)
 
     w1, w2, w3 = W.cfg1(), W.cfg2(), W.cfg3()
     p = w1.pattern

@@ -154,3 +154,32 @@ def test_units_pairing_rule():
     assert _units([0, 1, 128, 129, 256]) == [(0, 1), (2, -1)]
     from cuv_amd import _lib
     assert _lib.lib().cuvdia_plan_units(None, 3, None, None, 0) == _lib.EINVAL
+
+
+# ------------------------------------------------------------------ file io ---
+def test_dia_file_round_trip(tmp_path):
+    """The seven fields of sparse_matrix_io.hpp:52-66, same names and order,
+    survive a save/load; malformed field sets are rejected with the
+    constructor's own conditions (dia_matrix.hpp:98-109,131)."""
+    from cuv_amd import io
+    rng = np.random.default_rng(5)
+    offs = np.array([0, 3, -2, 17], np.int32)
+    f = dict(m_width=20, m_height=33, m_num_dia=4, m_stride=33, m_row_fact=1, m_offsets=offs,
+             m_vec=rng.normal(size=4 * 33).astype(np.float32))
+    path = str(tmp_path / "w.npz")
+    io.save_fields(path, f)
+    with np.load(path) as z:
+        assert tuple(z.files) == io.FIELDS
+    g = io.load_fields(path)
+    assert tuple(g) == io.FIELDS
+    assert [int(g[k]) for k in io.FIELDS[:5]] == [20, 33, 4, 33, 1]
+    assert np.array_equal(g["m_offsets"], offs) and g["m_offsets"].dtype == np.int32
+    assert np.array_equal(g["m_vec"], f["m_vec"]) and g["m_vec"].dtype == np.float32
+    with pytest.raises(RuntimeError):
+        io.check_fields(dict(f, m_row_fact=0))
+    with pytest.raises(RuntimeError):
+        io.check_fields(dict(f, m_stride=19))
+    with pytest.raises(ValueError):
+        io.check_fields(dict(f, m_vec=f["m_vec"][:-1]))
+    with pytest.raises(ValueError):
+        io.check_fields({k: v for k, v in f.items() if k != "m_offsets"})
