@@ -637,7 +637,7 @@ __device__ __forceinline__ void spmm_tile_edge(
 }
 
 // Loads that deliver straight into LDS (no vector register in between): lane i
-// of the wave writes its 16 (4) bytes at lds_byte_addr + 16*i (4*i); an
+// of the wave writes its 16 bytes at lds_byte_addr + 16*i; an
 // out-of-range lane writes zeros, an inactive lane writes nothing.  They are
 // vector-memory operations and complete in order with the wave's other loads
 // (s_waitcnt vmcnt).  Written in assembly so that the waits below can be
@@ -656,13 +656,6 @@ __device__ __forceinline__ void lds_load_b128(sp_int4 rsrc, unsigned lds_byte_ad
                  "buffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
-__device__ __forceinline__ void lds_load_b32(sp_int4 rsrc, unsigned lds_byte_addr, unsigned voff, unsigned soff)
-{
-    asm volatile("s_mov_b32 m0, %0\n\t"
-                 "s_nop 0\n\t"
-                 "buffer_load_dword %1, %2, %3 offen lds"
-                 :: "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-}
 
 // The lean body (see spmm_tile) with the staging done by loads that write LDS
 // directly.  A chunk stages 76 rows (19 16-byte pieces) of each of the 64
@@ -671,23 +664,21 @@ __device__ __forceinline__ void lds_load_b32(sp_int4 rsrc, unsigned lds_byte_add
 // fetching piece 64 * i + l) fills bytes [1024 * i, 1024 * i + 1024) and 19
 // instructions, every lane busy, stage the chunk.  Columns are then 76 floats
 // apart, which keeps the 16-byte window reads (one lane per column) free of
-// bank conflicts.  Wave w issues instructions w, w + 8 and w + 16 (where that
-// is past the last one it asks for nothing and zeros drop into a spare
-// kilobyte, so every wave has the same number of loads in flight) and diagonal
-// w of the chunk: 4 loads per wave and chunk, none through registers, no LDS
-// write instruction.  Three LDS buffers: chunk k lives in buffer k % 3; while
-// the FMAs of chunk c run, window(c+1) is being read, chunk c+2 is landing and
-// chunk c+3 has just been requested.
+// bank conflicts.  Wave w issues instructions w, w + 8 and (waves 0-2)
+// w + 16; waves 3 and 4 fetch the chunk's 8 diagonals for the 64 rows, 4
+// diagonals per instruction: 21 loads per chunk, none through registers, no
+// LDS write instruction.  Three LDS buffers: chunk k lives in buffer k % 3;
+// while the FMAs of chunk c run, window(c+1) is being read, chunk c+2 is
+// landing and chunk c+3 has just been requested.
 constexpr int SP_DQUADS = 19;                       // pieces per column staged by the direct loads (76 rows)
 constexpr int SP_DPITCH = 4 * SP_DQUADS;            // floats between staged columns
 constexpr int SP_DAVALS = SP_COLS * SP_DPITCH;      // diagonal values sit behind the dense rows
-constexpr int SP_DSPARE = SP_DAVALS + SP_AVALS;     // 256 floats that idle load slots fill with zeros
-constexpr int SP_DSTAGE_FLOATS = SP_DSPARE + 256;
+constexpr int SP_DSTAGE_FLOATS = SP_DAVALS + SP_AVALS;
 static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + CHUNK_MAX - 1 <= SP_DPITCH, "staging layout");
 
 template <int LCK, int NTAB, bool EP>
 __device__ __forceinline__ void spmm_tile_lean(
-    float (&lds)[3][SP_DSTAGE_FLOATS], int row0, int col0,
+    float (&lds)[3][SP_DSTAGE_FLOATS], int *slot_tab, int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, SpEpilogue ep)
@@ -702,16 +693,33 @@ __device__ __forceinline__ void spmm_tile_lean(
     const unsigned x_bytes = (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4);
     const float *xbase = X + (long long)col0 * ldx;
 
+    // The result leaves in 16-byte stores, a lane holding 4 consecutive rows of
+    // 2 columns (column wave*8 + lane/16 and the one 4 further), except when
+    // samples are drawn: the generator yields 4 columns of one row per call,
+    // so then a lane keeps one row and 8 columns.  Where beta scales the old
+    // destination values they are requested now, in the same arrangement, and
+    // their trip from memory overlaps the whole product.
+    const bool by_row = EP && ep.act == 2;
+    const int ecol = wave * CPW + (lane >> 4), erow = 4 * (lane & 15);
     float ypre[CPW];
-    {
-        const long long row = (long long)row0 + lane;
-        const __amdgpu_buffer_rsrc_t yr = make_rsrc(
-            Y + (long long)col0 * ldy, beta != 0.f ? (unsigned)(((long long)(cols_here - 1) * ldy + n_out) * 4) : 0u);
 #pragma unroll
-        for (int q = 0; q < CPW; ++q) {
-            const int col = wave * CPW + q;
-            ypre[q] = buffer_load_f32(yr, (row < n_out && col < cols_here)
-                                              ? (unsigned)(col * ldy + row) * 4u : OOB_OFFSET);
+    for (int q = 0; q < CPW; ++q) ypre[q] = 0.f;
+    if (beta != 0.f) {
+        const __amdgpu_buffer_rsrc_t yr = make_rsrc(
+            Y + (long long)col0 * ldy, (unsigned)(((long long)(cols_here - 1) * ldy + n_out) * 4));
+        if (by_row) {
+#pragma unroll
+            for (int q = 0; q < CPW; ++q) {
+                const int col = wave * CPW + q;
+                ypre[q] = buffer_load_f32(yr, col < cols_here ? (unsigned)(col * ldy + row0 + lane) * 4u : OOB_OFFSET);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const int col = ecol + 4 * k;
+                const float4 v = buffer_load_f32x4(yr, col < cols_here ? (unsigned)(col * ldy + row0 + erow) * 4u : OOB_OFFSET);
+                ypre[4 * k + 0] = v.x; ypre[4 * k + 1] = v.y; ypre[4 * k + 2] = v.z; ypre[4 * k + 3] = v.w;
+            }
         }
     }
 
@@ -723,37 +731,46 @@ __device__ __forceinline__ void spmm_tile_lean(
         const int i = wave + WAVES * it;
         const int piece = 64 * i + lane;
         const int col = piece / SP_DQUADS, quad = piece - col * SP_DQUADS;
-        const bool live = i < SP_DQUADS;     // SP_COLS * SP_DQUADS / 64 instructions stage a chunk
-        x_off[it] = live ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) + 16u * quad : OOB_OFFSET;
-        x_lds[it] = live ? 1024u * i : SP_DSPARE * 4u;
+        x_off[it] = (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) + 16u * quad;
+        x_lds[it] = 1024u * i;
     }
-    const int arow = row0 + lane;
+    // SP_COLS * SP_DQUADS / 64 = 19 instructions stage the dense rows of a chunk:
+    // waves 0-2 issue three of them, the others two.  Waves 3 and 4 fetch the
+    // chunk's diagonals instead, four diagonals x 64 rows each in one
+    // instruction (lane = 16 * diagonal + 16-byte piece).  A load instruction
+    // occupies the memory pipeline equally long whether it moves 4 or 16 bytes
+    // per lane, so the count per chunk -- 21 -- is what matters.
+    const bool x3 = wave < SP_DQUADS - 2 * WAVES;
+    const bool a_wave = (wave == 3) | (wave == 4);
+    const int a_j = 4 * (wave - 3) + (lane >> 4);          // the diagonal this lane fetches (waves 3, 4)
+    // every wave keeps its own count of loads per chunk: 3 for waves 0-4, 2 for the others
+    const bool three = wave < 5;
 
-    int tab_s0[NTAB], tab_len[NTAB], tab_slot[NTAB];
+    // table positions of every chunk's diagonals, for the lanes that fetch them
+    for (int t = threadIdx.x; t < nchunks * CHUNK_MAX; t += 64 * WAVES)
+        slot_tab[t] = reinterpret_cast<const int *>(chunks + t / CHUNK_MAX)[2 + t % CHUNK_MAX];
+
+    int tab_s0[NTAB], tab_len[NTAB];
 #pragma unroll
     for (int k = 0; k < NTAB; ++k) {
         const int *e = reinterpret_cast<const int *>(chunks + min(64 * k + lane, nchunks - 1));
         tab_s0[k] = e[0];
         tab_len[k] = e[1];
-        tab_slot[k] = e[2 + wave];
     }
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
     constexpr unsigned BUF_BYTES = SP_DSTAGE_FLOATS * 4u;
 
-    // requests chunk c into the buffer at byte address `buf`: 4 loads
+    // requests chunk c into the buffer at byte address `buf`: 3 or 2 loads
     auto issue = [&](int c, unsigned buf) {
         const int cc = min(c, nchunks - 1);
         const int l = cc & 63;
         int s0 = __builtin_amdgcn_readlane(tab_s0[0], l), len = __builtin_amdgcn_readlane(tab_len[0], l);
-        int sl = __builtin_amdgcn_readlane(tab_slot[0], l);
 #pragma unroll
         for (int k = 1; k < NTAB; ++k) {
             const bool here = (cc >> 6) == k;
             const int s0k = __builtin_amdgcn_readlane(tab_s0[k], l), lenk = __builtin_amdgcn_readlane(tab_len[k], l);
-            const int slk = __builtin_amdgcn_readlane(tab_slot[k], l);
             s0 = here ? s0k : s0;
             len = here ? lenk : len;
-            sl = here ? slk : sl;
         }
         const int a0 = row0 + s0;
         // past the table, and for a chunk whose rows lie outside the operand,
@@ -761,14 +778,16 @@ __device__ __forceinline__ void spmm_tile_lean(
         const bool real = (c < nchunks) & (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
         const sp_int4 xq = raw_rsrc(xbase, real ? x_bytes : 0u);
         const unsigned soff = real ? (unsigned)a0 * 4u : 0u;
-#pragma unroll
-        for (int it = 0; it < 3; ++it)
-            lds_load_b128(xq, buf + x_lds[it], x_off[it], soff);
-        const bool ok = real & (wave < len) & (sl >= 0);
-        const sp_int4 aq = raw_rsrc(vals, ok ? a_bytes : 0u);
-        const unsigned voff = (unsigned)(ashift ? arow + s0 + wave : arow) * 4u;
-        lds_load_b32(aq, buf + (unsigned)(SP_DAVALS + wave * SP_ROWS) * 4u, voff,
-                     ok ? (unsigned)sl * (unsigned)stride * 4u : 0u);
+        lds_load_b128(xq, buf + x_lds[0], x_off[0], soff);
+        lds_load_b128(xq, buf + x_lds[1], x_off[1], soff);
+        if (x3) lds_load_b128(xq, buf + x_lds[2], x_off[2], soff);
+        if (a_wave) {
+            const int sl = slot_tab[cc * CHUNK_MAX + a_j];
+            const bool ok = real & (a_j < len) & (sl >= 0);
+            const int arow = row0 + erow + (ashift ? s0 + a_j : 0);          // first of the lane's 4 rows of its diagonal
+            const unsigned voff = ok ? ((unsigned)sl * (unsigned)stride + (unsigned)arow) * 4u : OOB_OFFSET;
+            lds_load_b128(raw_rsrc(vals, a_bytes), buf + (unsigned)(SP_DAVALS + 4 * (wave - 3) * SP_ROWS) * 4u, voff, 0u);
+        }
     };
     auto read_window = [&](SpWindow<LCK, T> &win, int b) {
         const float *buf = lds[b];
@@ -776,10 +795,13 @@ __device__ __forceinline__ void spmm_tile_lean(
     };
 
     SpWindow<LCK, T> w0, w1;
+    __syncthreads();                                     // slot_tab is complete
     issue(0, lds0);
     issue(1, lds0 + BUF_BYTES);
     issue(2, lds0 + 2 * BUF_BYTES);
-    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");     // chunks 0 and 1 (and the destination values) are in
+    // chunks 0 and 1 (and the destination values) are in once only chunk 2's loads are outstanding
+    if (three) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
     __syncthreads();
     read_window(w0, 0);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -790,9 +812,10 @@ __device__ __forceinline__ void spmm_tile_lean(
         const bool more = c + 3 < nchunks;
         if (more) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES);    // over chunk c, whose window every wave holds
         spmm_rows<LCK, T, 0>(acc, cur);
-        // chunk c+2 must be in: everything but the 4 loads just issued
-        if (more) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        // chunk c+2 must be in: everything but the loads just issued
+        if (!more) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        else if (three) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
         __syncthreads();
     };
     int c = 0, b = 0, b1 = 1, b2 = 2;
@@ -812,26 +835,51 @@ __device__ __forceinline__ void spmm_tile_lean(
 #pragma unroll
     for (int t = 0; t < T; ++t) out[lane * SP_OPITCH + wave * T + t] = acc[t];
     __syncthreads();
-    const long long row = (long long)row0 + lane;
-    if (row < n_out) {
-        const float bias = (EP && ep.bias) ? ep.bias[row] : 0.f;
+    if (by_row) {
+        const long long row = (long long)row0 + lane;
+        const float bias = ep.bias ? ep.bias[row] : 0.f;
         float v[CPW];
 #pragma unroll
         for (int q = 0; q < CPW; ++q) v[q] = out[(wave * CPW + q) * SP_OPITCH + lane];   // all reads before the first store
         // the lane's 8 columns are two aligned blocks of 4: two generator calls
-        SpRand4 rnd[CPW / 4] = {};
-        if (EP && ep.act == 2) {
+        SpRand4 rnd[CPW / 4];
 #pragma unroll
-            for (int k = 0; k < CPW / 4; ++k)
-                rnd[k] = sp_philox((unsigned)row, (unsigned)(col0 + wave * CPW) / 4u + k, ep.seed_lo, ep.seed_hi);
-        }
+        for (int k = 0; k < CPW / 4; ++k)
+            rnd[k] = sp_philox((unsigned)row, (unsigned)(col0 + wave * CPW) / 4u + k, ep.seed_lo, ep.seed_hi);
 #pragma unroll
         for (int q = 0; q < CPW; ++q) {
             const int col = wave * CPW + q;
             if (col0 + col < batch) {
                 float *y = Y + (long long)(col0 + col) * ldy + row;
                 const float r = (beta == 0.f) ? alpha * v[q] : beta * ypre[q] + alpha * v[q];
-                *y = EP ? sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]) : r;
+                *y = sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]);
+            }
+        }
+    } else {
+        float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (EP && ep.bias) {
+            const float *bp = ep.bias + row0 + erow;
+            bias4 = make_float4(bp[0], bp[1], bp[2], bp[3]);
+        }
+        float4 v[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) v[k] = *reinterpret_cast<const float4 *>(out + (ecol + 4 * k) * SP_OPITCH + erow);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int col = ecol + 4 * k;
+            if (col0 + col < batch) {
+                const float s[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+                const float b4[4] = {bias4.x, bias4.y, bias4.z, bias4.w};
+                float r[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float t = (beta == 0.f) ? alpha * s[e] : beta * ypre[4 * k + e] + alpha * s[e];
+                    r[e] = EP ? sp_finish(t, b4[e], ep.act) : t;
+                }
+                // 4-byte alignment is all a 16-byte global store needs
+                float *y = Y + (long long)(col0 + col) * ldy + row0 + erow;
+                typedef float sp_f4u __attribute__((ext_vector_type(4), aligned(4)));
+                *reinterpret_cast<sp_f4u *>(y) = sp_f4u{r[0], r[1], r[2], r[3]};
             }
         }
     }
@@ -848,6 +896,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     static_assert(3 * SP_DSTAGE_FLOATS >= 2 * SP_STAGE_FLOATS, "the two bodies share one LDS block");
     __shared__ __attribute__((aligned(16))) float lds3[3][SP_DSTAGE_FLOATS];
     float (&lds)[2][SP_STAGE_FLOATS] = *reinterpret_cast<float (*)[2][SP_STAGE_FLOATS]>(&lds3[0][0]);
+    __shared__ int slot_tab[64 * NTAB * CHUNK_MAX];
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
     const int rowtile = tile / col_tiles;
     const int row0 = rowtile * SP_ROWS;
@@ -884,7 +933,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     }
     if (lean)
         // only the chunks inside the operand are walked; the others would add zeros
-        spmm_tile_lean<LCK, NTAB, EP>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
+        spmm_tile_lean<LCK, NTAB, EP>(lds3, slot_tab, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
                                       Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
     else
         spmm_tile_edge<LCK, T, NTAB, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,

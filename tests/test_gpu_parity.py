@@ -109,6 +109,11 @@ SHAPES = [
     (300, 300, list(range(-8, -1)) + list(range(0, 8)) + [100, 101], 1, 7),
     (260, 1000, [-200, -199, -198, -72, -71, 56, 57, 58, 59, 700], 1, 131),
     (1024, 768, [dy * 64 + dx for dy in range(-2, 3) for dx in range(0, 8)], 1, 1),
+    # window rows a multiple of the 64-row tile apart: square, rectangular both ways, a window with
+    # missing rows, ragged batch
+    (2048, 2048, [dy * 64 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 1, 70),
+    (1536, 2304, [dy * 128 + dx for dy in range(-2, 3) for dx in range(-2, 3)], 1, 130),
+    (2304, 1600, [dy * 128 + dx for dy in (-3, -2, -1, 1, 2) for dx in range(-1, 2)], 1, 64),
 ]
 
 
