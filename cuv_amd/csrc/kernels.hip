@@ -23,6 +23,8 @@
 //           serially in ascending column order.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "kernels.hpp"
 
 namespace cuvdia {
@@ -979,10 +981,10 @@ struct DdShape {
 };
 static_assert(DdShape<2>::PITCH >= DD_ROWS + PAIR_MAX_DELTA + CHUNK_MAX, "a pair's band must fit its buffer");
 
-template <int NCH>
+// What a wave has in flight of A for one group of 4 batch columns (two of
+// these alternate; B's pieces need one set of registers only, see the loop).
 struct DdStage {
-    float b[DD_BG * DdShape<NCH>::NQ + 1];   // B: NQ x 64 rows per column, + the last 8 rows of all 4 columns in one load
-    float a[DD_BG][4];                        // A: this lane's 4 rows of each column
+    float a[DD_BG][4];    // this lane's 4 rows of each column
 };
 
 template <int LC, int NCH>
@@ -1001,7 +1003,7 @@ __device__ __forceinline__ void dd2dia_unit(
     unsigned c_bytes)
 {
     typedef DdShape<NCH> S;
-    constexpr int NQ = S::NQ, PITCH = S::PITCH, WAVES = S::WAVES;
+    constexpr int PITCH = S::PITCH, WAVES = S::WAVES;
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
     constexpr int RED_T = NCH * LC * 64 + 8;        // floats between the 4 rows a lane owns: keeps the
@@ -1052,24 +1054,33 @@ __device__ __forceinline__ void dd2dia_unit(
             for (int j = 0; j < LC; ++j) cpre[n][j] = buffer_load_f32(cr, c_offset(n, j));
     }
 
-    // per-lane byte offsets inside one column; rows outside B, and staged rows
-    // no window reaches, use the out-of-range marker
-    unsigned b_off[NQ + 1];
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-        const int rr = q * 64 + lane, r = base + rr;
-        b_off[q] = (rr < need && r >= 0 && r < w) ? (unsigned)r * 4u : OOB_OFFSET;
-    }
-    // the last 8 staged rows of all 4 columns travel in one load: lane = 8 * column + row
-    const int hb = lane >> 3;
+    // The band of B travels as 16-byte pieces, a lane holding rows base + 4*lane
+    // .. + 3 and, where the band reaches that far, base + 256 + 4*lane .. + 3:
+    // two loads per column, whatever the alignment of base (a load instruction
+    // occupies the memory pipeline equally long for 4 and for 16 bytes per
+    // lane).  Rows of the band outside B need no care in general: they only
+    // meet sums of slots that hold no matrix element and are never stored, and
+    // a piece that leaves column c lands in a neighbouring column of the same
+    // allocation.  The whole byte offset goes into the vector operand, which
+    // is what the buffer's range check looks at, so nothing outside the
+    // allocation is ever touched.  Only where a column's band crosses the
+    // allocation's first or last byte (the first and the last batch columns of
+    // tiles at the ends of B) a piece could lose valid rows to the range check,
+    // which answers for the piece as a whole: those columns -- [0, rare_lo) and
+    // [rare_hi, batch) -- stay out of the pipelined loop and are worked row by
+    // row by wave 0 before it (see below).
+    const int nquad = (need + 3) / 4;                     // pieces per column that are ever read, 66 .. 98
+    const bool tail = lane < nquad - 64;
+    const unsigned vb_off0 = (unsigned)(base + 4 * lane) * 4u;
+    const long long b_floats = (long long)(batch - 1) * ldb + w;
+    // column c's band starts c*ldb + base floats into the allocation and is 4*nquad floats long
+    int rare_lo = 0, rare_hi = batch;
+    if (base < 0) rare_lo = (int)min((long long)batch, (-(long long)base + ldb - 1) / ldb);
     {
-        const int rr = 64 * NQ + (lane & 7), r = base + rr;
-        b_off[NQ] = (hb < DD_BG && rr < need && r >= 0 && r < w)
-                        ? ((unsigned)r + (unsigned)hb * (unsigned)ldb) * 4u : OOB_OFFSET;
+        const long long room = b_floats - base - 4 * nquad;                   // c*ldb must not exceed this
+        if (room < (long long)(batch - 1) * ldb) rare_hi = room < 0 ? 0 : (int)(room / ldb) + 1;
+        rare_hi = max(rare_hi, rare_lo);
     }
-    // where that load lands in buffer 0 / buffer 1 of this wave (idle lanes: the spare slot)
-    const int halo_at0 = hb < DD_BG ? hb * PITCH + 64 * NQ + (lane & 7) : 2 * DD_BG * PITCH;
-    const int halo_at1 = hb < DD_BG ? halo_at0 + DD_BG * PITCH : 2 * DD_BG * PITCH;
     unsigned a_off[4];
     if (AVEC) {
         a_off[0] = (myrow + 3 < h) ? (unsigned)myrow * 4u : OOB_OFFSET;
@@ -1097,21 +1108,22 @@ __device__ __forceinline__ void dd2dia_unit(
     float *mybuf = lds + wave * S::WAVE_FLOATS;
     const __amdgpu_buffer_rsrc_t b_all = make_rsrc(B, b_bytes);
 
-    // requests column i of group g: B rows into st.b, A rows into st.a (the
-    // load of the last 8 rows, which serves all 4 columns, travels with column 0)
-    auto issue_col = [&](int g, int i, DdStage<NCH> &st) {
+    // B in flight: per column, rows base + 4*lane .. + 3 and base + 256 + 4*lane .. + 3 of the band.  One set
+    // serves the current and the next group: column i of the next group is requested after column i of the
+    // current one has gone to LDS.
+    float4 bq[DD_BG][2];
+    // requests column i of group g: B rows into bq, A rows into st.a
+    auto issue_col = [&](int g, int i, DdStage &st) {
         const int b0 = __builtin_amdgcn_readfirstlane(g * DD_BG);   // wave-uniform: keeps column offsets scalar
-        const bool live = b0 + i < batch;
+        const int col = b0 + i;
+        const bool live = (col >= rare_lo) & (col < rare_hi);
         const __amdgpu_buffer_rsrc_t br = make_rsrc(B, live ? b_bytes : 0u);
-        const unsigned colb = (unsigned)(b0 + i) * ldb4;
-#pragma unroll
-        for (int q = 0; q < NQ; ++q)
-            st.b[i * NQ + q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, b_off[q], colb, 0));
-        if (i == 0)
-            st.b[DD_BG * NQ] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                b_all, (b0 + hb < batch) ? b_off[NQ] : OOB_OFFSET, (unsigned)b0 * ldb4, 0));
+        const unsigned colb = (unsigned)col * ldb4;
+        const unsigned v0 = vb_off0 + colb;
+        bq[i][0] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, v0, 0, 0));
+        bq[i][1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, tail ? v0 + 1024u : OOB_OFFSET, 0, 0));
         const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, live ? a_bytes : 0u);
-        const unsigned cola = (unsigned)(b0 + i) * lda4;
+        const unsigned cola = (unsigned)col * lda4;
         if (AVEC) {
             const float4 v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[0], cola, 0));
             st.a[i][0] = v.x; st.a[i][1] = v.y; st.a[i][2] = v.z; st.a[i][3] = v.w;
@@ -1121,15 +1133,15 @@ __device__ __forceinline__ void dd2dia_unit(
                 st.a[i][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, a_off[t], cola, 0));
         }
     };
-    auto issue = [&](int g, DdStage<NCH> &st) {
+    auto issue = [&](int g, DdStage &st) {
 #pragma unroll
         for (int i = 0; i < DD_BG; ++i) issue_col(g, i, st);
     };
-    auto commit_col = [&](const DdStage<NCH> &st, int par, int i) {
+    auto commit_col = [&](int par, int i) {
         float *buf = mybuf + par * (DD_BG * PITCH);
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) buf[i * PITCH + q * 64 + lane] = st.b[i * NQ + q];
-        if (i == 0) mybuf[par ? halo_at1 : halo_at0] = st.b[DD_BG * NQ];
+        *reinterpret_cast<float4 *>(buf + i * PITCH + 4 * lane) = bq[i][0];
+        // lanes past the band's end drop their (zero) piece in the spare slot
+        *reinterpret_cast<float4 *>(tail ? buf + i * PITCH + 256 + 4 * lane : mybuf + 2 * DD_BG * PITCH) = bq[i][1];
         wave_lds_fence();
     };
     struct Windows { float w[NCH][WQ * 4]; };
@@ -1158,25 +1170,25 @@ __device__ __forceinline__ void dd2dia_unit(
     // of the next group is requested right after, so every load has one whole
     // step to arrive and the requests are spread between the FMA blocks.  Past
     // the last group the requests hit the empty resource.
-    auto step = [&](int k, int par, DdStage<NCH> &cur, DdStage<NCH> &nxt) {
+    auto step = [&](int k, int par, DdStage &cur, DdStage &nxt) {
         const float *buf = mybuf + par * (DD_BG * PITCH);
         const int gn = wave + WAVES * (k + 1);
         Windows w0, w1;
-        commit_col(cur, par, 0);
+        commit_col(par, 0);
         read_windows(w0, buf, 0);
-        commit_col(cur, par, 1);
+        commit_col(par, 1);
         read_windows(w1, buf, 1);
         issue_col(gn, 0, nxt);
         __builtin_amdgcn_sched_barrier(0);
         fmas(cur.a[0], w0);
         __builtin_amdgcn_sched_barrier(0);
-        commit_col(cur, par, 2);
+        commit_col(par, 2);
         read_windows(w0, buf, 2);
         issue_col(gn, 1, nxt);
         __builtin_amdgcn_sched_barrier(0);
         fmas(cur.a[1], w1);
         __builtin_amdgcn_sched_barrier(0);
-        commit_col(cur, par, 3);
+        commit_col(par, 3);
         read_windows(w1, buf, 3);
         issue_col(gn, 2, nxt);
         __builtin_amdgcn_sched_barrier(0);
@@ -1188,8 +1200,36 @@ __device__ __forceinline__ void dd2dia_unit(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    DdStage<NCH> st0, st1;
+    DdStage st0, st1;
     issue(wave, st0);
+    // The columns left out above, while the first group's loads are on their
+    // way: wave 0 fetches its 4 rows of A and, value by value, its windows of
+    // B (rows outside B as zeros) and adds the column's products to its sums.
+    if (wave == 0) {
+#pragma clang loop unroll(disable)
+        for (int col = 0; col < batch; ++col) {
+            if (col == rare_lo) col = rare_hi;
+            if (col >= batch) break;
+            const unsigned colb = (unsigned)col * ldb4;
+            Windows win;
+#pragma unroll
+            for (int n = 0; n < NCH; ++n)
+#pragma unroll
+                for (int q = 0; q < WQ * 4; ++q) {
+                    const int r = base + 4 * lane + (n ? delta : 0) + q;
+                    win.w[n][q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        b_all, (r >= 0 && r < w) ? (unsigned)r * 4u + colb : OOB_OFFSET, 0, 0));
+                }
+            const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, a_bytes);
+            const unsigned cola = (unsigned)col * lda4;
+            float a[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                a[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    ar, (myrow + t < h) ? (unsigned)(myrow + t) * 4u + cola : OOB_OFFSET, 0, 0));
+            fmas(a, win);
+        }
+    }
     int k = 0;
     for (; k + 1 < steps; k += 2) {
         step(k, 0, st0, st1);
