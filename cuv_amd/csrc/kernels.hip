@@ -952,9 +952,10 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
 // pair by 8; wave q walks the batch-column groups g = q, q + WAVES, ...
 // (4 columns per group).  Per group and column the wave
 //   1. writes the column's rows [row0 + s0, row0 + s0 + 264 + delta) of B,
-//      fetched one step earlier with lanes along rows (dword buffer loads;
-//      rows outside B read as 0 through the buffer range check), to its
-//      private LDS buffer -- no workgroup barrier in the loop;
+//      fetched one step earlier as 16-byte pieces (a lane holds 4 consecutive
+//      rows, two loads per column), to its private LDS buffer -- no workgroup
+//      barrier in the loop.  Rows of that band outside B are not masked: they
+//      only meet sums of slots that hold no matrix element (see the loads);
 //   2. reads its 4 + LC - 1 wide window of B per chunk from LDS with 16-byte
 //      reads (the second chunk's window starts delta rows further);
 //   3. requests the same column of the next group: its rows of B and its own
@@ -973,7 +974,7 @@ constexpr int DD_BG = 4;           // batch columns per step
 
 template <int NCH>
 struct DdShape {
-    static constexpr int NQ = NCH == 1 ? 4 : 6;                 // 64-row loads per column
+    static constexpr int NQ = NCH == 1 ? 4 : 6;                 // 64-row blocks of the band
     static constexpr int PITCH = 64 * NQ + 8;                   // staged rows per column: 264 or 392
     static constexpr int WAVES = NCH == 1 ? 4 : 8;
     static constexpr int WAVE_FLOATS = 2 * DD_BG * PITCH + 4;   // two buffers + a slot idle lanes write to
