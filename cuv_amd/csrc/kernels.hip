@@ -1046,9 +1046,14 @@ __device__ __forceinline__ void dd2dia_unit(
         return ok ? ((unsigned)sl * (unsigned)stride + (unsigned)o) * 4u : OOB_OFFSET;
     };
     float cpre[NCH][LC];
-    {
-        // beta == 0: C is not read (an empty resource returns zeros without touching memory)
-        const __amdgpu_buffer_rsrc_t cr = make_rsrc(C, beta != 0.f ? c_bytes : 0u);
+#pragma unroll
+    for (int n = 0; n < NCH; ++n)
+#pragma unroll
+        for (int j = 0; j < LC; ++j) cpre[n][j] = 0.f;
+    // beta == 0: C is not read; waves 4..7 of a pair write nothing and ask for nothing (a load costs the
+    // memory pipeline its slot even when every lane is out of range)
+    if ((beta != 0.f) & (wave < 4)) {
+        const __amdgpu_buffer_rsrc_t cr = make_rsrc(C, c_bytes);
 #pragma unroll
         for (int n = 0; n < NCH; ++n)
 #pragma unroll

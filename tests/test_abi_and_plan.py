@@ -50,6 +50,13 @@ def test_no_device_is_an_error_not_a_fallback():
     assert rc == _lib.EINVAL
     assert L.cuvdia_spmm_f32(None, None, None, 0, None, 0, 1, b"n", 1.0, 0.0, None) == _lib.EINVAL
     assert L.cuvdia_set_path(7) == _lib.EINVAL and L.cuvdia_set_path(0) == 0
+    # argument checks come before any device work
+    assert L.cuvdia_learn_step_weight_decay_f32(None, None, -1, 0.1, 0.0, None) == _lib.EINVAL
+    assert L.cuvdia_learn_step_weight_decay_f32(None, None, 0, 0.1, 0.0, None) == 0
+    assert L.cuvdia_learn_step_weight_decay_f32(None, None, 4, 0.1, 0.0, None) == _lib.EINVAL
+    assert L.cuvdia_spmm_layer_f32(None, None, None, 0, None, 0, 1, b"n", 1.0, 0.0, None, 7, 0, None) == _lib.EINVAL
+    assert L.cuvdia_spmm_bias_act_f32(None, None, None, 0, None, 0, 1, b"n", 1.0, 0.0, None,
+                                      _lib.ACT_SIGMOID_SAMPLE, None) == _lib.EINVAL
 
 
 def _plan(offsets, transposed=False):
