@@ -653,6 +653,9 @@ __device__ __forceinline__ sp_int4 raw_rsrc(const void *base, unsigned bytes)
 }
 __device__ __forceinline__ void lds_load_b128(sp_int4 rsrc, unsigned lds_byte_addr, unsigned voff, unsigned soff)
 {
+    // both are wave-uniform by construction; this keeps them in scalar registers whatever the compiler infers
+    lds_byte_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
+    soff = __builtin_amdgcn_readfirstlane(soff);
     asm volatile("s_mov_b32 m0, %0\n\t"
                  "s_nop 0\n\t"
                  "buffer_load_dwordx4 %1, %2, %3 offen lds"
