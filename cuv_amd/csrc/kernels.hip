@@ -653,9 +653,11 @@ __device__ __forceinline__ sp_int4 raw_rsrc(const void *base, unsigned bytes)
 }
 __device__ __forceinline__ void lds_load_b128(sp_int4 rsrc, unsigned lds_byte_addr, unsigned voff, unsigned soff)
 {
-    // both are wave-uniform by construction; this keeps them in scalar registers whatever the compiler infers
+    // all three are wave-uniform by construction; this keeps them in scalar registers whatever the compiler infers
     lds_byte_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
     soff = __builtin_amdgcn_readfirstlane(soff);
+    rsrc = sp_int4{__builtin_amdgcn_readfirstlane(rsrc.x), __builtin_amdgcn_readfirstlane(rsrc.y),
+                   __builtin_amdgcn_readfirstlane(rsrc.z), __builtin_amdgcn_readfirstlane(rsrc.w)};
     asm volatile("s_mov_b32 m0, %0\n\t"
                  "s_nop 0\n\t"
                  "buffer_load_dwordx4 %1, %2, %3 offen lds"
@@ -683,7 +685,7 @@ static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + CHUNK_MAX - 1 <= SP_DPI
 
 template <int LCK, int NTAB, bool EP>
 __device__ __forceinline__ void spmm_tile_lean(
-    float (&lds)[3][SP_DSTAGE_FLOATS], int *slot_tab, int row0, int col0,
+    float (&lds)[3][SP_DSTAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, SpEpilogue ep)
@@ -751,32 +753,27 @@ __device__ __forceinline__ void spmm_tile_lean(
     // every wave keeps its own count of loads per chunk: 3 for waves 0-4, 2 for the others
     const bool three = wave < 5;
 
-    // table positions of every chunk's diagonals, for the lanes that fetch them
-    for (int t = threadIdx.x; t < nchunks * CHUNK_MAX; t += 64 * WAVES)
-        slot_tab[t] = reinterpret_cast<const int *>(chunks + t / CHUNK_MAX)[2 + t % CHUNK_MAX];
-
-    int tab_s0[NTAB], tab_len[NTAB];
-#pragma unroll
-    for (int k = 0; k < NTAB; ++k) {
-        const int *e = reinterpret_cast<const int *>(chunks + min(64 * k + lane, nchunks - 1));
-        tab_s0[k] = e[0];
-        tab_len[k] = e[1];
-    }
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
     constexpr unsigned BUF_BYTES = SP_DSTAGE_FLOATS * 4u;
 
-    // requests chunk c into the buffer at byte address `buf`: 3 or 2 loads
-    auto issue = [&](int c, unsigned buf) {
-        const int cc = min(c, nchunks - 1);
-        const int l = cc & 63;
-        int s0 = __builtin_amdgcn_readlane(tab_s0[0], l), len = __builtin_amdgcn_readlane(tab_len[0], l);
-#pragma unroll
-        for (int k = 1; k < NTAB; ++k) {
-            const bool here = (cc >> 6) == k;
-            const int s0k = __builtin_amdgcn_readlane(tab_s0[k], l), lenk = __builtin_amdgcn_readlane(tab_len[k], l);
-            s0 = here ? s0k : s0;
-            len = here ? lenk : len;
-        }
+    // A chunk's table entry travels through three 16-byte SCALAR loads into
+    // scalar registers, one iteration before the chunk is requested: no vector
+    // memory instruction, no LDS copy and no register table stand between the
+    // kernel's start and its first requests, and the loop's entries arrive
+    // under the wait that ends every iteration anyway.
+    struct Entry {
+        int s0, len, p0, p1, p2, p3, p4, p5, p6, p7;     // shift, length, table positions of the 8 diagonals
+    };
+    auto fetch = [&](int c) __attribute__((always_inline)) {
+        typedef int sp_i4 __attribute__((ext_vector_type(4)));
+        typedef const sp_i4 __attribute__((address_space(4))) *sc_i4_ptr;
+        const sc_i4_ptr e = (sc_i4_ptr)(chunks + min(c, nchunks - 1));
+        const sp_i4 e0 = e[0], e1 = e[1], e2 = e[2];
+        return Entry{e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w, e2.x, e2.y};
+    };
+    // requests chunk c, whose entry is en, into the buffer at byte address `buf`: 3 or 2 loads
+    auto issue = [&](int c, unsigned buf, const Entry &en) __attribute__((always_inline)) {
+        const int s0 = en.s0;
         const int a0 = row0 + s0;
         // past the table, and for a chunk whose rows lie outside the operand,
         // nothing is fetched: an empty resource delivers zeros
@@ -787,23 +784,33 @@ __device__ __forceinline__ void spmm_tile_lean(
         lds_load_b128(xq, buf + x_lds[1], x_off[1], soff);
         if (x3) lds_load_b128(xq, buf + x_lds[2], x_off[2], soff);
         if (a_wave) {
-            const int sl = slot_tab[cc * CHUNK_MAX + a_j];
-            const bool ok = real & (a_j < len) & (sl >= 0);
+            // table position of this lane's diagonal, a_j: picked from the 8 scalars (each passed through an
+            // empty asm so that the chain of selects stays one, and the entry stays in registers)
+            int p[CHUNK_MAX] = {en.p0, en.p1, en.p2, en.p3, en.p4, en.p5, en.p6, en.p7};
+#pragma unroll
+            for (int k = 0; k < CHUNK_MAX; ++k) asm("" : "+s"(p[k]));
+            int sl = p[0];
+#pragma unroll
+            for (int k = 1; k < CHUNK_MAX; ++k) sl = a_j == k ? p[k] : sl;
+            const bool ok = real & (a_j < en.len) & (sl >= 0);
             const int arow = row0 + erow + (ashift ? s0 + a_j : 0);          // first of the lane's 4 rows of its diagonal
             const unsigned voff = ok ? ((unsigned)sl * (unsigned)stride + (unsigned)arow) * 4u : OOB_OFFSET;
             lds_load_b128(raw_rsrc(vals, a_bytes), buf + (unsigned)(SP_DAVALS + 4 * (wave - 3) * SP_ROWS) * 4u, voff, 0u);
         }
     };
-    auto read_window = [&](SpWindow<LCK, T> &win, int b) {
+    auto read_window = [&](SpWindow<LCK, T> &win, int b) __attribute__((always_inline)) {
         const float *buf = lds[b];
         spmm_read_window<LCK, T>(win, buf + lane * SP_DPITCH + wave * T, buf + SP_DAVALS + wave * T + (lane & (T - 1)));
     };
 
     SpWindow<LCK, T> w0, w1;
-    __syncthreads();                                     // slot_tab is complete
-    issue(0, lds0);
-    issue(1, lds0 + BUF_BYTES);
-    issue(2, lds0 + 2 * BUF_BYTES);
+    {
+        const Entry h0 = fetch(0), h1 = fetch(1), h2 = fetch(2);
+        issue(0, lds0, h0);
+        issue(1, lds0 + BUF_BYTES, h1);
+        issue(2, lds0 + 2 * BUF_BYTES, h2);
+    }
+    Entry e0 = fetch(3), e1 = e0;
     // chunks 0 and 1 (and the destination values) are in once only chunk 2's loads are outstanding
     if (three) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
@@ -811,11 +818,13 @@ __device__ __forceinline__ void spmm_tile_lean(
     read_window(w0, 0);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __syncthreads();                                     // every wave has its window(0): buffer 0 may be reused
-    // iteration c: buffers b (chunk c), b1 (chunk c+1), b2 (chunk c+2)
-    auto iteration = [&](int c, int b, int b1, SpWindow<LCK, T> &cur, SpWindow<LCK, T> &nxt) {
-        read_window(nxt, b1);
+    // iteration c: buffers b (chunk c), b1 (chunk c+1), b2 (chunk c+2); `use` is the entry of chunk c+3,
+    // `next` receives the entry of chunk c+4
+    auto iteration = [&](int c, int b, int b1, SpWindow<LCK, T> &cur, SpWindow<LCK, T> &nxt, const Entry &use, Entry &next) __attribute__((always_inline)) {
         const bool more = c + 3 < nchunks;
-        if (more) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES);    // over chunk c, whose window every wave holds
+        if (more) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use);    // over chunk c, whose window every wave holds
+        next = fetch(c + 4);
+        read_window(nxt, b1);
         spmm_rows<LCK, T, 0>(acc, cur);
         // chunk c+2 must be in: everything but the loads just issued
         if (!more) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -825,14 +834,15 @@ __device__ __forceinline__ void spmm_tile_lean(
     };
     int c = 0, b = 0, b1 = 1, b2 = 2;
     if (nchunks & 1) {
-        iteration(0, b, b1, w0, w1);
+        iteration(0, b, b1, w0, w1, e0, e1);
         { const SpWindow<LCK, T> t = w0; w0 = w1; w1 = t; }
         { const int t = b; b = b1; b1 = b2; b2 = t; }
+        e0 = e1;
         c = 1;
     }
     for (; c < nchunks; c += 2) {
-        iteration(c, b, b1, w0, w1);
-        iteration(c + 1, b1, b2, w1, w0);
+        iteration(c, b, b1, w0, w1, e0, e1);
+        iteration(c + 1, b1, b2, w1, w0, e1, e0);
         { const int t0 = b, t1 = b1; b = b2; b1 = t0; b2 = t1; }
     }
     // (the last barrier came after every window read, and no load is in flight)
@@ -901,7 +911,6 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     static_assert(3 * SP_DSTAGE_FLOATS >= 2 * SP_STAGE_FLOATS, "the two bodies share one LDS block");
     __shared__ __attribute__((aligned(16))) float lds3[3][SP_DSTAGE_FLOATS];
     float (&lds)[2][SP_STAGE_FLOATS] = *reinterpret_cast<float (*)[2][SP_STAGE_FLOATS]>(&lds3[0][0]);
-    __shared__ int slot_tab[64 * NTAB * CHUNK_MAX];
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
     const int rowtile = tile / col_tiles;
     const int row0 = rowtile * SP_ROWS;
@@ -938,7 +947,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
     }
     if (lean)
         // only the chunks inside the operand are walked; the others would add zeros
-        spmm_tile_lean<LCK, NTAB, EP>(lds3, slot_tab, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
+        spmm_tile_lean<LCK, NTAB, EP>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
                                       Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
     else
         spmm_tile_edge<LCK, T, NTAB, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
