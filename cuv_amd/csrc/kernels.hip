@@ -375,6 +375,17 @@ __device__ __forceinline__ void spmm_rows(float (&acc)[T], const SpWindow<LCK, T
     }
 }
 
+// the diagonals J .. J1 - 1 of a chunk
+template <int LCK, int T, int J, int J1>
+__device__ __forceinline__ void spmm_rows_range(float (&acc)[T], const SpWindow<LCK, T> &win)
+{
+    if constexpr (J < J1) {
+        fma_block8<J, 0>(acc, win.a[J], win.w);
+        if constexpr (T == 16) fma_block8<J, 8>(acc, win.a[J], win.w);
+        spmm_rows_range<LCK, T, J + 1, J1>(acc, win);
+    }
+}
+
 template <int LCK, int T>
 __device__ __forceinline__ void spmm_read_window(SpWindow<LCK, T> &win, const float *win_lds,
                                                  const float *a_lds)
@@ -811,26 +822,29 @@ __device__ __forceinline__ void spmm_tile_lean(
         issue(2, lds0 + 2 * BUF_BYTES, h2);
     }
     Entry e0 = fetch(3), e1 = e0;
-    // chunks 0 and 1 (and the destination values) are in once only chunk 2's loads are outstanding
-    if (three) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    // The first window can be read as soon as chunk 0 (and the destination values) is in: the loads of
+    // chunks 1 and 2 stay outstanding.
+    if (three) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     __syncthreads();
     read_window(w0, 0);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __syncthreads();                                     // every wave has its window(0): buffer 0 may be reused
-    // iteration c: buffers b (chunk c), b1 (chunk c+1), b2 (chunk c+2); `use` is the entry of chunk c+3,
-    // `next` receives the entry of chunk c+4
+    // Iteration c: buffers b (chunk c), b1 (chunk c+1); `use` is the entry of chunk c+3, `next` receives
+    // the entry of chunk c+4.  The FMAs of chunk c are cut in two: the wait for chunk c+1, the barrier
+    // and the read of its window sit between the halves, so the second half hides the read and a chunk
+    // is waited for only when its turn has come -- the product starts with one chunk in LDS, not two.
+    constexpr int JH = (LCK + 1) / 2;
     auto iteration = [&](int c, int b, int b1, SpWindow<LCK, T> &cur, SpWindow<LCK, T> &nxt, const Entry &use, Entry &next) __attribute__((always_inline)) {
-        const bool more = c + 3 < nchunks;
-        if (more) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use);    // over chunk c, whose window every wave holds
-        next = fetch(c + 4);
-        read_window(nxt, b1);
-        spmm_rows<LCK, T, 0>(acc, cur);
-        // chunk c+2 must be in: everything but the loads just issued
-        if (!more) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        spmm_rows_range<LCK, T, 0, JH>(acc, cur);
+        // chunk c+1 must be in; the loads of chunk c+2 (requested whenever c+2 < 3 or it exists) may stay out
+        const bool younger = (c + 2 < 3) | (c + 2 < nchunks);
+        if (!younger) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         else if (three) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
+        __syncthreads();                                 // also: every wave holds window(c), buffer b may be reused
+        if (c + 1 < nchunks) read_window(nxt, b1);
+        if (c + 3 < nchunks) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use);
+        next = fetch(c + 4);
+        spmm_rows_range<LCK, T, JH, LCK>(acc, cur);
     };
     int c = 0, b = 0, b1 = 1, b2 = 2;
     if (nchunks & 1) {
@@ -845,7 +859,9 @@ __device__ __forceinline__ void spmm_tile_lean(
         iteration(c + 1, b1, b2, w1, w0, e1, e0);
         { const int t0 = b, t1 = b1; b = b2; b1 = t0; b2 = t1; }
     }
-    // (the last barrier came after every window read, and no load is in flight)
+    // every wave must be through with its window reads, and no load in flight, before the buffers are reused
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
     float *out = &lds[0][0];
 #pragma unroll
     for (int t = 0; t < T; ++t) out[lane * SP_OPITCH + wave * T + t] = acc[t];
