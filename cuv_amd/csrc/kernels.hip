@@ -290,9 +290,10 @@ __global__ __launch_bounds__(AXPBY_THREADS) void axpby_kernel(
 // so staging costs the waves 4 instructions per chunk.  The tiles at the
 // operand's ends take spmm_tile_edge, which stages through registers because
 // it has to clamp and shift what it fetches.  Both are software-pipelined
-// three chunks deep, keep the chunk table in vector registers (lane i <->
-// entry i, read with v_readlane), and transpose the sums through LDS at the
-// end so the store to dst is lanes-along-rows.
+// three chunks deep and transpose the sums through LDS at the end so that the
+// store to dst runs along the rows; the lean body reads the chunk table
+// through scalar loads, the edge body keeps it in vector registers (lane i
+// <-> entry i, read with v_readlane).
 
 constexpr int SP_ROWS = 64;        // output rows per workgroup
 constexpr int SP_COLS = 64;        // batch columns per workgroup (one per lane)
@@ -685,9 +686,10 @@ __device__ __forceinline__ void lds_load_b128(sp_int4 rsrc, unsigned lds_byte_ad
 // bank conflicts.  Wave w issues instructions w, w + 8 and (waves 0-2)
 // w + 16; waves 3 and 4 fetch the chunk's 8 diagonals for the 64 rows, 4
 // diagonals per instruction: 21 loads per chunk, none through registers, no
-// LDS write instruction.  Three LDS buffers: chunk k lives in buffer k % 3;
-// while the FMAs of chunk c run, window(c+1) is being read, chunk c+2 is
-// landing and chunk c+3 has just been requested.
+// LDS write instruction.  Three LDS buffers: chunk k lives in buffer k % 3.
+// The FMAs of chunk c are cut in two; between the halves sit the wait for
+// chunk c+1, the barrier, the read of window(c+1) and the request for chunk
+// c+3, while chunk c+2 is landing.
 constexpr int SP_DQUADS = 19;                       // pieces per column staged by the direct loads (76 rows)
 constexpr int SP_DPITCH = 4 * SP_DQUADS;            // floats between staged columns
 constexpr int SP_DAVALS = SP_COLS * SP_DPITCH;      // diagonal values sit behind the dense rows
