@@ -55,6 +55,7 @@ def lib():
     L.cuvdia_spmm_layer_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp, c_int,
                                         ctypes.c_ulonglong, c_vp]
     L.cuvdia_learn_step_weight_decay_f32.argtypes = [c_vp, c_vp, c_ll, c_f, c_f, c_vp]
+    L.cuvdia_learn_step_weight_decay_momentum_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_f, c_f, c_f, c_vp]
     L.cuvdia_dd2dia_f32.argtypes = [c_vp, c_vp, c_vp, c_ll, c_vp, c_ll, c_int, c_f, c_f, c_vp]
     L.cuvdia_avg_diagonals_f32.argtypes = [c_vp, c_vp, c_vp, c_vp]
     L.cuvdia_spmm_offsets_f32.argtypes = [c_vp, ip, c_int, c_int, c_int, c_int, c_int, c_vp, c_ll,
@@ -65,7 +66,7 @@ def lib():
                  "cuvdia_desc_info", "cuvdia_spmm_f32", "cuvdia_dd2dia_f32", "cuvdia_spmm_offsets_f32",
                  "cuvdia_dd2dia_offsets_f32", "cuvdia_cache_clear", "cuvdia_spmm_bias_act_f32",
                  "cuvdia_spmm_layer_f32", "cuvdia_learn_step_weight_decay_f32", "cuvdia_avg_diagonals_f32",
-                 "cuvdia_plan_units"):
+                 "cuvdia_plan_units", "cuvdia_learn_step_weight_decay_momentum_f32"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

@@ -324,6 +324,18 @@ int cuvdia_learn_step_weight_decay_f32(float *W, const float *dW, long long n, f
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "learn_step_weight_decay kernel launch");
 }
 
+int cuvdia_learn_step_weight_decay_momentum_f32(float *W, float *momentum, const float *dW, long long n,
+                                                float learnrate, float momentum_weight, float decay, void *stream)
+{
+    if (n < 0) return CUVDIA_EINVAL;
+    if (n == 0) return CUVDIA_OK;
+    if (!W || !momentum || !dW) return CUVDIA_EINVAL;    // src/cuv/tensor_ops/rprop.cu:377-381
+    if (const int rc = require_device()) return rc;
+    const hipError_t e = launch_momentum(W, momentum, dW, n, learnrate, momentum_weight, decay,
+                                         static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "learn_step_weight_decay_momentum kernel launch");
+}
+
 int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals, const float *B, long long ldb,
                     float *dst, long long ldd, int batch, char transA,
                     float alpha, float beta, void *stream)

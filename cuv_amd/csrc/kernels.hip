@@ -264,6 +264,44 @@ __global__ __launch_bounds__(AXPBY_THREADS) void axpby_kernel(
     }
 }
 
+// m = momentum_weight*m - lr*(dW + l2decay*W); W += m; M = m
+// (src/cuv/tensor_ops/rprop.cu:158-170, the device kernel's formula).  Three
+// arrays read, two written: 20 bytes per element, HBM-bound; same layout of
+// the work as axpby_kernel.
+__global__ __launch_bounds__(AXPBY_THREADS) void momentum_kernel(
+    float *__restrict__ W, float *__restrict__ M, const float *__restrict__ dW, long long n,
+    float lr, float mw, float l2, int head, int vec)
+{
+    const long long tid = (long long)blockIdx.x * AXPBY_THREADS + threadIdx.x;
+    const long long nthreads = (long long)gridDim.x * AXPBY_THREADS;
+    auto one = [&](long long i) {
+        const float m = mw * M[i] - lr * (dW[i] + l2 * W[i]);
+        W[i] += m;
+        M[i] = m;
+    };
+    if (!vec) {
+        for (long long i = tid; i < n; i += nthreads) one(i);
+        return;
+    }
+    const long long nvec = (n - head) / 4;
+    float4 *W4 = reinterpret_cast<float4 *>(W + head);
+    float4 *M4 = reinterpret_cast<float4 *>(M + head);
+    const float4 *D4 = reinterpret_cast<const float4 *>(dW + head);
+    for (long long i = tid; i < nvec; i += nthreads) {
+        const float4 d = D4[i];
+        float4 w = W4[i], m = M4[i];
+        m.x = mw * m.x - lr * (d.x + l2 * w.x); w.x += m.x;
+        m.y = mw * m.y - lr * (d.y + l2 * w.y); w.y += m.y;
+        m.z = mw * m.z - lr * (d.z + l2 * w.z); w.z += m.z;
+        m.w = mw * m.w - lr * (d.w + l2 * w.w); w.w += m.w;
+        W4[i] = w;
+        M4[i] = m;
+    }
+    const long long rest = n - head - 4 * nvec;      // < 4
+    if (tid < head) one(tid);
+    if (tid < rest) one(head + 4 * nvec + tid);
+}
+
 // -------------------------------------------------------------- tiled spmm --
 //
 // Workgroup = 64 output rows x 64 batch columns, 8 waves of T = 8 rows each.
@@ -1474,6 +1512,23 @@ hipError_t launch_axpby(float *W, const float *dW, long long n, float alpha, flo
     if (blocks > 256 * 16) blocks = 256 * 16;         // 16 workgroups per CU, grid-stride beyond that
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(axpby_kernel, dim3((unsigned)blocks), dim3(AXPBY_THREADS), 0, stream, W, dW, n, alpha, beta,
+                       (int)head, (int)vec);
+    return hipGetLastError();
+}
+
+hipError_t launch_momentum(float *W, float *M, const float *dW, long long n, float lr, float mw, float l2,
+                           hipStream_t stream)
+{
+    if (n <= 0) return hipSuccess;
+    const unsigned long long wa = reinterpret_cast<unsigned long long>(W), ma = reinterpret_cast<unsigned long long>(M),
+                             da = reinterpret_cast<unsigned long long>(dW);
+    const bool vec = (wa & 15u) == (da & 15u) && (wa & 15u) == (ma & 15u) && (wa & 3u) == 0 && n >= 8;
+    const long long head = vec ? (long long)(((16u - (wa & 15u)) & 15u) / 4u) : 0;
+    const long long items = vec ? (n - head) / 4 : n;
+    long long blocks = (items + AXPBY_THREADS - 1) / AXPBY_THREADS;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(momentum_kernel, dim3((unsigned)blocks), dim3(AXPBY_THREADS), 0, stream, W, M, dW, n, lr, mw, l2,
                        (int)head, (int)vec);
     return hipGetLastError();
 }

@@ -48,6 +48,10 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, SpEpilogue ep, hipStream_t stream);
 
+// m = mw*M[i] - lr*(dW[i] + l2*W[i]); W[i] += m; M[i] = m, i < n.
+hipError_t launch_momentum(float *W, float *M, const float *dW, long long n, float lr, float mw, float l2,
+                           hipStream_t stream);
+
 // W[i] = alpha*dW[i] + beta*W[i], i < n.
 hipError_t launch_axpby(float *W, const float *dW, long long n, float alpha, float beta, hipStream_t stream);
 

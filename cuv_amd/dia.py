@@ -201,6 +201,26 @@ def learn_step_weight_decay(W, dW, learnrate, decay=0.0, sync=True):
     return W
 
 
+def learn_step_weight_decay_momentum(W, momentum, dW, learnrate, momentum_weight=0.9, decay=0.0, sync=True):
+    """m = momentum_weight*momentum - learnrate*(dW + decay*W); W += m; momentum = m
+    (src/cuv/tensor_ops/rprop.cu:158-170,369-376).  Operands as in learn_step_weight_decay."""
+    w, m, d = (t.vec if isinstance(t, dev_dia_matrix_f) else t for t in (W, momentum, dW))
+    for t in (w, m, d):
+        if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+            raise RuntimeError("W.ptr() / dW.ptr(): contiguous float32 CUDA tensors")
+    if w.numel() != d.numel():
+        raise RuntimeError("W.size() == dW.size()")
+    if w.numel() != m.numel():
+        raise RuntimeError("W.size() == momentum.size()")
+    with torch.cuda.device(w.device):
+        _lib.check(_lib.lib().cuvdia_learn_step_weight_decay_momentum_f32(
+            w.data_ptr(), m.data_ptr(), d.data_ptr(), w.numel(), learnrate, momentum_weight, decay, _stream_ptr()),
+            "cuvdia_learn_step_weight_decay_momentum_f32")
+        if sync:
+            torch.cuda.current_stream().synchronize()
+    return W
+
+
 def to_device_colmajor(a, device="cuda:0"):
     """numpy (rows, batch) array -> torch (batch, rows) contiguous CUDA tensor
     holding the same column-major matrix."""

@@ -26,5 +26,25 @@ inline void learn_step_weight_decay(tensor<float, dev_memory_space, L> &W, const
     cuvSafeCall(hipStreamSynchronize(NULL));
 }
 
+/// m = momentum_weight*momentum - learnrate*(dW + decay*W); W += m; momentum = m  (sparsedecay ignored, as in the
+/// reference's kernel)
+template <class L>
+inline void learn_step_weight_decay_momentum(tensor<float, dev_memory_space, L> &W,
+                                             tensor<float, dev_memory_space, L> &momentum,
+                                             const tensor<float, dev_memory_space, L> &dW, const float &learnrate,
+                                             const float &momentum_weight = 0.9f, const float &decay = 0.0f,
+                                             const float &sparsedecay = 0.0f)
+{
+    (void)sparsedecay;
+    cuvAssert(dW.ptr());
+    cuvAssert(W.ptr());
+    cuvAssert(W.size() == dW.size());
+    cuvAssert(W.size() == momentum.size());
+    checkDiaCall(cuvdia_learn_step_weight_decay_momentum_f32(W.ptr(), momentum.ptr(), dW.ptr(), (long long)W.size(),
+                                                             learnrate, momentum_weight, decay, NULL),
+                 "cuvdia_learn_step_weight_decay_momentum_f32");
+    cuvSafeCall(hipStreamSynchronize(NULL));
+}
+
 }  // namespace cuv
 #endif

@@ -164,6 +164,20 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals_device,
 int cuvdia_learn_step_weight_decay_f32(float *W_device, const float *dW_device, long long n,
                                        float learnrate, float decay, void *stream);
 
+/* m = momentum_weight*momentum[i] - learnrate*(dW[i] + decay*W[i]);
+ * W[i] += m; momentum[i] = m, for i < n: replaces
+ * learn_step_weight_decay_momentum<float,dev_memory_space>
+ * (src/cuv/tensor_ops/rprop.cu:158-170,348-353,369-376, declared in
+ * src/cuv/tensor_ops/rprop.hpp:142-143; sparsedecay is ignored there,
+ * rprop.cu:166-167).  The reference's host loop (rprop.cu:356-367) has the
+ * decay term with the opposite sign; this entry follows the device kernel it
+ * replaces, which is the one that shrinks the weights.  The three arrays must
+ * not overlap.  n == 0 is a no-op. */
+int cuvdia_learn_step_weight_decay_momentum_f32(float *W_device, float *momentum_device,
+                                                const float *dW_device, long long n,
+                                                float learnrate, float momentum_weight,
+                                                float decay, void *stream);
+
 /* C = beta*C + alpha*proj(A*B') restricted to the stored diagonals of C:
  *   C_d[i] = beta*C_d[i] + alpha * sum_c A[i,c] * B[offsets[d] + i/row_fact, c]
  * for every valid slot.  Replaces densedense_to_dia<float,column_major>

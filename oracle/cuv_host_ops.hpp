@@ -113,6 +113,29 @@ inline void learn_step_weight_decay(tensor<float, host_memory_space, L> &W, cons
     for (size_t i = 0; i < (size_t)W.size(); ++i) w[i] = alpha * d[i] + beta * w[i];
 }
 
+// m = momentum_weight*m - learnrate*(dW + decay*W); W += m, following the device kernel
+// (src/cuv/tensor_ops/rprop.cu:158-170), whose decay term shrinks the weights.
+template <class L>
+inline void learn_step_weight_decay_momentum(tensor<float, host_memory_space, L> &W,
+                                             tensor<float, host_memory_space, L> &momentum,
+                                             const tensor<float, host_memory_space, L> &dW, const float &learnrate,
+                                             const float &momentum_weight = 0.9f, const float &decay = 0.0f,
+                                             const float &sparsedecay = 0.0f)
+{
+    (void)sparsedecay;
+    cuvAssert(dW.ptr());
+    cuvAssert(W.ptr());
+    cuvAssert(W.size() == dW.size());
+    cuvAssert(W.size() == momentum.size());
+    float *w = W.ptr(), *mo = momentum.ptr();
+    const float *d = dW.ptr();
+    for (size_t i = 0; i < (size_t)W.size(); ++i) {
+        const float m = momentum_weight * mo[i] - learnrate * (d[i] + decay * w[i]);
+        w[i] += m;
+        mo[i] = m;
+    }
+}
+
 // Dense C = factC*C + factAB*op(A)*op(B), fp64 accumulation: stands in for the
 // CBLAS sgemm the reference cross-checks against (src/cuv/matrix_ops/matrix_ops.cu:177-304).
 inline void prod(tensor<float, host_memory_space, column_major> &dst,

@@ -264,6 +264,17 @@ def learn_step_weight_decay(W, dW, learnrate, decay=0.0):
     return (np.float32(alpha) * dW).astype(np.float32) + (np.float32(beta) * W).astype(np.float32)
 
 
+def learn_step_weight_decay_momentum(W, momentum, dW, learnrate, momentum_weight=0.9, decay=0.0):
+    """src/cuv/tensor_ops/rprop.cu:158-170 (the device kernel; the host loop at rprop.cu:356-367 has the decay
+    term's sign flipped): m = momentum_weight*m - learnrate*(dW + decay*W); W += m.  Returns (W, momentum), every
+    operation rounded to fp32."""
+    f = np.float32
+    W, m, dW = (np.asarray(t, f) for t in (W, momentum, dW))
+    inner = (dW + (f(decay) * W).astype(f)).astype(f)
+    m = ((f(momentum_weight) * m).astype(f) - (f(learnrate) * inner).astype(f)).astype(f)
+    return (W + m).astype(f), m
+
+
 def avg_diagonals(dia):
     out = np.zeros(dia.nd, np.float32)
     lib().oracle_avg_diagonals_f32(dia.h, dia.w, dia.nd, dia.stride,

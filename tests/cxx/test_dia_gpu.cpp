@@ -182,6 +182,36 @@ TEST_CASE(learn_step_weight_decay_dev)
     CHECK_THROWS(learn_step_weight_decay(wd.vec(), shorter, 0.5f));
 }
 
+// With learnrate 0.5, momentum weight 0.5, decay 0.25 and W = 8 i, m = 4 i,
+// dW = 0 every product is exact: m' = 2 i - 0.5*(2 i) = i, W' = 9 i.
+TEST_CASE(learn_step_weight_decay_momentum_dev)
+{
+    const unsigned n = 1000;
+    tensor<float, host_memory_space> w(n), m(n), dw(n);
+    for (unsigned i = 0; i < n; ++i) {
+        w[i] = 8.f * i;
+        m[i] = 4.f * i;
+        dw[i] = 0.f;
+    }
+    tensor<float, dev_memory_space> wd(n), md(n), dwd(n);
+    convert(wd, w);
+    convert(md, m);
+    convert(dwd, dw);
+    learn_step_weight_decay_momentum(wd, md, dwd, 0.5f, 0.5f, 0.25f);
+    learn_step_weight_decay_momentum(w, m, dw, 0.5f, 0.5f, 0.25f);
+    tensor<float, host_memory_space> wb(n), mb(n);
+    convert(wb, wd);
+    convert(mb, md);
+    for (unsigned i = 0; i < n; ++i) {
+        CHECK(wb[i] == 9.f * i);
+        CHECK(mb[i] == 1.f * i);
+        CHECK(wb[i] == w[i]);
+        CHECK(mb[i] == m[i]);
+    }
+    tensor<float, dev_memory_space> shorter(5);
+    CHECK_THROWS(learn_step_weight_decay_momentum(wd, shorter, dwd, 0.5f));
+}
+
 TEST_CASE(spmv_uninit)
 {
     dia_matrix<float, host_memory_space> w(32, 16, 3, 32, 1);

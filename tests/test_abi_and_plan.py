@@ -54,6 +54,9 @@ def test_no_device_is_an_error_not_a_fallback():
     assert L.cuvdia_learn_step_weight_decay_f32(None, None, -1, 0.1, 0.0, None) == _lib.EINVAL
     assert L.cuvdia_learn_step_weight_decay_f32(None, None, 0, 0.1, 0.0, None) == 0
     assert L.cuvdia_learn_step_weight_decay_f32(None, None, 4, 0.1, 0.0, None) == _lib.EINVAL
+    assert L.cuvdia_learn_step_weight_decay_momentum_f32(None, None, None, -1, 0.1, 0.9, 0.0, None) == _lib.EINVAL
+    assert L.cuvdia_learn_step_weight_decay_momentum_f32(None, None, None, 0, 0.1, 0.9, 0.0, None) == 0
+    assert L.cuvdia_learn_step_weight_decay_momentum_f32(None, None, None, 4, 0.1, 0.9, 0.0, None) == _lib.EINVAL
     assert L.cuvdia_spmm_layer_f32(None, None, None, 0, None, 0, 1, b"n", 1.0, 0.0, None, 7, 0, None) == _lib.EINVAL
     assert L.cuvdia_spmm_bias_act_f32(None, None, None, 0, None, 0, 1, b"n", 1.0, 0.0, None,
                                       _lib.ACT_SIGMOID_SAMPLE, None) == _lib.EINVAL

@@ -605,6 +605,56 @@ def test_learn_step_weight_decay(oracle, n, shift_w, shift_d):
     assert np.array_equal(dv.cpu().numpy(), dW)
 
 
+@pytest.mark.parametrize("n,shift", [(1, 0), (7, 0), (4096, 0), (100003, 1), (100003, (3, 2, 1)), (49 * 16384, 0)])
+def test_learn_step_weight_decay_momentum(oracle, n, shift):
+    """m = mw*m - lr*(dW + decay*W); W += m (rprop.cu:158-170) against the fp32
+    host restatement.  The GPU may contract decay*W + dW and mw*m - lr*(...)
+    into FMAs, each saving one rounding: tolerance 2e-6 * (|mw*m| + lr*|dW| +
+    lr*decay*|W|) on m and that plus 1e-6*|W| on W.  Aligned, equally and
+    mutually misaligned arrays; bytes around them stay untouched."""
+    import torch
+    from cuv_amd import dia as D
+    sw, sm, sd = shift if isinstance(shift, tuple) else (shift, shift, shift)
+    rng = np.random.default_rng(n + sw)
+    W = rng.normal(0, 0.01, n).astype(np.float32)
+    M = rng.normal(0, 0.01, n).astype(np.float32)
+    dW = rng.normal(0, 1.0, n).astype(np.float32)
+    lr, mw, decay = 0.05, 0.9, 0.002
+    ref_w, ref_m = oracle.learn_step_weight_decay_momentum(W, M, dW, lr, mw, decay)
+    bufs = [torch.full((n + 16,), fill, device="cuda:0") for fill in (123.0, 55.0, -7.0)]
+    wv, mv, dv = (b[4 + s:4 + s + n] for b, s in zip(bufs, (sw, sm, sd)))
+    for v, h in ((wv, W), (mv, M), (dv, dW)):
+        v.copy_(torch.from_numpy(h))
+    D.learn_step_weight_decay_momentum(wv, mv, dv, lr, mw, decay)
+    W64, M64, d64 = (a.astype(np.float64) for a in (W, M, dW))
+    tol_m = 2e-6 * (np.abs(mw * M64) + lr * np.abs(d64) + lr * decay * np.abs(W64)) + 1e-30
+    got_m, got_w = mv.cpu().numpy(), wv.cpu().numpy()
+    assert np.all(np.abs(got_m.astype(np.float64) - ref_m) <= tol_m)
+    assert np.all(np.abs(got_w.astype(np.float64) - ref_w) <= tol_m + 1e-6 * np.abs(W64))
+    for b, s, fill in zip(bufs, (sw, sm, sd), (123.0, 55.0, -7.0)):
+        host = b.cpu().numpy()
+        assert np.all(host[:4 + s] == fill) and np.all(host[4 + s + n:] == fill)
+    assert np.array_equal(dv.cpu().numpy(), dW)
+
+
+def test_momentum_steps_reach_the_optimum():
+    """The reference's own check of this update (src/tests/optimize.cpp:89-123), on
+    the device: 1000 steps on f(W) = 2 (W - optimum)^2, learnrate 0.01, momentum
+    weight 1 - iter/1000, end within 0.01% of the optimum."""
+    import torch
+    from cuv_amd import dia as D
+    g = torch.Generator(device="cpu").manual_seed(3)
+    optimum = torch.rand(100, generator=g).cuda()
+    W = torch.rand(100, generator=g).cuda()
+    mom = torch.zeros(100, device="cuda:0")
+    for it in range(1000):
+        D.learn_step_weight_decay_momentum(W, mom, W - optimum, 0.01, 1.0 - it / 1000.0, 0.0, sync=False)
+    torch.cuda.synchronize()
+    assert not torch.isnan(W).any()
+    assert torch.all(((W + 1) - (optimum + 1)).abs() <= 1e-4 * (optimum + 1))
+    assert float((2 * (W - optimum) ** 2).mean()) <= 1e-4
+
+
 def test_weight_update_fused_into_the_projection(oracle, gu):
     """examples/rbm/base.py:71-81: w_tmp = proj(v0*h0') ; w_tmp = -1/b*proj(v1*h1') + 1/b*w_tmp ;
     W = -lr*w_tmp + (1 - lr*cost)*W.  The same update in two projection calls

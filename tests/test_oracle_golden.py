@@ -320,3 +320,35 @@ def test_learn_step_weight_decay_closed_form(oracle):
     got = oracle.learn_step_weight_decay(8 * i, 2 * i, 0.5, 0.25)
     assert got.dtype == np.float32 and np.array_equal(got, 6 * i)
     assert np.array_equal(oracle.learn_step_weight_decay(i, i, 0.0, 3.0), i)
+
+
+def test_learn_step_weight_decay_momentum_pins(oracle):
+    """Three checks of the momentum step (rprop.cu:158-170).
+    Exact arithmetic: lr 0.5, momentum weight 0.5, decay 0.25, W = 8 i, m = 4 i, dW = 2 i give
+    m' = 2 i - 0.5*(2 i + 2 i) = 0 and W' = W; with dW = 0 instead m' = 2 i - i = i, W' = 9 i.
+    Reduction: without momentum the step is learn_step_weight_decay (rprop.cu:341-346), whose decay shrinks
+    the weights -- the sign the host loop at rprop.cu:364 gets wrong.
+    The reference's own test (src/tests/optimize.cpp:89-123): 1000 steps on f(W) = 2 (W - optimum)^2 with
+    learnrate 0.01 and momentum weight 1 - iter/1000 end within 0.01% of the optimum."""
+    i = np.arange(1000, dtype=np.float32)
+    W, m = oracle.learn_step_weight_decay_momentum(8 * i, 4 * i, 2 * i, 0.5, 0.5, 0.25)
+    assert np.array_equal(W, 8 * i) and np.array_equal(m, 0 * i)
+    W, m = oracle.learn_step_weight_decay_momentum(8 * i, 4 * i, 0 * i, 0.5, 0.5, 0.25)
+    assert np.array_equal(W, 9 * i) and np.array_equal(m, i)
+
+    rng = np.random.default_rng(5)
+    W0 = rng.normal(0, 1, 4096).astype(np.float32)
+    dW = rng.normal(0, 1, 4096).astype(np.float32)
+    W, m = oracle.learn_step_weight_decay_momentum(W0, np.zeros_like(W0), dW, 0.05, 0.0, 0.002)
+    plain = oracle.learn_step_weight_decay(W0, dW, 0.05, 0.002)
+    assert np.allclose(W, plain, rtol=0, atol=4e-7 * (np.abs(W0) + 0.05 * np.abs(dW)).max())
+    assert np.array_equal(m, (W - W0).astype(np.float32)) or np.allclose(m, W - W0, rtol=0, atol=2e-7)
+
+    optimum = rng.random(100).astype(np.float32)
+    W = rng.random(100).astype(np.float32)
+    mom = np.zeros(100, np.float32)
+    for it in range(1000):
+        W, mom = oracle.learn_step_weight_decay_momentum(W, mom, (W - optimum).astype(np.float32), 0.01,
+                                                         1.0 - it / 1000.0, 0.0)
+    assert np.all(np.abs((W + 1) - (optimum + 1)) <= 1e-4 * (optimum + 1))
+    assert abs(float(np.mean(2 * (W - optimum) ** 2))) <= 1e-4
