@@ -721,3 +721,92 @@ def test_dia_file_round_trip_device(oracle, gu, tmp_path):
     D.prod(y0, dev, B)
     D.prod(y1, back, B)
     assert torch.equal(y0, y1)
+
+
+# --------------------------------------------------- streams and HIP graphs ---
+def _layer_state(oracle, rng, n=2048, batch=96):
+    import torch
+    from cuv_amd import dia as D
+    offs = [dy * 64 + dx for dy in range(-3, 4) for dx in range(-3, 4)]
+    host = _rand_dia(oracle, rng, n, n, offs, pad=0.0, lo=-0.05, hi=0.05)
+
+    def dev():
+        m = D.dev_dia_matrix_f(n, n, len(offs), host.stride)
+        m.set_offsets(host.offsets)
+        return m
+
+    W, G, M = dev().push(host.vals), dev(), dev()
+    for m in (W, G, M):
+        m.desc                                             # descriptors are built outside any capture
+    v0 = torch.from_numpy((rng.random((batch, n)) < 0.3).astype(np.float32)).cuda()
+    return dict(W=W, G=G, M=M, v0=v0, h0=torch.empty(batch, n, device="cuda:0"),
+                v1=torch.empty(batch, n, device="cuda:0"), bias=torch.zeros(n, device="cuda:0"))
+
+
+def _cd_step(s, seed):
+    """One contrastive-divergence-shaped pass over a DIA layer: sampled up-pass,
+    down-pass, gradient, momentum step; every call on the current stream."""
+    from cuv_amd import _lib, dia as D
+    D.prod_bias_act(s["h0"], s["W"], s["v0"], "n", 1.0, 0.0, s["bias"], _lib.ACT_SIGMOID_SAMPLE, seed, sync=False)
+    D.prod_bias_act(s["v1"], s["W"], s["h0"], "t", 1.0, 0.0, s["bias"], _lib.ACT_SIGMOID, sync=False)
+    D.densedense_to_dia(s["G"], None, s["h0"], s["v0"], -1.0 / s["v0"].shape[0], 0.0, sync=False)
+    D.densedense_to_dia(s["G"], None, s["h0"], s["v1"], 1.0 / s["v0"].shape[0], 1.0, sync=False)
+    D.learn_step_weight_decay_momentum(s["W"], s["M"], s["G"], 0.1, 0.5, 0.001, sync=False)
+
+
+def test_graph_replays_match_eager_calls(oracle):
+    """The entry points only launch kernels on the caller's stream, so a
+    training pass can be captured into a HIP graph.  Three replays, with eager
+    work and synchronisations of the program between them, must each leave
+    exactly the state the same calls made eagerly leave."""
+    import torch
+    eager = _layer_state(oracle, np.random.default_rng(77))
+    graph = _layer_state(oracle, np.random.default_rng(77))
+    assert torch.equal(eager["W"].vec, graph["W"].vec) and torch.equal(eager["v0"], graph["v0"])
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        _cd_step(graph, 5)                                 # warm-up on the capture stream, outside the graph
+    side.synchronize()
+    _cd_step(eager, 5)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        _cd_step(graph, 5)
+    for replay in range(3):
+        g.replay()
+        _cd_step(eager, 5)
+        torch.cuda.synchronize()
+        filler = torch.rand(1 << 20, device="cuda:0").sum().item()      # unrelated eager work between replays
+        assert filler > 0
+        for k in ("h0", "v1"):
+            assert torch.equal(eager[k], graph[k]), (replay, k)
+        for k in ("W", "G", "M"):
+            assert torch.equal(eager[k].vec, graph[k].vec), (replay, k)
+    assert float(graph["M"].vec.abs().max()) > 0
+
+
+def test_calls_run_on_the_callers_stream(oracle):
+    """Work is ordered with the stream handed in, not with the null stream: a
+    product issued on a side stream right behind a long-running fill of its
+    operand on that stream sees the filled operand."""
+    import torch
+    from cuv_amd import dia as D
+    rng = np.random.default_rng(9)
+    A = _rand_dia(oracle, rng, 4096, 4096, list(range(-3, 4)), pad=0.0)
+    dA = D.dev_dia_matrix_f(4096, 4096, 7, A.stride)
+    dA.set_offsets(A.offsets)
+    dA.push(A.vals)
+    dA.desc
+    side = torch.cuda.Stream()
+    B = torch.zeros(64, 4096, device="cuda:0")
+    dst = torch.full((64, 4096), float("nan"), device="cuda:0")
+    big = torch.empty(1 << 28, device="cuda:0")
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(4):
+            big.fill_(1.0)                                 # keeps the side stream busy for a while
+        B.fill_(1.0)
+        D.prod(dst, dA, B, "n", "n", 1.0, 0.0, sync=False)
+    side.synchronize()
+    ref = oracle.prod(A, np.ones((4096, 64), np.float32, order="F"), None, "n", 1.0, 0.0)
+    got = D.to_host_colmajor(dst)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-6)
