@@ -1,6 +1,6 @@
 """Seeded random sweep: both kernel families of the HIP path against the CPU
 oracle on shapes nobody picked by hand -- ragged sizes, shuffled, duplicate and
-out-of-range offsets, operands that are misaligned views of wider allocations
+out-of-range offsets, steep matrices (row factor 2-4), operands that are misaligned views of wider allocations
 (any leading dimension, base address not a multiple of 16 bytes), beta == 0 over
 NaN destinations.  Tolerance as in test_gpu_parity (1e-5 of the summed
 magnitudes); bytes around the destination view must stay as they were.
@@ -54,12 +54,14 @@ def _one_case(oracle, seed, lo, hi):
     alpha = float(rng.choice([1.0, -0.5, 2.25]))
     beta = float(rng.choice([0.0, 0.0, 1.0, -1.5]))
     stride = max(h, w) + (int(rng.integers(0, 7)) if rng.random() < 0.5 else 0)
-    A = oracle.Dia(h, w, offs, stride, 1)
+    rf = int(rng.choice([2, 3, 4])) if rng.random() < 0.15 else 1        # steep matrices: the generic kernels only
+    A = oracle.Dia(h, w, offs, stride, rf)
     A.vals[:] = np.nan
     valid = oracle.valid_mask(A)
     A.vals[valid] = rng.uniform(-1, 1, int(valid.sum())).astype(np.float32)
     Ad = gu.make_dev_dia(A)
-    what = "seed %d: %dx%d, %d offsets, batch %d, alpha %g, beta %g" % (seed, h, w, len(offs), batch, alpha, beta)
+    what = "seed %d: %dx%d, row factor %d, %d offsets, batch %d, alpha %g, beta %g" % (
+        seed, h, w, rf, len(offs), batch, alpha, beta)
 
     def forced(path, call):
         """runs call() on the given kernel family; False when the tiled family does not take the shape"""
@@ -92,11 +94,11 @@ def _one_case(oracle, seed, lo, hi):
 
     P = np.asfortranarray(rng.uniform(-1, 1, (h, batch)).astype(np.float32))
     Q = np.asfortranarray(rng.uniform(-1, 1, (w, batch)).astype(np.float32))
-    C = oracle.Dia(h, w, offs, stride, 1, A.vals.copy())
+    C = oracle.Dia(h, w, offs, stride, rf, A.vals.copy())
     if beta == 0:
         C.vals[valid] = np.nan
     ref = oracle.dd2dia(C, P, Q, alpha, beta)
-    mag = oracle.dd2dia_f64(oracle.Dia(h, w, offs, stride, 1, np.abs(np.nan_to_num(C.vals))),
+    mag = oracle.dd2dia_f64(oracle.Dia(h, w, offs, stride, rf, np.abs(np.nan_to_num(C.vals))),
                             np.abs(P), np.abs(Q), abs(alpha), abs(beta))
     for path in (_lib.PATH_GENERIC, _lib.PATH_TILED):
         Cd = gu.make_dev_dia(C)
