@@ -125,13 +125,13 @@ int cuvdia_set_path(int path)
 
 int cuvdia_last_path(void) { return t_last_path; }
 
-int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
-                       int *s0, int *len, int *slot, int cap)
+int cuvdia_plan_chunks_max(const int *offsets_host, int nd, int transposed, int max_len,
+                           int *s0, int *len, int *slot, int cap)
 {
-    if (!offsets_host || nd < 1) return CUVDIA_EINVAL;
+    if (!offsets_host || nd < 1 || max_len < 1 || max_len > SP_CHUNK_MAX) return CUVDIA_EINVAL;
     std::vector<Chunk> ch;
     try {
-        ch = plan_chunks(offsets_host, nd, transposed != 0);
+        ch = plan_chunks(offsets_host, nd, transposed != 0, max_len);
     } catch (const std::bad_alloc &) {
         return CUVDIA_ENOMEM;
     }
@@ -140,10 +140,16 @@ int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
         for (int c = 0; c < n; ++c) {
             s0[c] = ch[c].s0;
             len[c] = ch[c].len;
-            for (int j = 0; j < CHUNK_MAX; ++j) slot[c * CHUNK_MAX + j] = j < ch[c].len ? ch[c].slot[j] : -1;
+            for (int j = 0; j < max_len; ++j) slot[c * max_len + j] = j < ch[c].len ? ch[c].slot[j] : -1;
         }
     }
     return n;
+}
+
+int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
+                       int *s0, int *len, int *slot, int cap)
+{
+    return cuvdia_plan_chunks_max(offsets_host, nd, transposed, CHUNK_MAX, s0, len, slot, cap);
 }
 
 int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap)
@@ -182,15 +188,16 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     }
 
     cuvdia_desc *d = nullptr;
-    std::vector<Chunk> cn, ct;
+    std::vector<Chunk> cn, ct, cp;
     std::vector<Unit> un, us;
     try {
         d = new cuvdia_desc();
         d->offsets.assign(offsets_host, offsets_host + nd);
-        cn = plan_chunks(offsets_host, nd, false);
-        ct = plan_chunks(offsets_host, nd, true);
-        un = plan_units(cn);
-        for (int c = 0; c < (int)cn.size(); ++c) us.push_back(Unit{c, -1});
+        cn = plan_chunks(offsets_host, nd, false, SP_CHUNK_MAX);
+        ct = plan_chunks(offsets_host, nd, true, SP_CHUNK_MAX);
+        cp = plan_chunks(offsets_host, nd, false, CHUNK_MAX);
+        un = plan_units(cp);
+        for (int c = 0; c < (int)cp.size(); ++c) us.push_back(Unit{c, -1});
     } catch (const std::bad_alloc &) {
         delete d;
         return CUVDIA_ENOMEM;
@@ -202,16 +209,19 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     d->dev_block = nullptr;
     if ((e = hipGetDevice(&d->device)) != hipSuccess) { delete d; return hip_fail(e, "hipGetDevice"); }
 
-    // one device block: offsets (padded to 64 B) | chunks_n | chunks_t | units | one unit per chunk
+    // one device block: offsets (padded to 64 B) | chunks_n | chunks_t | projection chunks | units | one unit per chunk
     const size_t off_bytes = ((size_t)nd * sizeof(int) + 63) / 64 * 64;
     const size_t cn_bytes = cn.size() * sizeof(Chunk), ct_bytes = ct.size() * sizeof(Chunk);
+    const size_t cp_bytes = cp.size() * sizeof(Chunk);
     const size_t un_bytes = un.size() * sizeof(Unit), us_bytes = us.size() * sizeof(Unit);
-    std::vector<unsigned char> staging(off_bytes + cn_bytes + ct_bytes + un_bytes + us_bytes, 0);
+    const size_t cp_at = off_bytes + cn_bytes + ct_bytes, un_at = cp_at + cp_bytes, us_at = un_at + un_bytes;
+    std::vector<unsigned char> staging(us_at + us_bytes, 0);
     std::memcpy(staging.data(), offsets_host, (size_t)nd * sizeof(int));
     std::memcpy(staging.data() + off_bytes, cn.data(), cn_bytes);
     std::memcpy(staging.data() + off_bytes + cn_bytes, ct.data(), ct_bytes);
-    std::memcpy(staging.data() + off_bytes + cn_bytes + ct_bytes, un.data(), un_bytes);
-    std::memcpy(staging.data() + off_bytes + cn_bytes + ct_bytes + un_bytes, us.data(), us_bytes);
+    std::memcpy(staging.data() + cp_at, cp.data(), cp_bytes);
+    std::memcpy(staging.data() + un_at, un.data(), un_bytes);
+    std::memcpy(staging.data() + us_at, us.data(), us_bytes);
     if ((e = hipMalloc(&d->dev_block, staging.size())) != hipSuccess) {
         delete d;
         return e == hipErrorOutOfMemory ? CUVDIA_ENOMEM : hip_fail(e, "hipMalloc(descriptor)");
@@ -227,8 +237,9 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
                       reinterpret_cast<const Chunk *>(base + off_bytes), d->n_chunks_n,
                       reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t,
                       0, 0, 0, 0, 0, 0,
-                      reinterpret_cast<const Unit *>(base + off_bytes + cn_bytes + ct_bytes), (int)un.size(),
-                      reinterpret_cast<const Unit *>(base + off_bytes + cn_bytes + ct_bytes + un_bytes)};
+                      reinterpret_cast<const Chunk *>(base + cp_at), (int)cp.size(), 0,
+                      reinterpret_cast<const Unit *>(base + un_at), (int)un.size(),
+                      reinterpret_cast<const Unit *>(base + us_at)};
     auto span = [](const std::vector<Chunk> &t, int &max_len, int &s_min, int &s_max) {
         max_len = 0;
         s_min = t.empty() ? 0 : t.front().s0;
@@ -241,6 +252,8 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     };
     span(cn, d->view.max_len_n, d->view.s_min_n, d->view.s_max_n);
     span(ct, d->view.max_len_t, d->view.s_min_t, d->view.s_max_t);
+    int unused_min = 0, unused_max = 0;
+    span(cp, d->view.max_len_p, unused_min, unused_max);
     *out = d;
     return CUVDIA_OK;
 }

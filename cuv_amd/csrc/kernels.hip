@@ -341,7 +341,8 @@ constexpr int SP_GROUPS = (SP_COLS + SP_CPI - 1) / SP_CPI;             // 22 col
 constexpr int SP_PITCH = 84;       // floats between staged columns
 constexpr int SP_OPITCH = 68;      // floats between columns in the epilogue
 constexpr int SP_XFLOATS = SP_COLS * SP_PITCH;
-constexpr int SP_AVALS = CHUNK_MAX * SP_ROWS;   // diagonal values per workgroup per chunk
+constexpr int SP_ADIAGS = 16;      // diagonals a chunk's LDS block has room for (>= SP_CHUNK_MAX)
+constexpr int SP_AVALS = SP_ADIAGS * SP_ROWS;   // diagonal values per workgroup per chunk
 constexpr int SP_DUMP = SP_XFLOATS + SP_AVALS;  // where idle lanes write
 constexpr int SP_STAGE_FLOATS = SP_DUMP + 4;
 constexpr int SP_MAX_CHUNKS = 256;   // chunk-table entries a wave can keep in registers (4 sets of 64)
@@ -353,24 +354,24 @@ struct SpShape {
     static_assert(T == 8 || T == 16, "rows per wave");
     static constexpr int WAVES = SP_ROWS / T;
     static constexpr int LOADS = (SP_GROUPS + WAVES - 1) / WAVES;      // 16-byte loads per wave per chunk
-    static constexpr int APW = CHUNK_MAX / WAVES;                      // diagonals each wave fetches per chunk
     static constexpr int CPW = SP_COLS / WAVES;                        // columns each wave stores in the epilogue
 };
 
-template <int T>
+// APW: diagonals each wave fetches per chunk, ceil(LCK / waves)
+template <int T, int APW>
 struct SpStage {
     float4 x[SpShape<T>::LOADS];
-    float a[SpShape<T>::APW];
+    float a[APW];
     int shift;              // rows the pieces were fetched away from their place (0 except at the operand's ends)
     bool edge;              // some staged row does not exist (wave-uniform)
 };
 
 // One chunk-table entry as a wave needs it: shift, length, and the table
 // positions of the diagonals this wave fetches.
-template <int T>
+template <int APW>
 struct SpInfo {
     int s0, len;
-    int slot[SpShape<T>::APW];
+    int slot[APW];
 };
 
 template <int LCK, int T>
@@ -474,7 +475,9 @@ __device__ __forceinline__ void spmm_tile_edge(
     int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, SpEpilogue ep)
 {
     typedef SpShape<T> S;
-    constexpr int SP_WAVES = S::WAVES, SP_LOADS = S::LOADS, SP_APW = S::APW, SP_CPW = S::CPW, SP_T = T;
+    constexpr int SP_WAVES = S::WAVES, SP_LOADS = S::LOADS, SP_APW = (LCK + S::WAVES - 1) / S::WAVES, SP_CPW = S::CPW, SP_T = T;
+    typedef SpStage<T, SP_APW> Stage;
+    typedef SpInfo<SP_APW> Info;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     float acc[SP_T];
@@ -530,9 +533,9 @@ __device__ __forceinline__ void spmm_tile_edge(
         tab_s0[k] = e[0];
         tab_len[k] = e[1];
 #pragma unroll
-        for (int q = 0; q < SP_APW; ++q) tab_slot[k][q] = e[2 + wave + SP_WAVES * q];
+        for (int q = 0; q < SP_APW; ++q) tab_slot[k][q] = wave + SP_WAVES * q < CHUNK_SLOTS ? e[2 + wave + SP_WAVES * q] : -1;
     }
-    auto fetch_info = [&](int c, SpInfo<T> &info) {
+    auto fetch_info = [&](int c, Info &info) {
         const int cc = min(c, nchunks - 1);
         const int l = cc & 63;
         info.s0 = __builtin_amdgcn_readlane(tab_s0[0], l);
@@ -557,7 +560,7 @@ __device__ __forceinline__ void spmm_tile_edge(
     // first or last row is fetched from the nearest in-range position instead
     // (rows rc..rc+3) and shifted into place when it is written to LDS, so the
     // loads themselves never branch.
-    auto issue = [&](const SpInfo<T> &info, SpStage<T> &st, int c) {
+    auto issue = [&](const Info &info, Stage &st, int c) {
         const int s0 = info.s0;
         const int a0 = row0 + s0;
         const int r = a0 + 4 * quad;                       // first dense row of this lane's piece
@@ -580,7 +583,7 @@ __device__ __forceinline__ void spmm_tile_edge(
             st.a[q] = buffer_load_f32(ar, ok ? off : OOB_OFFSET);
         }
     };
-    auto commit = [&](const SpStage<T> &st, float *buf) {
+    auto commit = [&](const Stage &st, float *buf) {
         if (!st.edge) {
 #pragma unroll
             for (int it = 0; it < SP_LOADS; ++it)
@@ -617,8 +620,8 @@ __device__ __forceinline__ void spmm_tile_edge(
     // Nothing in an iteration is conditional: past the end of the table the
     // last chunk is staged again (and never used), so the number of loads in
     // flight is the same on every path and each wait counts exactly.
-    auto iteration = [&](int c, SpStage<T> &next, SpWindow<LCK, T> &win_cur, SpWindow<LCK, T> &win_next,
-                         SpInfo<T> &info, SpInfo<T> &info_next) {
+    auto iteration = [&](int c, Stage &next, SpWindow<LCK, T> &win_cur, SpWindow<LCK, T> &win_next,
+                         Info &info, Info &info_next) {
         commit(next, lds[(c + 1) & 1]);
         fetch_info(c + 4, info_next);
         issue(info, next, c + 3);
@@ -627,9 +630,9 @@ __device__ __forceinline__ void spmm_tile_edge(
         read_window(win_next, lds[(c + 1) & 1]);
     };
 
-    SpStage<T> st0, st1;
+    Stage st0, st1;
     SpWindow<LCK, T> w0, w1;
-    SpInfo<T> i0, i1;
+    Info i0, i1;
     fetch_info(0, i0);
     fetch_info(1, i1);
     issue(i0, st0, 0);
@@ -645,9 +648,9 @@ __device__ __forceinline__ void spmm_tile_edge(
         // odd table: one chunk alone first, then the register sets trade
         // places so the paired loop below starts in its usual state
         iteration(0, st1, w0, w1, i1, i0);
-        { const SpStage<T> t = st0; st0 = st1; st1 = t; }
+        { const Stage t = st0; st0 = st1; st1 = t; }
         { const SpWindow<LCK, T> t = w0; w0 = w1; w1 = t; }
-        { const SpInfo<T> t = i0; i0 = i1; i1 = t; }
+        { const Info t = i0; i0 = i1; i1 = t; }
         c = 1;
     }
     for (; c < nchunks; c += 2) {
@@ -732,7 +735,8 @@ constexpr int SP_DQUADS = 19;                       // pieces per column staged 
 constexpr int SP_DPITCH = 4 * SP_DQUADS;            // floats between staged columns
 constexpr int SP_DAVALS = SP_COLS * SP_DPITCH;      // diagonal values sit behind the dense rows
 constexpr int SP_DSTAGE_FLOATS = SP_DAVALS + SP_AVALS;
-static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + CHUNK_MAX - 1 <= SP_DPITCH, "staging layout");
+static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + SP_CHUNK_MAX - 1 <= SP_DPITCH && SP_CHUNK_MAX <= SP_ADIAGS,
+              "staging layout");
 
 template <int LCK, int NTAB, bool EP>
 __device__ __forceinline__ void spmm_tile_lean(
@@ -799,10 +803,11 @@ __device__ __forceinline__ void spmm_tile_lean(
     // occupies the memory pipeline equally long whether it moves 4 or 16 bytes
     // per lane, so the count per chunk -- 21 -- is what matters.
     const bool x3 = wave < SP_DQUADS - 2 * WAVES;
-    const bool a_wave = (wave == 3) | (wave == 4);
-    const int a_j = 4 * (wave - 3) + (lane >> 4);          // the diagonal this lane fetches (waves 3, 4)
-    // every wave keeps its own count of loads per chunk: 3 for waves 0-4, 2 for the others
-    const bool three = wave < 5;
+    constexpr int A_LOADS = LCK > 8 ? 4 : 2;               // instructions that fetch diagonals: waves 3 .. 3 + A_LOADS - 1
+    const bool a_wave = (wave >= 3) & (wave < 3 + A_LOADS);
+    const int a_j = 4 * (wave - 3) + (lane >> 4);          // the diagonal this lane fetches (those waves)
+    // every wave keeps its own count of loads per chunk: 3 for waves 0 .. 2 + A_LOADS, 2 for the others
+    const bool three = wave < 3 + A_LOADS;
 
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
     constexpr unsigned BUF_BYTES = SP_DSTAGE_FLOATS * 4u;
@@ -813,14 +818,19 @@ __device__ __forceinline__ void spmm_tile_lean(
     // kernel's start and its first requests, and the loop's entries arrive
     // under the wait that ends every iteration anyway.
     struct Entry {
-        int s0, len, p0, p1, p2, p3, p4, p5, p6, p7;     // shift, length, table positions of the 8 diagonals
+        int s0, len, p0, p1, p2, p3, p4, p5, p6, p7, p8, p9, p10, p11, p12;     // shift, length, table positions
     };
     auto fetch = [&](int c) __attribute__((always_inline)) {
         typedef int sp_i4 __attribute__((ext_vector_type(4)));
         typedef const sp_i4 __attribute__((address_space(4))) *sc_i4_ptr;
         const sc_i4_ptr e = (sc_i4_ptr)(chunks + min(c, nchunks - 1));
         const sp_i4 e0 = e[0], e1 = e[1], e2 = e[2];
-        return Entry{e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w, e2.x, e2.y};
+        if constexpr (LCK > 8) {
+            const sp_i4 e3 = e[3];
+            return Entry{e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w, e2.x, e2.y, e2.z, e2.w, e3.x, e3.y, e3.z};
+        } else {
+            return Entry{e0.x, e0.y, e0.z, e0.w, e1.x, e1.y, e1.z, e1.w, e2.x, e2.y, -1, -1, -1, -1, -1};
+        }
     };
     // requests chunk c, whose entry is en, into the buffer at byte address `buf`: 3 or 2 loads
     auto issue = [&](int c, unsigned buf, const Entry &en) __attribute__((always_inline)) {
@@ -837,12 +847,13 @@ __device__ __forceinline__ void spmm_tile_lean(
         if (a_wave) {
             // table position of this lane's diagonal, a_j: picked from the 8 scalars (each passed through an
             // empty asm so that the chain of selects stays one, and the entry stays in registers)
-            int p[CHUNK_MAX] = {en.p0, en.p1, en.p2, en.p3, en.p4, en.p5, en.p6, en.p7};
+            constexpr int NP = LCK > 8 ? SP_CHUNK_MAX : 8;
+            int p[SP_CHUNK_MAX] = {en.p0, en.p1, en.p2, en.p3, en.p4, en.p5, en.p6, en.p7, en.p8, en.p9, en.p10, en.p11, en.p12};
 #pragma unroll
-            for (int k = 0; k < CHUNK_MAX; ++k) asm("" : "+s"(p[k]));
+            for (int k = 0; k < NP; ++k) asm("" : "+s"(p[k]));
             int sl = p[0];
 #pragma unroll
-            for (int k = 1; k < CHUNK_MAX; ++k) sl = a_j == k ? p[k] : sl;
+            for (int k = 1; k < NP; ++k) sl = a_j == k ? p[k] : sl;
             const bool ok = real & (a_j < en.len) & (sl >= 0);
             const int arow = row0 + erow + (ashift ? s0 + a_j : 0);          // first of the lane's 4 rows of its diagonal
             const unsigned voff = ok ? ((unsigned)sl * (unsigned)stride + (unsigned)arow) * 4u : OOB_OFFSET;
@@ -958,7 +969,7 @@ __device__ __forceinline__ void spmm_tile_lean(
 
 // EP = false: the plain product (no bias, no activation); EP = true applies `ep`.
 template <int LCK, int T, int NTAB, bool EP>
-__global__ __launch_bounds__(64 * SpShape<T>::WAVES) void spmm_tiled_kernel(
+__global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes,
@@ -1466,6 +1477,8 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     switch (lck) {
         CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
         CUVDIA_SPMM_LAUNCH(5) CUVDIA_SPMM_LAUNCH(6) CUVDIA_SPMM_LAUNCH(7) CUVDIA_SPMM_LAUNCH(8)
+        CUVDIA_SPMM_LAUNCH(9) CUVDIA_SPMM_LAUNCH(10) CUVDIA_SPMM_LAUNCH(11) CUVDIA_SPMM_LAUNCH(12)
+        CUVDIA_SPMM_LAUNCH(13)
         default: return hipErrorInvalidValue;
     }
 #undef CUVDIA_SPMM_LAUNCH
@@ -1540,7 +1553,7 @@ bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch)
     const long long a_bytes = ((nb - 1) * lda + C.h) * 4;
     const long long b_bytes = ((nb - 1) * ldb + C.w) * 4;
     const long long c_bytes = (long long)C.nd * C.stride * 4;
-    return C.rf == 1 && C.max_len_n >= 1 && a_bytes < (long long)OOB_OFFSET &&
+    return C.rf == 1 && C.max_len_p >= 1 && a_bytes < (long long)OOB_OFFSET &&
            b_bytes < (long long)OOB_OFFSET && c_bytes < (long long)OOB_OFFSET;
 }
 
@@ -1563,14 +1576,14 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     // without pairs the units are the chunks themselves, in table order
     // (pairs only with 16-byte loads of A: the dword-load variant of the pair
     // body needs more registers than a wave has)
-    const bool use_units = C.n_units < C.n_chunks_n && a_vec && !g_dd2dia_no_pairs;
+    const bool use_units = C.n_units < C.n_chunks_p && a_vec && !g_dd2dia_no_pairs;
     const bool pairs = use_units;
     const Unit *units = use_units ? C.units_dev : C.single_units_dev;
-    const int nunits = use_units ? C.n_units : C.n_chunks_n;
+    const int nunits = use_units ? C.n_units : C.n_chunks_p;
     const long long blocks = row_tiles * nunits;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks);
-#define CUVDIA_DD_ARGS C.chunks_n_dev, units, nunits, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
+#define CUVDIA_DD_ARGS C.chunks_p_dev, units, nunits, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
                        a_bytes, b_bytes, c_bytes
 #define CUVDIA_DD_LAUNCH(L)                                                                              \
     case L:                                                                                              \
@@ -1581,7 +1594,7 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
             else hipLaunchKernelGGL((dd2dia_tiled_kernel<L, false, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);       \
         }                                                                                                \
         break;
-    switch (C.max_len_n) {
+    switch (C.max_len_p) {
         CUVDIA_DD_LAUNCH(1) CUVDIA_DD_LAUNCH(2) CUVDIA_DD_LAUNCH(3) CUVDIA_DD_LAUNCH(4)
         CUVDIA_DD_LAUNCH(5) CUVDIA_DD_LAUNCH(6) CUVDIA_DD_LAUNCH(7) CUVDIA_DD_LAUNCH(8)
         default: return hipErrorInvalidValue;

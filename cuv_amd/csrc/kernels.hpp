@@ -11,13 +11,16 @@ namespace cuvdia {
 struct DiaView {
     int h, w, nd, stride, rf;
     const int *offsets_dev;      // nd ints, table order
-    const Chunk *chunks_n_dev;   // shifts = offsets
+    const Chunk *chunks_n_dev;   // the products' tables (chunks of up to SP_CHUNK_MAX): shifts = offsets
     int n_chunks_n;
     const Chunk *chunks_t_dev;   // shifts = -offsets
     int n_chunks_t;
     int max_len_n, max_len_t;    // longest chunk of each table
     int s_min_n, s_max_n;        // smallest / largest chunk shift of each table
     int s_min_t, s_max_t;
+    const Chunk *chunks_p_dev;   // the projection's table (chunks of up to CHUNK_MAX): shifts = offsets
+    int n_chunks_p;
+    int max_len_p;
     const Unit *units_dev;       // units of the normal table (dense x dense^T projection)
     int n_units;
     const Unit *single_units_dev;   // one unit per chunk of the normal table, in table order

@@ -6,8 +6,9 @@
 
 namespace cuvdia {
 
-std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed)
+std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, int max_len)
 {
+    max_len = std::min(std::max(max_len, 1), CHUNK_SLOTS);
     std::vector<std::pair<long long, int>> s(nd);      // (shift, table position)
     for (int d = 0; d < nd; ++d)
         s[d] = { transposed ? -(long long)offsets[d] : (long long)offsets[d], d };
@@ -21,14 +22,14 @@ std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed)
         int j = i + 1;
         while (j < nd && s[j].first == s[j - 1].first + 1) ++j;
         const int run = j - i;
-        const int pieces = (run + CHUNK_MAX - 1) / CHUNK_MAX;
+        const int pieces = (run + max_len - 1) / max_len;
         int done = 0;
         for (int p = 0; p < pieces; ++p) {
             const int len = (run - done + (pieces - p) - 1) / (pieces - p);
             Chunk c{};
             c.s0 = (int)s[i + done].first;
             c.len = len;
-            for (int q = 0; q < CHUNK_MAX; ++q) c.slot[q] = q < len ? s[i + done + q].second : -1;
+            for (int q = 0; q < CHUNK_SLOTS; ++q) c.slot[q] = q < len ? s[i + done + q].second : -1;
             out.push_back(c);
             done += len;
         }

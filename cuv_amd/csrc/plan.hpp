@@ -1,32 +1,36 @@
 // Host-side decomposition of a DIA offset table into run chunks.
 //
 // A tiled kernel does not walk the offset table diagonal by diagonal; it
-// walks *chunks*: up to CHUNK_MAX consecutive shifts (s0, s0+1, ...) whose
+// walks *chunks*: a few consecutive shifts (s0, s0+1, ...) whose
 // dense-operand rows overlap, so one staged window of the dense tile serves
-// all of them.  For the normal product the shift of diagonal d is its offset
+// all of them.  The products take chunks of up to SP_CHUNK_MAX shifts (what
+// the 76 dense rows they stage per chunk can serve for 64 output rows), the
+// dense x dense^T projection chunks of up to CHUNK_MAX (it keeps 4 running
+// sums per shift and lane).  For the normal product the shift of diagonal d is its offset
 // k_d (input row = output row + k_d); for the transposed product it is -k_d.
 #pragma once
 #include <vector>
 
 namespace cuvdia {
 
-constexpr int CHUNK_MAX = 8;
+constexpr int CHUNK_MAX = 8;        // longest chunk of the projection's table
+constexpr int SP_CHUNK_MAX = 13;    // longest chunk of the products' tables
+constexpr int CHUNK_SLOTS = 14;
 
-// 48 bytes; read by the kernels through scalar loads.
+// 64 bytes; read by the kernels through scalar loads.
 struct Chunk {
     int s0;                 // shift of the first position in the chunk
-    int len;                // number of positions, 1..CHUNK_MAX
-    int slot[CHUNK_MAX];    // table position (d) of each, so values sit at vals[slot*stride + ...];
+    int len;                // number of positions, 1..max_len of the table
+    int slot[CHUNK_SLOTS];  // table position (d) of each, so values sit at vals[slot*stride + ...];
                             // -1 marks a position no diagonal occupies
-    int pad[2];
 };
-static_assert(sizeof(Chunk) == 48, "Chunk layout is part of the device table");
+static_assert(sizeof(Chunk) == 64 && SP_CHUNK_MAX <= CHUNK_SLOTS, "Chunk layout is part of the device table");
 
 // Sort shifts (stable in table position), cut into maximal runs of
 // consecutive shifts -- a repeated shift starts a new run -- and split each
-// run into near-equal chunks of at most CHUNK_MAX.  Positions past a chunk's
-// length carry slot -1.
-std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed);
+// run into near-equal chunks of at most max_len (<= CHUNK_SLOTS).  Positions
+// past a chunk's length carry slot -1.
+std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, int max_len = CHUNK_MAX);
 
 // A unit of work of the tiled dense x dense^T projection: one chunk, or two
 // chunks of the normal table whose first shifts differ by a multiple of 4 of

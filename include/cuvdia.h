@@ -81,11 +81,18 @@ int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t,
 /* Pure host function (no GPU needed): decomposes an offset table into the
  * run chunks the tiled kernels walk.  Shifts are the offsets themselves
  * (transposed == 0) or their negation (transposed != 0), sorted ascending;
- * a run is a maximal sequence of consecutive shifts and is cut into chunks
- * of at most 8.  Chunk c covers shifts s0[c] .. s0[c]+len[c]-1 and
- * slot[8*c + j] is the table position of the j-th one (-1 for j >= len[c]).
- * Returns the number of chunks (also when it exceeds cap; then nothing is
- * written), or a negative error. */
+ * a run is a maximal sequence of consecutive shifts and is cut into
+ * near-equal chunks of at most max_len, 1 <= max_len <= 13.  The products
+ * walk the tables of max_len 13 (one staged block of 76 dense rows serves 64
+ * output rows and 13 shifts), the dense x dense^T projection the table of
+ * max_len 8, transposed == 0.  Chunk c covers shifts s0[c] .. s0[c]+len[c]-1
+ * and slot[max_len*c + j] is the table position of the j-th one (-1 for
+ * j >= len[c]).  Returns the number of chunks (also when it exceeds cap; then
+ * nothing is written), or a negative error. */
+int cuvdia_plan_chunks_max(const int *offsets_host, int nd, int transposed, int max_len,
+                           int *s0, int *len, int *slot, int cap);
+
+/* cuvdia_plan_chunks_max with max_len 8. */
 int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
                        int *s0, int *len, int *slot, int cap);
 

@@ -62,26 +62,31 @@ def test_no_device_is_an_error_not_a_fallback():
                                       _lib.ACT_SIGMOID_SAMPLE, None) == _lib.EINVAL
 
 
-def _plan(offsets, transposed=False):
+def _plan(offsets, transposed=False, max_len=8):
     from cuv_amd import _lib
     L = _lib.lib()
     offs = np.ascontiguousarray(offsets, np.int32)
     ip = ctypes.POINTER(ctypes.c_int)
-    n = L.cuvdia_plan_chunks(offs.ctypes.data_as(ip), offs.size, int(transposed), None, None, None, 0)
+    if max_len == 8:
+        def call(*out):
+            return L.cuvdia_plan_chunks(offs.ctypes.data_as(ip), offs.size, int(transposed), *out)
+    else:
+        def call(*out):
+            return L.cuvdia_plan_chunks_max(offs.ctypes.data_as(ip), offs.size, int(transposed), max_len, *out)
+    n = call(None, None, None, 0)
     assert n > 0
-    s0, ln, sl = np.zeros(n, np.int32), np.zeros(n, np.int32), np.zeros(8 * n, np.int32)
-    assert L.cuvdia_plan_chunks(offs.ctypes.data_as(ip), offs.size, int(transposed), s0.ctypes.data_as(ip),
-                                ln.ctypes.data_as(ip), sl.ctypes.data_as(ip), n) == n
-    return s0, ln, sl.reshape(n, 8)
+    s0, ln, sl = np.zeros(n, np.int32), np.zeros(n, np.int32), np.zeros(max_len * n, np.int32)
+    assert call(s0.ctypes.data_as(ip), ln.ctypes.data_as(ip), sl.ctypes.data_as(ip), n) == n
+    return s0, ln, sl.reshape(n, max_len)
 
 
-def _check_plan_covers(offsets, transposed):
-    s0, ln, sl = _plan(offsets, transposed)
+def _check_plan_covers(offsets, transposed, max_len=8):
+    s0, ln, sl = _plan(offsets, transposed, max_len)
     sign = -1 if transposed else 1
     seen = []
     for c in range(len(s0)):
-        assert 1 <= ln[c] <= 8
-        for j in range(8):
+        assert 1 <= ln[c] <= max_len
+        for j in range(max_len):
             if j < ln[c] and sl[c, j] >= 0:
                 assert sign * offsets[sl[c, j]] == s0[c] + j       # the slot really has that shift
                 seen.append(int(sl[c, j]))
@@ -110,6 +115,20 @@ def test_plan_long_runs_are_split_evenly():
     assert len(s0) == 104 and sorted(set(ln.tolist())) == [6, 7]
 
 
+def test_plan_of_the_products_takes_chunks_of_13():
+    """The products' tables: a 13-wide window row is one chunk, longer runs are cut evenly."""
+    offs = [c * 65536 + dy * 256 + dx for c in range(4) for dy in range(-6, 7) for dx in range(-6, 7)]
+    for transposed in (False, True):
+        s0, ln, sl = _check_plan_covers(offs, transposed, 13)
+        assert len(s0) == 52 and set(ln.tolist()) == {13}
+    s0, ln, _ = _check_plan_covers(list(range(-16, 17)), False, 13)      # one run of 33 -> 11 + 11 + 11
+    assert ln.tolist() == [11, 11, 11] and s0.tolist() == [-16, -5, 6]
+    s0, ln, _ = _check_plan_covers([dy * 128 + dx for dy in range(-3, 4) for dx in range(-3, 4)], False, 13)
+    assert ln.tolist() == [7] * 7                                         # runs of 7 stay as they are
+    _check_plan_covers([0, 0, 3, 2000, -2000, 3], True, 13)
+    _check_plan_covers(list(range(40)), False, 1)
+
+
 def test_plan_isolated_and_adjacent_runs():
     offs = [0, 1, -1, 10, 11, 12, 13, 14, 15, 16, 17, 18, 40]
     s0, ln, sl = _check_plan_covers(offs, False)
@@ -129,6 +148,9 @@ def test_plan_rejects_bad_arguments():
     from cuv_amd import _lib
     L = _lib.lib()
     assert L.cuvdia_plan_chunks(None, 3, 0, None, None, None, 0) == _lib.EINVAL
+    three = np.arange(3, dtype=np.int32).ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+    assert L.cuvdia_plan_chunks_max(three, 3, 0, 0, None, None, None, 0) == _lib.EINVAL
+    assert L.cuvdia_plan_chunks_max(three, 3, 0, 14, None, None, None, 0) == _lib.EINVAL
     offs = np.array([1], np.int32)
     assert L.cuvdia_plan_chunks(offs.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), 0, 0, None, None, None, 0) == _lib.EINVAL
 
