@@ -306,7 +306,7 @@ __global__ __launch_bounds__(AXPBY_THREADS) void momentum_kernel(
 //
 // Workgroup = 64 output rows x 64 batch columns, 8 waves of T = 8 rows each.
 // Lane l of every wave owns batch column col0 + l and T running sums.  Per
-// run chunk (<= 8 consecutive shifts starting at s0):
+// run chunk (<= 13 consecutive shifts starting at s0):
 //   1. the dense rows a0 .., a0 = row0 + s0, that the chunk touches are staged
 //      in LDS for the 64 columns, LDS row i of a column holding dense row
 //      a0 + i, together with the chunk's diagonals for the 64 rows (wave w
@@ -725,9 +725,9 @@ __device__ __forceinline__ void lds_load_b128(sp_int4 rsrc, unsigned lds_byte_ad
 // instructions, every lane busy, stage the chunk.  Columns are then 76 floats
 // apart, which keeps the 16-byte window reads (one lane per column) free of
 // bank conflicts.  Wave w issues instructions w, w + 8 and (waves 0-2)
-// w + 16; waves 3 and 4 fetch the chunk's 8 diagonals for the 64 rows, 4
-// diagonals per instruction: 21 loads per chunk, none through registers, no
-// LDS write instruction.  Three LDS buffers: chunk k lives in buffer k % 3.
+// w + 16; waves 3 and 4 (3 to 6 for tables with chunks longer than 8) fetch
+// the chunk's diagonals for the 64 rows, 4 diagonals per instruction: 21 (23)
+// loads per chunk, none through registers, no LDS write instruction.  Three LDS buffers: chunk k lives in buffer k % 3.
 // The FMAs of chunk c are cut in two; between the halves sit the wait for
 // chunk c+1, the barrier, the read of window(c+1) and the request for chunk
 // c+3, while chunk c+2 is landing.
@@ -812,7 +812,7 @@ __device__ __forceinline__ void spmm_tile_lean(
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
     constexpr unsigned BUF_BYTES = SP_DSTAGE_FLOATS * 4u;
 
-    // A chunk's table entry travels through three 16-byte SCALAR loads into
+    // A chunk's table entry travels through three (four: chunks longer than 8) 16-byte SCALAR loads into
     // scalar registers, one iteration before the chunk is requested: no vector
     // memory instruction, no LDS copy and no register table stand between the
     // kernel's start and its first requests, and the loop's entries arrive

@@ -73,8 +73,9 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
 int cuvdia_desc_destroy(cuvdia_desc *desc);
 
 /* Host-side facts about a descriptor (any pointer may be NULL):
- * number of run chunks for the normal and transposed traversal, and the
- * number of valid (non-padding) elements. */
+ * number of run chunks the products walk for the normal and the transposed
+ * traversal (cuvdia_plan_chunks_max with max_len 13), and the number of
+ * valid (non-padding) elements. */
 int cuvdia_desc_info(const cuvdia_desc *desc, int *chunks_n, int *chunks_t,
                      long long *nnz);
 
