@@ -1051,15 +1051,23 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
 constexpr int DD_ROWS = 256;
 constexpr int DD_BG = 4;           // batch columns per step
 
-template <int NCH>
+// LC > CHUNK_MAX: the unit is one long chunk of the products' table (up to
+// SP_CHUNK_MAX shifts: a whole row of a wide 2-d window), never a pair.  It
+// keeps as many running sums as a pair and is worked by 8 waves as well.
+template <int NCH, int LC>
 struct DdShape {
+    static_assert(NCH == 1 || LC <= CHUNK_MAX, "pairs are made of short chunks");
+    static constexpr bool LONG = LC > CHUNK_MAX;
+    static constexpr int SPAN = LONG ? SP_CHUNK_MAX : CHUNK_MAX;    // shifts a chunk can have
     static constexpr int NQ = NCH == 1 ? 4 : 6;                 // 64-row blocks of the band
-    static constexpr int PITCH = 64 * NQ + 8;                   // staged rows per column: 264 or 392
-    static constexpr int WAVES = NCH == 1 ? 4 : 8;
+    static constexpr int PITCH = 64 * NQ + (LONG ? 16 : 8);     // staged rows per column: 264, 272 or 392
+    static constexpr int WAVES = (NCH == 2 || LONG) ? 8 : 4;
     static constexpr int WAVE_FLOATS = 2 * DD_BG * PITCH + 4;   // two buffers + a slot idle lanes write to
     static constexpr int STAGE_FLOATS = WAVES * WAVE_FLOATS;
 };
-static_assert(DdShape<2>::PITCH >= DD_ROWS + PAIR_MAX_DELTA + CHUNK_MAX, "a pair's band must fit its buffer");
+static_assert(DdShape<2, CHUNK_MAX>::PITCH >= DD_ROWS + PAIR_MAX_DELTA + CHUNK_MAX, "a pair's band must fit its buffer");
+static_assert(DdShape<1, SP_CHUNK_MAX>::PITCH >= DD_ROWS + 4 * ((4 + SP_CHUNK_MAX - 1 + 3) / 4) - 4,
+              "a long chunk's last window must fit its buffer");
 
 // What a wave has in flight of A for one group of 4 batch columns (two of
 // these alternate; B's pieces need one set of registers only, see the loop).
@@ -1072,7 +1080,8 @@ constexpr int dd_red_floats() { return 4 * 4 * (NCH * LC * 64 + 8); }
 template <int LC, int NCH>
 constexpr int dd_lds_floats()
 {
-    return DdShape<NCH>::STAGE_FLOATS > dd_red_floats<LC, NCH>() ? DdShape<NCH>::STAGE_FLOATS : dd_red_floats<LC, NCH>();
+    return DdShape<NCH, LC>::STAGE_FLOATS > dd_red_floats<LC, NCH>() ? DdShape<NCH, LC>::STAGE_FLOATS
+                                                                     : dd_red_floats<LC, NCH>();
 }
 
 template <int LC, int NCH, bool AVEC>
@@ -1082,7 +1091,7 @@ __device__ __forceinline__ void dd2dia_unit(
     int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
     unsigned c_bytes)
 {
-    typedef DdShape<NCH> S;
+    typedef DdShape<NCH, LC> S;
     constexpr int PITCH = S::PITCH, WAVES = S::WAVES;
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
@@ -1092,10 +1101,10 @@ __device__ __forceinline__ void dd2dia_unit(
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // each table entry in three 16-byte scalar loads
+    // each table entry in three (a long chunk: four) 16-byte scalar loads
     typedef int int4v __attribute__((ext_vector_type(4)));
     typedef const int4v __attribute__((address_space(4))) *sc_int4_ptr;
-    int s0[NCH], slots[NCH][CHUNK_MAX];
+    int s0[NCH], slots[NCH][S::SPAN];
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
         const sc_int4_ptr e = (sc_int4_ptr)(n == 0 ? ck1 : ck2);
@@ -1103,9 +1112,13 @@ __device__ __forceinline__ void dd2dia_unit(
         s0[n] = e0.x;
         slots[n][0] = e0.z; slots[n][1] = e0.w; slots[n][2] = e1.x; slots[n][3] = e1.y;
         slots[n][4] = e1.z; slots[n][5] = e1.w; slots[n][6] = e2.x; slots[n][7] = e2.y;
+        if constexpr (S::LONG) {
+            const int4v e3 = e[3];
+            slots[n][8] = e2.z; slots[n][9] = e2.w; slots[n][10] = e3.x; slots[n][11] = e3.y; slots[n][12] = e3.z;
+        }
     }
     const int delta = NCH == 2 ? s0[NCH - 1] - s0[0] : 0;      // rows between the two windows
-    const int need = DD_ROWS + delta + CHUNK_MAX;               // staged rows that are ever read
+    const int need = DD_ROWS + delta + S::SPAN;                 // staged rows that are ever read
     const int base = row0 + s0[0];                              // first staged row of B
     // Every slot of the unit pairs row i with row i + s0 + j of B: with the
     // whole band outside B the unit stores no matrix element, and there is
@@ -1375,20 +1388,21 @@ __device__ __forceinline__ void dd2dia_unit(
     }
 }
 
-// PAIRS = false: every unit is a single chunk, 4 waves per workgroup.
+// PAIRS = false: every unit is a single chunk, 4 waves per workgroup (8 for
+// the long chunks of LC > CHUNK_MAX).
 // PAIRS = true: 8 waves per workgroup; a workgroup whose unit is a single
 // chunk retires its upper four waves at once.
 template <int LC, bool AVEC, bool PAIRS>
-__global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
+__global__ __launch_bounds__((PAIRS || LC > CHUNK_MAX) ? 512 : 256) void dd2dia_tiled_kernel(
     const Chunk *__restrict__ chunks, const Unit *__restrict__ units, int nunits,
     float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
     int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
     unsigned c_bytes)
 {
-    constexpr int LDS_FLOATS = PAIRS ? (dd_lds_floats<LC, 2>() > dd_lds_floats<LC, 1>() ? dd_lds_floats<LC, 2>()
-                                                                                         : dd_lds_floats<LC, 1>())
-                                     : dd_lds_floats<LC, 1>();
+    constexpr int NCH_MAX = PAIRS ? 2 : 1;
+    constexpr int LDS_FLOATS = dd_lds_floats<LC, NCH_MAX>() > dd_lds_floats<LC, 1>() ? dd_lds_floats<LC, NCH_MAX>()
+                                                                                     : dd_lds_floats<LC, 1>();
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
     const int rowtile = tile / nunits;
@@ -1396,14 +1410,16 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     const sc_unit_ptr u = (sc_unit_ptr)units + (tile - rowtile * nunits);
     const int c1 = u->c1, c2 = u->c2;
     const int row0 = rowtile * DD_ROWS;
-    if (PAIRS && c2 >= 0) {
-        dd2dia_unit<LC, 2, AVEC>(lds, row0, chunks + c1, chunks + c2, C, stride, A, lda, B, ldb, h, w, batch,
-                                 alpha, beta, a_bytes, b_bytes, c_bytes);
-    } else {
-        if (PAIRS && threadIdx.x >= 256) return;
-        dd2dia_unit<LC, 1, AVEC>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
-                                 alpha, beta, a_bytes, b_bytes, c_bytes);
+    if constexpr (PAIRS) {
+        if (c2 >= 0) {
+            dd2dia_unit<LC, 2, AVEC>(lds, row0, chunks + c1, chunks + c2, C, stride, A, lda, B, ldb, h, w, batch,
+                                     alpha, beta, a_bytes, b_bytes, c_bytes);
+            return;
+        }
     }
+    if (PAIRS && threadIdx.x >= 256) return;
+    dd2dia_unit<LC, 1, AVEC>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
+                             alpha, beta, a_bytes, b_bytes, c_bytes);
 }
 
 }  // namespace
@@ -1577,13 +1593,20 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     // (pairs only with 16-byte loads of A: the dword-load variant of the pair
     // body needs more registers than a wave has)
     const bool use_units = C.n_units < C.n_chunks_p && a_vec && !g_dd2dia_no_pairs;
-    const bool pairs = use_units;
-    const Unit *units = use_units ? C.units_dev : C.single_units_dev;
-    const int nunits = use_units ? C.n_units : C.n_chunks_p;
+    // A table with runs longer than CHUNK_MAX is walked in the long chunks of
+    // the products' table instead (a 13-wide window row as one unit rather
+    // than two that cannot pair): the same registers as a pair, half the
+    // loads and LDS traffic per FMA.  (16-byte loads of A only, as for pairs.)
+    const bool long_chunks = C.max_len_n > CHUNK_MAX && a_vec && !g_dd2dia_no_pairs;
+    const bool pairs = use_units && !long_chunks;
+    const Unit *units = pairs ? C.units_dev : C.single_units_dev;      // the single units count 0, 1, 2, ...
+    const int nunits = long_chunks ? C.n_chunks_n : pairs ? C.n_units : C.n_chunks_p;
+    const Chunk *table = long_chunks ? C.chunks_n_dev : C.chunks_p_dev;
+    const int lc = long_chunks ? C.max_len_n : C.max_len_p;
     const long long blocks = row_tiles * nunits;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks);
-#define CUVDIA_DD_ARGS C.chunks_p_dev, units, nunits, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
+#define CUVDIA_DD_ARGS table, units, nunits, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
                        a_bytes, b_bytes, c_bytes
 #define CUVDIA_DD_LAUNCH(L)                                                                              \
     case L:                                                                                              \
@@ -1594,11 +1617,18 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
             else hipLaunchKernelGGL((dd2dia_tiled_kernel<L, false, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);       \
         }                                                                                                \
         break;
-    switch (C.max_len_p) {
+#define CUVDIA_DD_LAUNCH_LONG(L)                                                                         \
+    case L:                                                                                              \
+        hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, false>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);      \
+        break;
+    switch (lc) {
         CUVDIA_DD_LAUNCH(1) CUVDIA_DD_LAUNCH(2) CUVDIA_DD_LAUNCH(3) CUVDIA_DD_LAUNCH(4)
         CUVDIA_DD_LAUNCH(5) CUVDIA_DD_LAUNCH(6) CUVDIA_DD_LAUNCH(7) CUVDIA_DD_LAUNCH(8)
+        CUVDIA_DD_LAUNCH_LONG(9) CUVDIA_DD_LAUNCH_LONG(10) CUVDIA_DD_LAUNCH_LONG(11) CUVDIA_DD_LAUNCH_LONG(12)
+        CUVDIA_DD_LAUNCH_LONG(13)
         default: return hipErrorInvalidValue;
     }
+#undef CUVDIA_DD_LAUNCH_LONG
 #undef CUVDIA_DD_LAUNCH
 #undef CUVDIA_DD_ARGS
     return hipGetLastError();
