@@ -1027,8 +1027,11 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
 // shifts differ by delta (a multiple of 4, at most 128) -- e.g. two rows of a
 // 2-d window.  Lane l owns rows row0 + 4l .. 4l+3 and 4 x LC partial sums per
 // chunk (LC = the longest chunk of the table; positions past a chunk's own
-// length are computed and dropped).  A single chunk is worked by 4 waves, a
-// pair by 8; wave q walks the batch-column groups g = q, q + WAVES, ...
+// length are computed and dropped).  A table with runs of more than 8 shifts
+// (window rows wider than 8) is walked in the products' chunks of up to 13
+// instead, every unit one such chunk: as many sums as a pair, one band, one
+// copy of A's rows.  A single short chunk is worked by 4 waves, a pair or a
+// long chunk by 8; wave q walks the batch-column groups g = q, q + WAVES, ...
 // (4 columns per group).  Per group and column the wave
 //   1. writes the column's rows [row0 + s0, row0 + s0 + 264 + delta) of B,
 //      fetched one step earlier as 16-byte pieces (a lane holds 4 consecutive
