@@ -114,6 +114,10 @@ SHAPES = [
     (2048, 2048, [dy * 64 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 1, 70),
     (1536, 2304, [dy * 128 + dx for dy in range(-2, 3) for dx in range(-2, 3)], 1, 130),
     (2304, 1600, [dy * 128 + dx for dy in (-3, -2, -1, 1, 2) for dx in range(-1, 2)], 1, 64),
+    # window rows wider than 8: one long chunk each (13), and runs of 9 and 12 in one table
+    (512, 640, [dy * 96 + dx for dy in range(-1, 2) for dx in range(-6, 7)], 1, 72),
+    (768, 512, list(range(-4, 5)) + [100 + k for k in range(12)], 1, 33),
+    (1280, 1280, [dy * 128 + dx for dy in range(-4, 5) for dx in range(-4, 5)], 1, 128),
 ]
 
 
