@@ -1030,8 +1030,8 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
 // length are computed and dropped).  A table with runs of more than 8 shifts
 // (window rows wider than 8) is walked in the products' chunks of up to 13
 // instead, every unit one such chunk: as many sums as a pair, one band, one
-// copy of A's rows.  A single short chunk is worked by 4 waves, a pair or a
-// long chunk by 8; wave q walks the batch-column groups g = q, q + WAVES, ...
+// copy of A's rows.  A single chunk is worked by 4 waves, a pair by 8; wave
+// q walks the batch-column groups g = q, q + WAVES, ...
 // (4 columns per group).  Per group and column the wave
 //   1. writes the column's rows [row0 + s0, row0 + s0 + 264 + delta) of B,
 //      fetched one step earlier as 16-byte pieces (a lane holds 4 consecutive
@@ -1056,7 +1056,9 @@ constexpr int DD_BG = 4;           // batch columns per step
 
 // LC > CHUNK_MAX: the unit is one long chunk of the products' table (up to
 // SP_CHUNK_MAX shifts: a whole row of a wide 2-d window), never a pair.  It
-// keeps as many running sums as a pair and is worked by 8 waves as well.
+// keeps as many running sums as a pair but is worked by 4 waves: three such
+// workgroups share a CU (registers allow 3 waves per SIMD, and the block the
+// sums are added in is kept just under a third of the CU's LDS).
 template <int NCH, int LC>
 struct DdShape {
     static_assert(NCH == 1 || LC <= CHUNK_MAX, "pairs are made of short chunks");
@@ -1064,7 +1066,8 @@ struct DdShape {
     static constexpr int SPAN = LONG ? SP_CHUNK_MAX : CHUNK_MAX;    // shifts a chunk can have
     static constexpr int NQ = NCH == 1 ? 4 : 6;                 // 64-row blocks of the band
     static constexpr int PITCH = 64 * NQ + (LONG ? 16 : 8);     // staged rows per column: 264, 272 or 392
-    static constexpr int WAVES = (NCH == 2 || LONG) ? 8 : 4;
+    static constexpr int WAVES = NCH == 2 ? 8 : 4;
+    static constexpr int RED_PAD = LONG ? 4 : 8;              // a long chunk's sums then fit a third of a CU's LDS
     static constexpr int WAVE_FLOATS = 2 * DD_BG * PITCH + 4;   // two buffers + a slot idle lanes write to
     static constexpr int STAGE_FLOATS = WAVES * WAVE_FLOATS;
 };
@@ -1079,7 +1082,7 @@ struct DdStage {
 };
 
 template <int LC, int NCH>
-constexpr int dd_red_floats() { return 4 * 4 * (NCH * LC * 64 + 8); }
+constexpr int dd_red_floats() { return 4 * 4 * (NCH * LC * 64 + DdShape<NCH, LC>::RED_PAD); }
 template <int LC, int NCH>
 constexpr int dd_lds_floats()
 {
@@ -1098,7 +1101,7 @@ __device__ __forceinline__ void dd2dia_unit(
     constexpr int PITCH = S::PITCH, WAVES = S::WAVES;
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
-    constexpr int RED_T = NCH * LC * 64 + 8;        // floats between the 4 rows a lane owns: keeps the
+    constexpr int RED_T = NCH * LC * 64 + S::RED_PAD;        // floats between the 4 rows a lane owns: keeps the
                                                     // row-major read below free of bank conflicts
     constexpr int RED_WAVE = 4 * RED_T;
 
@@ -1391,12 +1394,11 @@ __device__ __forceinline__ void dd2dia_unit(
     }
 }
 
-// PAIRS = false: every unit is a single chunk, 4 waves per workgroup (8 for
-// the long chunks of LC > CHUNK_MAX).
+// PAIRS = false: every unit is a single chunk, 4 waves per workgroup.
 // PAIRS = true: 8 waves per workgroup; a workgroup whose unit is a single
 // chunk retires its upper four waves at once.
 template <int LC, bool AVEC, bool PAIRS>
-__global__ __launch_bounds__((PAIRS || LC > CHUNK_MAX) ? 512 : 256) void dd2dia_tiled_kernel(
+__global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     const Chunk *__restrict__ chunks, const Unit *__restrict__ units, int nunits,
     float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
@@ -1622,7 +1624,7 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
         break;
 #define CUVDIA_DD_LAUNCH_LONG(L)                                                                         \
     case L:                                                                                              \
-        hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, false>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);      \
+        hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);      \
         break;
     switch (lc) {
         CUVDIA_DD_LAUNCH(1) CUVDIA_DD_LAUNCH(2) CUVDIA_DD_LAUNCH(3) CUVDIA_DD_LAUNCH(4)
