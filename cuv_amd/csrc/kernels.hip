@@ -1578,10 +1578,6 @@ bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch)
            b_bytes < (long long)OOB_OFFSET && c_bytes < (long long)OOB_OFFSET;
 }
 
-// 0: pair chunks where the plan allows it; 1: every chunk on its own (tests
-// and measurements of the unpaired kernel)
-int g_dd2dia_no_pairs = 0;
-
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream)
@@ -1597,12 +1593,12 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     // without pairs the units are the chunks themselves, in table order
     // (pairs only with 16-byte loads of A: the dword-load variant of the pair
     // body needs more registers than a wave has)
-    const bool use_units = C.n_units < C.n_chunks_p && a_vec && !g_dd2dia_no_pairs;
+    const bool use_units = C.n_units < C.n_chunks_p && a_vec;
     // A table with runs longer than CHUNK_MAX is walked in the long chunks of
     // the products' table instead (a 13-wide window row as one unit rather
     // than two that cannot pair): the same registers as a pair, half the
     // loads and LDS traffic per FMA.  (16-byte loads of A only, as for pairs.)
-    const bool long_chunks = C.max_len_n > CHUNK_MAX && a_vec && !g_dd2dia_no_pairs;
+    const bool long_chunks = C.max_len_n > CHUNK_MAX && a_vec;
     const bool pairs = use_units && !long_chunks;
     const Unit *units = pairs ? C.units_dev : C.single_units_dev;      // the single units count 0, 1, 2, ...
     const int nunits = long_chunks ? C.n_chunks_n : pairs ? C.n_units : C.n_chunks_p;
