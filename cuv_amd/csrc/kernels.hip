@@ -37,6 +37,10 @@ namespace {
 // in groups of 8 spans of XCD_SPAN, one span per XCD and group, so that work
 // which varies along the rows (chunks falling outside the operand) still
 // spreads evenly; the last, partial group is split into 8 near-equal spans.
+// The very last span is dealt backwards: the tiles at the high end of the
+// rows take the slower body for tiles at the operand's ends, exactly like the
+// first tiles of the first span, and dealt in order they would be the last to
+// start as well -- a launch of one or two rounds then ends when they do.
 constexpr int XCD_SPAN = 64;
 __device__ __forceinline__ int xcd_tile(int bid, int nblk)
 {
@@ -44,12 +48,16 @@ __device__ __forceinline__ int xcd_tile(int bid, int nblk)
     const int full = nblk / GROUP * GROUP;           // tiles in whole groups
     if (bid < full) {
         const int g = bid / GROUP, in = bid - g * GROUP;
-        const int xcd = in % XCDS, slot = in / XCDS;
+        const int xcd = in % XCDS;
+        int slot = in / XCDS;
+        if (xcd == XCDS - 1 && (g + 1) * GROUP == nblk) slot = XCD_SPAN - 1 - slot;
         return g * GROUP + xcd * XCD_SPAN + slot;
     }
     const int rest = nblk - full, b = bid - full;
     const int q = rest / XCDS, r = rest % XCDS;
-    const int xcd = b % XCDS, slot = b / XCDS;
+    const int xcd = b % XCDS;
+    int slot = b / XCDS;
+    if (xcd == XCDS - 1) slot = q - 1 - slot;        // the last span has q tiles (r < XCDS)
     return full + xcd * q + (xcd < r ? xcd : r) + slot;
 }
 
