@@ -724,6 +724,17 @@ __device__ __forceinline__ void lds_load_b128(sp_int4 rsrc, unsigned lds_byte_ad
                  "buffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_byte_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
+// the same with 4 bytes per lane: lane i writes at lds_byte_addr + 4*i
+__device__ __forceinline__ void lds_load_b32(sp_int4 rsrc, unsigned lds_byte_addr, unsigned voff)
+{
+    lds_byte_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
+    rsrc = sp_int4{__builtin_amdgcn_readfirstlane(rsrc.x), __builtin_amdgcn_readfirstlane(rsrc.y),
+                   __builtin_amdgcn_readfirstlane(rsrc.z), __builtin_amdgcn_readfirstlane(rsrc.w)};
+    asm volatile("s_mov_b32 m0, %0\n\t"
+                 "s_nop 0\n\t"
+                 "buffer_load_dword %1, %2, 0 offen lds"
+                 :: "s"(lds_byte_addr), "v"(voff), "s"(rsrc) : "memory");
+}
 
 // The lean body (see spmm_tile) with the staging done by loads that write LDS
 // directly.  A chunk stages 76 rows (19 16-byte pieces) of each of the 64
@@ -796,6 +807,7 @@ __device__ __forceinline__ void spmm_tile_lean(
     // this lane's pieces in the three load instructions the wave issues
     unsigned x_off[3];
     unsigned x_lds[3];                      // byte offset inside a stage buffer that the instruction fills
+    int x_quad[3];                          // the piece's place in its column (only chunks at the operand's ends ask)
 #pragma unroll
     for (int it = 0; it < 3; ++it) {
         const int i = wave + WAVES * it;
@@ -803,6 +815,7 @@ __device__ __forceinline__ void spmm_tile_lean(
         const int col = piece / SP_DQUADS, quad = piece - col * SP_DQUADS;
         x_off[it] = (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) + 16u * quad;
         x_lds[it] = 1024u * i;
+        x_quad[it] = quad;
     }
     // SP_COLS * SP_DQUADS / 64 = 19 instructions stage the dense rows of a chunk:
     // waves 0-2 issue three of them, the others two.  Waves 3 and 4 fetch the
@@ -846,12 +859,50 @@ __device__ __forceinline__ void spmm_tile_lean(
         const int a0 = row0 + s0;
         // past the table, and for a chunk whose rows lie outside the operand,
         // nothing is fetched: an empty resource delivers zeros
-        const bool real = (c < nchunks) & (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
+        const bool inside = (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
+        const bool outside = (a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in);
+        const bool real = (c < nchunks) & !outside;
         const sp_int4 xq = raw_rsrc(xbase, real ? x_bytes : 0u);
-        const unsigned soff = real ? (unsigned)a0 * 4u : 0u;
-        lds_load_b128(xq, buf + x_lds[0], x_off[0], soff);
-        lds_load_b128(xq, buf + x_lds[1], x_off[1], soff);
-        if (x3) lds_load_b128(xq, buf + x_lds[2], x_off[2], soff);
+        if (inside | !real) {
+            const unsigned soff = real ? (unsigned)a0 * 4u : 0u;
+            lds_load_b128(xq, buf + x_lds[0], x_off[0], soff);
+            lds_load_b128(xq, buf + x_lds[1], x_off[1], soff);
+            if (x3) lds_load_b128(xq, buf + x_lds[2], x_off[2], soff);
+        } else {
+            // The chunk's rows cross an end of the operand.  The staged block then starts at the multiple of
+            // 4 at or below a0 (so that, the operand's row count being a multiple of 4 too, every 16-byte
+            // piece lies wholly inside or wholly outside), each lane checks its own piece, and the pieces
+            // outside arrive as zeros.  The same number of loads as for any other chunk: the waits still count.
+            // Its diagonal values take a way of their own: where a diagonal leaves the matrix its storage holds
+            // padding, and a 16-byte piece that crosses the first or last byte of the value array is answered
+            // with zeros as a whole.  So every wave fetches the values of its own 8 rows one by one (lane =
+            // 8 * diagonal + row, one more load for every wave; 0 where the product's input row does not
+            // exist) into the upper half of the buffer's block of diagonal values, which chunks of at most 8
+            // leave free.  A wait that counts one load too few only waits a little longer.
+            {
+                const int j = lane >> 3;
+                int p[8] = {en.p0, en.p1, en.p2, en.p3, en.p4, en.p5, en.p6, en.p7};
+#pragma unroll
+                for (int k = 0; k < 8; ++k) asm("" : "+s"(p[k]));
+                int sl = p[0];
+#pragma unroll
+                for (int k = 1; k < 8; ++k) sl = j == k ? p[k] : sl;
+                const int orow = row0 + wave * T + (lane & (T - 1));
+                const int in = orow + s0 + j;
+                const bool ok = (j < en.len) & (sl >= 0) & ((unsigned)in < (unsigned)n_in);
+                const unsigned off = ((unsigned)sl * (unsigned)stride + (unsigned)(ashift ? in : orow)) * 4u;
+                lds_load_b32(raw_rsrc(vals, a_bytes), buf + (unsigned)(SP_DAVALS + 8 * SP_ROWS + 64 * wave) * 4u,
+                             ok ? off : OOB_OFFSET);
+            }
+            const int a0p = a0 & ~3;
+#pragma unroll
+            for (int it = 0; it < 3; ++it) {
+                const int r = a0p + 4 * x_quad[it];
+                const bool ok = (r >= 0) & (r + 4 <= n_in);
+                const unsigned voff = ok ? x_off[it] + (unsigned)(a0p * 4) : OOB_OFFSET;
+                if (it < 2 || x3) lds_load_b128(xq, buf + x_lds[it], voff, 0u);
+            }
+        }
         if (a_wave) {
             // table position of this lane's diagonal, a_j: picked from the 8 scalars (each passed through an
             // empty asm so that the chain of selects stays one, and the entry stays in registers)
@@ -868,17 +919,38 @@ __device__ __forceinline__ void spmm_tile_lean(
             lds_load_b128(raw_rsrc(vals, a_bytes), buf + (unsigned)(SP_DAVALS + 4 * (wave - 3) * SP_ROWS) * 4u, voff, 0u);
         }
     };
-    auto read_window = [&](SpWindow<LCK, T> &win, int b) __attribute__((always_inline)) {
+    // Reads the window of the chunk whose shift is s0.  A chunk that crosses an end of the operand was staged
+    // from the multiple of 4 below its first row: its window starts up to 3 rows into the column (4-byte
+    // reads then), and its diagonal values sit in the wave's own corner of the buffer (see issue).
+    auto read_window = [&](SpWindow<LCK, T> &win, int b, int s0) __attribute__((always_inline)) {
         const float *buf = lds[b];
-        spmm_read_window<LCK, T>(win, buf + lane * SP_DPITCH + wave * T, buf + SP_DAVALS + wave * T + (lane & (T - 1)));
+        const int a0 = row0 + s0;
+        const bool inside = (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
+        const bool outside = (a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in);
+        if (inside | outside) {
+            spmm_read_window<LCK, T>(win, buf + lane * SP_DPITCH + wave * T, buf + SP_DAVALS + wave * T + (lane & (T - 1)));
+        } else {
+            const float *src = buf + lane * SP_DPITCH + wave * T + (a0 & 3);
+#pragma unroll
+            for (int i = 0; i < T + LCK - 1; ++i) win.w[i] = src[i];
+            const float *own = buf + SP_DAVALS + 8 * SP_ROWS + 64 * wave + (lane & (T - 1));
+#pragma unroll
+            for (int j = 0; j < LCK; ++j) win.a[j] = own[8 * j];
+            // keeps this rare path apart from the one above: merged into one, both would read 4 bytes at a time
+            asm volatile("");
+        }
     };
 
     SpWindow<LCK, T> w0, w1;
+    int s_cur, s_n1, s_n2;                  // shifts of the chunk whose window is read next, and of the two after it
     {
         const Entry h0 = fetch(0), h1 = fetch(1), h2 = fetch(2);
         issue(0, lds0, h0);
         issue(1, lds0 + BUF_BYTES, h1);
         issue(2, lds0 + 2 * BUF_BYTES, h2);
+        s_cur = h0.s0;
+        s_n1 = h1.s0;
+        s_n2 = h2.s0;
     }
     Entry e0 = fetch(3), e1 = e0;
     // The first window can be read as soon as chunk 0 (and the destination values) is in: the loads of
@@ -886,7 +958,7 @@ __device__ __forceinline__ void spmm_tile_lean(
     if (three) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     __syncthreads();
-    read_window(w0, 0);
+    read_window(w0, 0, s_cur);
     // Iteration c: buffers b (chunk c), b1 (chunk c+1); `use` is the entry of chunk c+3, `next` receives
     // the entry of chunk c+4.  The FMAs of chunk c are cut in two: the wait for chunk c+1, the barrier
     // and the read of its window sit between the halves, so the second half hides the read and a chunk
@@ -900,8 +972,10 @@ __device__ __forceinline__ void spmm_tile_lean(
         else if (three) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
         __syncthreads();                                 // also: every wave holds window(c), buffer b may be reused
-        if (c + 1 < nchunks) read_window(nxt, b1);
+        if (c + 1 < nchunks) read_window(nxt, b1, s_n1);
         if (c + 3 < nchunks) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use);
+        s_n1 = s_n2;
+        s_n2 = use.s0;
         next = fetch(c + 4);
         spmm_rows_range<LCK, T, JH, LCK>(acc, cur);
     };
@@ -995,9 +1069,15 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     // [row0 + s0, row0 + s0 + 80) lie either inside it or wholly outside (such
     // a chunk contributes nothing and is skipped through an empty resource).
     bool lean = row0 + SP_ROWS <= n_out;
-    int c_lo = 0, c_hi = nchunks;                   // the chunks whose rows lie inside the operand: a contiguous
+    int c_lo = 0, c_hi = nchunks;                   // the chunks with rows inside the operand: a contiguous
                                                     // range, the table being sorted by shift
     constexpr int STAGED = 4 * SP_DQUADS;           // rows the lean body stages per chunk
+    // A chunk whose staged rows cross an end of the operand is staged from the multiple of 4 below its first
+    // row, which costs up to 3 of the STAGED rows, and only works when no 16-byte piece crosses the end.
+    // The lean body takes such chunks when they have at most 8 diagonals (their values are fetched into
+    // the half of the buffer's diagonal block that longer chunks would need).
+    const bool crossing_ok = (LCK <= 8) & ((n_in & 3) == 0);
+    int crossing = 0;
     if (!((row0 + s_min >= 0) & (row0 + s_max + STAGED <= n_in))) {
         const int lane = threadIdx.x & 63;
         c_lo = nchunks;
@@ -1008,8 +1088,8 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
             const int a0 = row0 + chunks[min(idx, nchunks - 1)].s0;
             const bool inside = (a0 >= 0) & (a0 + STAGED <= n_in);
             const bool outside = (a0 + STAGED <= 0) | (a0 >= n_in);
-            lean &= __builtin_amdgcn_ballot_w64(!(inside | outside)) == 0;
-            const unsigned long long m = __builtin_amdgcn_ballot_w64(inside & (idx < nchunks));
+            crossing += (int)__builtin_popcountll(__builtin_amdgcn_ballot_w64(!(inside | outside) & (idx < nchunks)));
+            const unsigned long long m = __builtin_amdgcn_ballot_w64(!outside & (idx < nchunks));
             if (m) {
                 c_lo = min(c_lo, 64 * k + (int)__builtin_ctzll(m));
                 c_hi = max(c_hi, 64 * k + 64 - (int)__builtin_clzll(m));
@@ -1019,6 +1099,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
             c_lo = 0;
             c_hi = 1;
         }
+        lean &= crossing == 0 || crossing_ok;
     }
     if (lean)
         // only the chunks inside the operand are walked; the others would add zeros
