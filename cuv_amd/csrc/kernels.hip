@@ -863,8 +863,8 @@ __device__ __forceinline__ void spmm_tile_lean(
         const bool outside = (a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in);
         const bool real = (c < nchunks) & !outside;
         const sp_int4 xq = raw_rsrc(xbase, real ? x_bytes : 0u);
-        if (inside | !real) {
-            const unsigned soff = real ? (unsigned)a0 * 4u : 0u;
+        if (LCK > 8 || (inside | !real)) {       // (longer chunks never come here crossing an end: see the kernel)
+            const unsigned soff = (real & inside) ? (unsigned)a0 * 4u : 0u;
             lds_load_b128(xq, buf + x_lds[0], x_off[0], soff);
             lds_load_b128(xq, buf + x_lds[1], x_off[1], soff);
             if (x3) lds_load_b128(xq, buf + x_lds[2], x_off[2], soff);
@@ -927,7 +927,7 @@ __device__ __forceinline__ void spmm_tile_lean(
         const int a0 = row0 + s0;
         const bool inside = (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
         const bool outside = (a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in);
-        if (inside | outside) {
+        if (LCK > 8 || (inside | outside)) {
             spmm_read_window<LCK, T>(win, buf + lane * SP_DPITCH + wave * T, buf + SP_DAVALS + wave * T + (lane & (T - 1)));
         } else {
             const float *src = buf + lane * SP_DPITCH + wave * T + (a0 & 3);
