@@ -29,19 +29,145 @@ def _check_dense(t, rows, name):
     return t.shape[0], max(t.stride(0), rows) if t.shape[0] > 1 else max(rows, 1)
 
 
-class dev_dia_matrix_f:
-    """DIA matrix in device memory: element (i, j) at vec[d*stride + i] with
-    offsets[d] == j - i//row_fact (src/cuv/basics/dia_matrix.hpp:57-276)."""
+class _dia_matrix_f:
+    """What the host and the device DIA matrix share: shape, offset table with
+    its reverse map, element access and files.  Element (i, j) lives at
+    vec[d*stride + i] with offsets[d] == j - i//row_fact
+    (src/cuv/basics/dia_matrix.hpp:57-276)."""
 
-    def __init__(self, h, w, num_dia, stride, row_fact=1, device="cuda:0"):
+    def _init_shape(self, h, w, num_dia, stride, row_fact):
         if row_fact <= 0:
             raise RuntimeError("m_row_fact>0")
         if not (stride >= h or stride >= w):
             raise RuntimeError("m_stride >= this->h() || m_stride >= this->w()")
-        self.h, self.w, self.num_dia, self.stride, self.row_fact = h, w, num_dia, stride, row_fact
-        self.vec = torch.zeros(num_dia * stride, dtype=torch.float32, device=device)
-        self._offsets = np.zeros(num_dia, np.int32)
+        self.h, self.w, self.num_dia, self.stride, self.row_fact = int(h), int(w), int(num_dia), int(stride), int(row_fact)
+        self._offsets = np.zeros(self.num_dia, np.int32)
+        self._dia2off = {}
+
+    @property
+    def shape(self):
+        return (self.h, self.w)
+
+    def __len__(self):
+        """Number of matrix entries, h*w (matrix.hpp:103)."""
+        return self.h * self.w
+
+    def set_offsets(self, offsets):
+        offsets = np.ascontiguousarray(offsets, dtype=np.int32)
+        if offsets.size != self.num_dia:
+            raise RuntimeError("expected %d offsets" % self.num_dia)
+        self._offsets = offsets.copy()
+        self.post_update_offsets()
+
+    def post_update_offsets(self):
+        """Rebuilds the offset -> table position map; of two equal offsets the
+        later position wins (dia_matrix.hpp:181-185)."""
+        self._dia2off = {int(o): i for i, o in enumerate(self._offsets)}
+        self._offsets_changed()
+
+    def _offsets_changed(self):
+        pass
+
+    def set_offset(self, idx, val):
+        self._offsets[idx] = val
+        self._dia2off[int(val)] = int(idx)
+        self._offsets_changed()
+
+    def get_offsets(self):
+        return self._offsets.copy()
+
+    def get_offset(self, idx):
+        return int(self._offsets[idx])
+
+    def _slot(self, i, j):
+        """Position of element (i, j) in the value vector, or None off the band."""
+        d = self._dia2off.get(int(j) - int(i) // self.row_fact)
+        return None if d is None else d * self.stride + int(i)
+
+    def has(self, i, j):
+        """Whether the matrix stores element (i, j) (dia_matrix.hpp:244-251)."""
+        return self._slot(i, j) is not None
+
+    def __call__(self, i, j):
+        """Element (i, j); 0 off the band (dia_matrix.hpp:236-243)."""
+        s = self._slot(i, j)
+        return 0.0 if s is None else float(self.vec[s])
+
+    def set(self, i, j, val):
+        """Writes element (i, j); silently ignored off the band (dia_matrix.hpp:228-235)."""
+        s = self._slot(i, j)
+        if s is not None:
+            self.vec[s] = val
+
+    def dia(self, k):
+        """View of the whole stored diagonal with offset k: `stride` entries,
+        padding included (dia_matrix.hpp:205-221)."""
+        d = self._dia2off[int(k)]
+        return self.vec[d * self.stride:(d + 1) * self.stride]
+
+    def save(self, path):
+        """Writes the matrix to a file; a device matrix goes through the host
+        (src/cuv_python/export_dia_mat.cpp:90-104)."""
+        from . import io
+        io.save_fields(path, io.dia_to_fields(self))
+
+    def load(self, path):
+        """Replaces shape, offsets and values by the file's."""
+        from . import io
+        w, h, nd, stride, rf, offs, vec = io.check_fields(io.load_fields(path))
+        self._init_shape(h, w, nd, stride, rf)
+        self.alloc()
+        self.set_offsets(offs)
+        self.push(vec)
+        return self
+
+
+class host_dia_matrix_f(_dia_matrix_f):
+    """DIA matrix in host memory (a NumPy value vector): the container of the
+    reference's host_dia_matrix_f (src/cuv_python/export_dia_mat.cpp:113-150).
+    It holds data for conversion, files and element access; products run on the
+    device only."""
+
+    def __init__(self, h, w, num_dia, stride, row_fact=1):
+        self._init_shape(h, w, num_dia, stride, row_fact)
+        self.vec = None
+        self.alloc()
+
+    def alloc(self):
+        self.vec = np.zeros(self.num_dia * self.stride, np.float32)
+
+    def dealloc(self):
+        self.vec = None
+
+    def push(self, host_vals):
+        v = np.ascontiguousarray(host_vals, dtype=np.float32).reshape(-1)
+        if v.size != self.num_dia * self.stride:
+            raise RuntimeError("value vector has %d entries, expected %d" % (v.size, self.num_dia * self.stride))
+        self.vec = v.copy()
+        return self
+
+    def pull(self):
+        return self.vec.copy()
+
+
+class dev_dia_matrix_f(_dia_matrix_f):
+    """DIA matrix in device memory (src/cuv/basics/dia_matrix.hpp:57-276).
+    Element access copies one value between device and host, as the
+    reference's does (src/cuv/basics/reference.cu:18-28)."""
+
+    def __init__(self, h, w, num_dia, stride, row_fact=1, device="cuda:0"):
         self._desc = None
+        self._init_shape(h, w, num_dia, stride, row_fact)
+        self._device = device
+        self.vec = None
+        self.alloc()
+
+    def alloc(self):
+        self.vec = torch.zeros(self.num_dia * self.stride, dtype=torch.float32, device=self._device)
+
+    def dealloc(self):
+        self._drop_desc()
+        self.vec = None
 
     def __del__(self):
         self._drop_desc()
@@ -52,15 +178,12 @@ class dev_dia_matrix_f:
             _lib.lib().cuvdia_desc_destroy(self._desc)
             self._desc = None
 
-    def set_offsets(self, offsets):
-        offsets = np.ascontiguousarray(offsets, dtype=np.int32)
-        if offsets.size != self.num_dia:
-            raise RuntimeError("expected %d offsets" % self.num_dia)
-        self._offsets = offsets.copy()
+    def _init_shape(self, h, w, num_dia, stride, row_fact):
         self._drop_desc()
+        super()._init_shape(h, w, num_dia, stride, row_fact)
 
-    def get_offsets(self):
-        return self._offsets.copy()
+    def _offsets_changed(self):
+        self._drop_desc()
 
     @property
     def desc(self):
@@ -92,6 +215,132 @@ class dev_dia_matrix_f:
         return self.vec.cpu().numpy()
 
 
+def _adopt(dst, src):
+    """Gives dst the shape of src when they differ, as the reference's
+    conversions re-create a destination that does not fit
+    (src/cuv/convert/convert.cu:71-112)."""
+    if dst.shape != src.shape or dst.row_fact != src.row_fact or dst.vec is None \
+            or dst.num_dia != src.num_dia or dst.stride != src.stride:
+        dst._init_shape(src.h, src.w, src.num_dia, src.stride, src.row_fact)
+        dst.alloc()
+
+
+def dia_to_dense(src):
+    """Host DIA matrix -> dense (h, w) float32 array in column-major (Fortran)
+    order: zeros, then every stored diagonal's valid run
+    (src/cuv/convert/convert.cu:42-66)."""
+    if not isinstance(src, host_dia_matrix_f):
+        raise TypeError("dia_to_dense takes a host_dia_matrix_f")
+    dense = np.zeros((src.h, src.w), np.float32, order="F")
+    rf = src.row_fact
+    for o in src._offsets:
+        o = int(o)
+        i0, j0 = rf * max(0, -o), max(0, o)
+        n = min(src.h - i0, rf * (src.w - j0))
+        if n <= 0:
+            continue
+        i = i0 + np.arange(n)
+        dense[i, j0 + np.arange(n) // rf] = src.vec[src._dia2off[o] * src.stride + i]
+    return dense
+
+
+def convert(dst, src):
+    """The reference's DIA conversions (src/cuv_python/export_dia_mat.cpp:203-208):
+    host DIA -> device DIA, device DIA -> host DIA (offset table and value
+    vector copied, the destination re-created if it does not fit), and host
+    DIA -> dense, where dst is a writable (h, w) float32 NumPy array."""
+    if isinstance(dst, _dia_matrix_f) and isinstance(src, _dia_matrix_f):
+        if type(dst) is type(src):
+            raise TypeError("convert copies between a host and a device DIA matrix")
+        _adopt(dst, src)
+        dst.set_offsets(src.get_offsets())
+        dst.push(src.pull())
+        return dst
+    if isinstance(dst, np.ndarray) and isinstance(src, host_dia_matrix_f):
+        if dst.shape != src.shape or dst.dtype != np.float32:
+            raise RuntimeError("dst.shape() == src.shape()")
+        dst[...] = dia_to_dense(src)
+        return dst
+    raise TypeError("unsupported conversion")
+
+
+def pull(m):
+    """Device DIA matrix -> dense host matrix, through a host DIA copy
+    (dev_dia_mat2tensor, src/cuv_python/export_dia_mat.cpp:161-170)."""
+    if not isinstance(m, dev_dia_matrix_f):
+        raise TypeError("pull takes a dev_dia_matrix_f")
+    hostdia = host_dia_matrix_f(m.h, m.w, m.num_dia, m.stride, m.row_fact)
+    convert(hostdia, m)
+    return dia_to_dense(hostdia)
+
+
+class filter_factory_float:
+    """Offset tables of locally connected layers
+    (src/cuv/basics/filter_factory.hpp:13-80): an fs x fs window on a px x py
+    map, input_maps -> output_maps."""
+
+    def __init__(self, px, py, fs, input_maps, output_maps):
+        self.px, self.py, self.fs, self.input_maps, self.output_maps = px, py, fs, input_maps, output_maps
+        self.dias_per_filter = 0
+
+    def offsets(self):
+        """fs*fs*(output_maps + input_maps - 1) offsets i*px + j + m*px*py, map-major
+        then window row then window column, shifted by -(px+1)*(fs//2) -
+        (input_maps-1)*px*py (filter_factory.hpp:45-72)."""
+        px, py, fs = self.px, self.py, self.fs
+        m, i, j = np.meshgrid(np.arange(self.output_maps + self.input_maps - 1), np.arange(fs), np.arange(fs),
+                              indexing="ij")
+        off = (i * px + j + m * px * py).reshape(-1)
+        return (off - (px + 1) * (fs // 2) - (self.input_maps - 1) * px * py).astype(np.int32)
+
+    def get_dia(self, device=None):
+        """A zero-valued DIA matrix with that pattern: px*py*input_maps rows,
+        px*py*output_maps columns (filter_factory.hpp:43-76).  A host matrix,
+        or a device matrix when `device` is given."""
+        off = self.offsets()
+        n = self.px * self.py
+        h, w = n * self.input_maps, n * self.output_maps
+        self.dias_per_filter = self.fs * self.fs
+        dia = host_dia_matrix_f(h, w, off.size, max(h, w)) if device is None \
+            else dev_dia_matrix_f(h, w, off.size, max(h, w), device=device)
+        dia.set_offsets(off)
+        return dia
+
+    def extract_filter(self, dia, filternumber):
+        """The weights that feed column `filternumber`, per input map: a
+        (fs*fs, input_maps) row-major array whose flat entry map*fs*fs + k is
+        the k-th stored element (ascending row) of that column among the rows
+        of input map `map`; filling stops when the array is full.  This is
+        what filter_factory.hpp:22-41 sets out to do; its own statement of it
+        indexes the result pointer instead of the tensor and cannot be run, so
+        no reference output exists for it."""
+        if isinstance(dia, dev_dia_matrix_f):
+            hostdia = host_dia_matrix_f(dia.h, dia.w, dia.num_dia, dia.stride, dia.row_fact)
+            dia = convert(hostdia, dia)
+        fs2 = self.fs * self.fs
+        mat = np.zeros(fs2 * self.input_maps, np.float32)
+        map_size = dia.h // self.input_maps
+        for map_num in range(self.input_maps):
+            fi = 0
+            for i in range(map_size):
+                r = i + map_num * map_size
+                if not dia.has(r, filternumber):
+                    continue
+                mat[map_num * fs2 + fi] = dia(r, filternumber)
+                fi += 1
+                if map_num * fs2 + fi >= mat.size:
+                    break
+        return mat.reshape(fs2, self.input_maps)
+
+
+class host_block_descriptor_f:
+    """The reference's host descriptor is an empty stand-in
+    (src/cuv/matrix_ops/densedense_to_sparse.hpp:53-62); so is this."""
+
+    def __init__(self, dia):
+        self.dia = dia
+
+
 class dev_block_descriptor_f:
     """Kept for signature compatibility with densedense_to_dia(C, bd, A, B, ...)
     (src/cuv/matrix_ops/densedense_to_sparse.hpp:69-105); the run table lives in
@@ -103,6 +352,8 @@ class dev_block_descriptor_f:
 
     def len(self):
         return self.dia.info()["chunks_n"]
+
+    __len__ = len
 
 
 def prod(dst, A, B, transA="n", transB="n", factAB=1.0, factC=0.0, sync=True):
