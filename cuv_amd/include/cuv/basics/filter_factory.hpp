@@ -12,6 +12,7 @@
 #include <vector>
 
 #include <cuv/basics/dia_matrix.hpp>
+#include <cuv/basics/tensor.hpp>
 
 namespace cuv {
 
@@ -37,6 +38,33 @@ class filter_factory {
         const int shift = -(m_px + 1) * (m_fs / 2) - (m_input_maps - 1) * m_px * m_py;
         for (size_t i = 0; i < off.size(); i++) off[i] += shift;
         return off;
+    }
+
+    /// The weights that feed column `filternumber`, per input map: a new
+    /// (fs*fs) x input_maps row-major tensor (caller owns it) whose flat entry
+    /// map*fs*fs + k is the k-th stored element, rows ascending, of that
+    /// column among the rows of input map `map`; filling stops when the
+    /// tensor is full.  This is what src/cuv/basics/filter_factory.hpp:22-41
+    /// sets out to do; its own text indexes the result pointer rather than
+    /// the tensor, so there is no reference output to compare with.
+    template <class M2>
+    tensor<T, M, row_major> *extract_filter(const dia_matrix<T, M2, I> &dia, unsigned int filternumber)
+    {
+        const unsigned int fs2 = (unsigned int)(m_fs * m_fs);
+        tensor<T, M, row_major> *mat = new tensor<T, M, row_major>(extents[fs2][m_input_maps]);
+        const unsigned int total = mat->size();
+        for (unsigned int k = 0; k < total; ++k) (*mat)[k] = (T)0;
+        const unsigned int map_size = dia.h() / m_input_maps;
+        for (unsigned int map_num = 0; map_num < (unsigned int)m_input_maps; map_num++) {
+            unsigned int fi = 0;
+            for (unsigned int i = 0; i < map_size; ++i) {
+                const unsigned int row = i + map_num * map_size;
+                if (!dia.has(row, filternumber)) continue;
+                (*mat)[map_num * fs2 + fi++] = dia(row, filternumber);
+                if (map_num * fs2 + fi >= total) break;
+            }
+        }
+        return mat;
     }
 
     /// A new, value-uninitialised DIA matrix with that pattern (caller owns it).

@@ -179,4 +179,28 @@ TEST_CASE(filter_factory_offsets)
     delete d;
 }
 
+TEST_CASE(filter_factory_extract_filter)
+{
+    // 6 x 6 map, 3 x 3 window, two input maps -> one output map: column 14 is map
+    // position (2, 2), whose window lies fully inside both input maps
+    filter_factory<float, host_memory_space> ff(6, 6, 3, 2, 1);
+    dia_matrix<float, host_memory_space> *d = ff.get_dia();
+    CHECK(d->h() == 72 && d->w() == 36 && d->num_dia() == 18);
+    for (unsigned int i = 0; i < 72; i++)
+        for (unsigned int j = 0; j < 36; j++) d->set(i, j, 1000.f * i + j);
+    tensor<float, host_memory_space, row_major> *f = ff.extract_filter(*d, 14);
+    CHECK(f->shape(0) == 9 && f->shape(1) == 2);
+    for (unsigned int m = 0; m < 2; m++) {
+        unsigned int k = 0;
+        for (unsigned int i = m * 36; i < (m + 1) * 36; i++)
+            if (d->has(i, 14)) {
+                CHECK((float)(*f)[m * 9 + k] == 1000.f * i + 14);
+                k++;
+            }
+        CHECK(k == 9);
+    }
+    delete f;
+    delete d;
+}
+
 int main(int argc, char **argv) { return run_all(argc, argv); }
