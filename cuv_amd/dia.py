@@ -170,7 +170,12 @@ class dev_dia_matrix_f(_dia_matrix_f):
         self.vec = None
 
     def __del__(self):
-        self._drop_desc()
+        try:
+            self._drop_desc()
+        except Exception:
+            # interpreter shutdown: torch or the library may already be gone, and the
+            # process's device memory goes with it
+            pass
 
     def _drop_desc(self):
         if getattr(self, "_desc", None):
