@@ -30,6 +30,15 @@
 namespace cuvdia {
 namespace {
 
+// Results leave through non-temporal stores: they are streamed past the
+// caches instead of waiting there, dirty, for the write-back at the kernel's
+// end, which every store of a one-round kernel would otherwise meet at once.
+template <class V>
+__device__ __forceinline__ void stream_store(V *p, V v)
+{
+    __builtin_nontemporal_store(v, p);
+}
+
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and each
 // XCD has its own L2.  Remap so that every XCD works on contiguous spans of
 // tiles: neighbouring row tiles share dense-operand rows (the halo and the
@@ -170,7 +179,7 @@ __global__ __launch_bounds__(256) void spmm_generic_kernel(
             const float v = (beta == 0.f) ? alpha * acc[c] : beta * (*y) + alpha * acc[c];
             const unsigned col = (unsigned)(c0 + c);
             const unsigned word = ep.act == 2 ? sp_philox((unsigned)o, col >> 2, ep.seed_lo, ep.seed_hi).w[col & 3u] : 0u;
-            *y = sp_finish(v, ep.bias ? ep.bias[o] : 0.f, ep.act, word);
+            stream_store(y, sp_finish(v, ep.bias ? ep.bias[o] : 0.f, ep.act, word));
         }
     }
 }
@@ -693,7 +702,7 @@ __device__ __forceinline__ void spmm_tile_edge(
             if (col0 + col < batch) {
                 float *y = Y + (long long)(col0 + col) * ldy + row;
                 const float r = (beta == 0.f) ? alpha * v[q] : beta * ypre[q] + alpha * v[q];
-                *y = EP ? sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]) : r;
+                stream_store(y, EP ? sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]) : r);
             }
         }
     }
@@ -1016,7 +1025,7 @@ __device__ __forceinline__ void spmm_tile_lean(
             if (col0 + col < batch) {
                 float *y = Y + (long long)(col0 + col) * ldy + row;
                 const float r = (beta == 0.f) ? alpha * v[q] : beta * ypre[q] + alpha * v[q];
-                *y = sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]);
+                stream_store(y, sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3]));
             }
         }
     } else {
@@ -1043,7 +1052,7 @@ __device__ __forceinline__ void spmm_tile_lean(
                 // 4-byte alignment is all a 16-byte global store needs
                 float *y = Y + (long long)(col0 + col) * ldy + row0 + erow;
                 typedef float sp_f4u __attribute__((ext_vector_type(4), aligned(4)));
-                *reinterpret_cast<sp_f4u *>(y) = sp_f4u{r[0], r[1], r[2], r[3]};
+                stream_store(reinterpret_cast<sp_f4u *>(y), sp_f4u{r[0], r[1], r[2], r[3]});
             }
         }
     }
@@ -1477,7 +1486,7 @@ __device__ __forceinline__ void dd2dia_unit(
                 const unsigned off = c_offset(n, j);
                 if (off != OOB_OFFSET) {
                     float *cd = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
-                    *cd = (beta == 0.f) ? alpha * total : beta * cpre[n][j] + alpha * total;
+                    stream_store(cd, (beta == 0.f) ? alpha * total : beta * cpre[n][j] + alpha * total);
                 }
             }
     }
