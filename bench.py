@@ -58,6 +58,7 @@ def parse():
                     help="'step' (default): cfg1 + cfg2 + cfg3, the configuration the metric is quoted on; "
                          "'cfg4': the large layer (262144 rows, 676 diagonals, batch 256), each product timed "
                          "on its own -- an auxiliary line, no CPU leg (the oracle needs minutes for it); "
+                         "'scale': the headline layer's pattern at growing map and batch sizes, an auxiliary line; "
                          "'layer': the steps either side of the products at cfg1's shape (fused bias + sigmoid "
                          "(+ sample) against separate passes, the weight-decay step) -- an auxiliary line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -137,6 +138,76 @@ def bench_cfg4(args, torch, D, W, dev):
                              "batch 256; forward, transposed and gradient products each timed alone",
                     rows=n, diagonals=nd, batch=batch, nnz=nnz),
         ops=res, aux=aux, note="bound by the fp32 vector rate (57 FLOP per algorithmic byte), not by HBM")))
+
+
+def bench_scale(args, torch, D, W, dev):
+    """The layer of the headline configuration (7x7 window, one channel, 49 diagonals) at growing map and
+    batch sizes: shows what the same kernels reach once a launch holds many rounds of workgroups and its fixed
+    costs (launch, first loads, final stores) no longer weigh.  Inputs are drawn on the device; from the second case
+    on the operands of a call exceed the 256 MB Infinity Cache, so every launch streams from HBM."""
+    cases = [(128, 128), (128, 512), (128, 2048), (128, 4096), (256, 1024), (512, 128), (512, 512), (1024, 128)]
+    g = torch.Generator(device=dev)
+    g.manual_seed(0xC0FFEE + 5)
+    stream = torch.cuda.current_stream()
+    out = []
+    for px, batch in cases:
+        n = px * px
+        p = W.Pattern(n, n, W.window_offsets(px, 7), n)
+        nd = p.nd
+
+        def dia():
+            m = D.dev_dia_matrix_f(n, n, nd, n, 1, device=dev)
+            m.set_offsets(p.offsets)
+            m.vec.copy_(torch.randn(nd * n, generator=g, device=dev) * 0.01)
+            return m
+        A, G = dia(), dia()
+        X = torch.rand(batch, n, generator=g, device=dev)
+        H = torch.rand(batch, n, generator=g, device=dev)
+        Y = torch.rand(batch, n, generator=g, device=dev)
+        bd = D.dev_block_descriptor_f(G)
+        A.desc
+        ops = {
+            "up_pass": (lambda: D.prod(Y, A, X, "n", "n", 1.0, 0.0, sync=False), W.spmm_bytes(p, batch, "n", 0.0)),
+            "down_pass": (lambda: D.prod(Y, A, H, "t", "n", 1.0, 0.5, sync=False), W.spmm_bytes(p, batch, "t", 0.5)),
+            "weight_gradient": (lambda: D.densedense_to_dia(G, bd, X, H, 1.0 / batch, 0.9, sync=False),
+                                W.dd2dia_bytes(p, batch, 0.9)),
+        }
+        flops = W.flops(p, batch)
+        row = dict(map=px, rows=n, batch=batch, flops=flops)
+        for name, (fn, nbytes) in ops.items():
+            # ten launches per graph replay: Python cannot issue launches every few microseconds
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(10):
+                    fn()
+            graph.replay()
+            torch.cuda.synchronize()
+            reps = max(2, min(20, int(2e4 / max(1.0, nbytes / 2e6))))
+            s = torch.cuda.current_stream()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(s)
+            for _ in range(reps):
+                graph.replay()
+            e1.record(s)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / (10 * reps) * 1e3
+            row[name] = dict(us=us, bytes=nbytes, gbs=nbytes / us / 1e3, frac_hbm=nbytes / us / 1e3 / HBM_PEAK_GBS,
+                             tflops=flops / us / 1e6)
+            del graph
+        out.append(row)
+        del A, G, X, H, Y, bd
+        torch.cuda.empty_cache()
+    best = max(r[k]["gbs"] for r in out for k in ("up_pass", "down_pass", "weight_gradient"))
+    print(json.dumps(dict(
+        metric="achieved HBM GB/s, DIA SpMM (both transposes) + densedense_to_dia, size sweep", unit="GB/s",
+        value=best, n_gpus=1, steps=None, warmup=3, higher_is_better=True, scaling="weak", vs_baseline=None,
+        dtype="f32", data="synthetic",
+        config=dict(workload="7x7 window on a px x px map (49 diagonals), batch b, for several (px, b); "
+                             "each product timed alone; value = the best single figure of the sweep"),
+        cases=out)))
 
 
 def bench_layer(args, torch, D, W, dev):
@@ -227,6 +298,8 @@ def main():
 
     if args.workload == "cfg4":
         return bench_cfg4(args, torch, D, W, dev)
+    if args.workload == "scale":
+        return bench_scale(args, torch, D, W, dev)
     if args.workload == "layer":
         return bench_layer(args, torch, D, W, dev)
 

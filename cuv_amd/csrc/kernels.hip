@@ -38,6 +38,12 @@ __device__ __forceinline__ void stream_store(V *p, V v)
 {
     __builtin_nontemporal_store(v, p);
 }
+// Four consecutive floats as one 16-byte store; 4-byte alignment is all a 16-byte global store needs.
+__device__ __forceinline__ void stream_store4(float *p, float a, float b, float c, float d)
+{
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    __builtin_nontemporal_store(f4u{a, b, c, d}, reinterpret_cast<f4u *>(p));
+}
 
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, and each
 // XCD has its own L2.  Remap so that every XCD works on contiguous spans of
@@ -1049,10 +1055,7 @@ __device__ __forceinline__ void spmm_tile_lean(
                     const float t = (beta == 0.f) ? alpha * s[e] : beta * ypre[4 * k + e] + alpha * s[e];
                     r[e] = EP ? sp_finish(t, b4[e], ep.act) : t;
                 }
-                // 4-byte alignment is all a 16-byte global store needs
-                float *y = Y + (long long)(col0 + col) * ldy + row0 + erow;
-                typedef float sp_f4u __attribute__((ext_vector_type(4), aligned(4)));
-                stream_store(reinterpret_cast<sp_f4u *>(y), sp_f4u{r[0], r[1], r[2], r[3]});
+                stream_store4(Y + (long long)(col0 + col) * ldy + row0 + erow, r[0], r[1], r[2], r[3]);
             }
         }
     }
@@ -1063,16 +1066,30 @@ template <int LCK, int T, int NTAB, bool EP>
 __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
-    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes,
+    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, int col_group, unsigned a_bytes,
     int s_min, int s_max, SpEpilogue ep)
 {
     static_assert(3 * SP_DSTAGE_FLOATS >= 2 * SP_STAGE_FLOATS, "the two bodies share one LDS block");
     __shared__ __attribute__((aligned(16))) float lds3[3][SP_DSTAGE_FLOATS];
     float (&lds)[2][SP_STAGE_FLOATS] = *reinterpret_cast<float (*)[2][SP_STAGE_FLOATS]>(&lds3[0][0]);
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int rowtile = tile / col_tiles;
+    // Tiles are numbered column group by column group; inside a group of col_group column tiles the
+    // column tile runs fastest, then the row tile.  The 64 tiles an XCD holds at a time are then
+    // 64 / col_group neighbouring row tiles -- which share the dense rows of their bands -- of the same few
+    // column tiles, however wide the batch is.
+    int rowtile, coltile;
+    if (col_group >= col_tiles) {
+        rowtile = tile / col_tiles;
+        coltile = tile - rowtile * col_tiles;
+    } else {
+        const int per_group = (int)(gridDim.x / (unsigned)col_tiles) * col_group;
+        const int g = tile / per_group, in = tile - g * per_group;
+        const int width = min(col_group, col_tiles - g * col_group);
+        rowtile = in / width;
+        coltile = g * col_group + (in - rowtile * width);
+    }
     const int row0 = rowtile * SP_ROWS;
-    const int col0 = (tile - rowtile * col_tiles) * SP_COLS;
+    const int col0 = coltile * SP_COLS;
     // The lean body serves a tile all of whose 64 output rows exist and none of
     // whose chunks straddles an end of the operand: each chunk's staged rows
     // [row0 + s0, row0 + s0 + 80) lie either inside it or wholly outside (such
@@ -1577,10 +1594,17 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const unsigned a_bytes = (unsigned)((long long)A.nd * A.stride * 4);
     const int s_min = trans ? A.s_min_t : A.s_min_n, s_max = trans ? A.s_max_t : A.s_max_n;
     const dim3 grid((unsigned)(row_tiles * col_tiles));
+    // Up to 4 column tiles form one group (the diagonals are fetched once per group and row tile); wider
+    // batches are walked in groups of 2 column tiles, so that the tiles resident in an XCD stay neighbours
+    // along the rows and find each other's dense rows in its L2.
+#ifndef SP_COL_GROUP
+#define SP_COL_GROUP 2
+#endif
+    const int col_group = col_tiles <= 4 ? (int)col_tiles : SP_COL_GROUP;
     // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
     // at the sizes this path is measured on.
 #define CUVDIA_SPMM_ARGS chunks, nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha, \
-                         beta, (int)col_tiles, a_bytes, s_min, s_max, ep
+                         beta, (int)col_tiles, col_group, a_bytes, s_min, s_max, ep
 #define CUVDIA_SPMM_LAUNCH(L)                                                                                   \
     case L:                                                                                                     \
         if (nchunks <= 64 && !fused)                                                                            \

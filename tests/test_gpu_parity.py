@@ -118,6 +118,11 @@ SHAPES = [
     (512, 640, [dy * 96 + dx for dy in range(-1, 2) for dx in range(-6, 7)], 1, 72),
     (768, 512, list(range(-4, 5)) + [100 + k for k in range(12)], 1, 33),
     (1280, 1280, [dy * 128 + dx for dy in range(-4, 5) for dx in range(-4, 5)], 1, 128),
+    # batches wider than 4 column tiles (walked in groups of 2 column tiles): 5 tiles (groups 2, 2, 1),
+    # 8 tiles with a ragged last one, 10 tiles whose last holds a single column
+    (384, 384, [dy * 32 + dx for dy in range(-1, 2) for dx in range(-2, 3)], 1, 320),
+    (200, 333, list(range(-20, 21)), 1, 449),
+    (700, 650, [d * 25 + e for d in range(-2, 3) for e in range(-2, 3)], 1, 577),
 ]
 
 
