@@ -772,7 +772,9 @@ constexpr int SP_DSTAGE_FLOATS = SP_DAVALS + SP_AVALS;
 static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + SP_CHUNK_MAX - 1 <= SP_DPITCH && SP_CHUNK_MAX <= SP_ADIAGS,
               "staging layout");
 
-template <int LCK, int NTAB, bool EP>
+// INNER: every chunk the call walks lies wholly inside the operand (true for all but the tiles near its ends);
+// the loop then carries neither the tests that tell such chunks from the others nor the code for the others.
+template <int LCK, int NTAB, bool EP, bool INNER>
 __device__ __forceinline__ void spmm_tile_lean(
     float (&lds)[3][SP_DSTAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
@@ -874,8 +876,8 @@ __device__ __forceinline__ void spmm_tile_lean(
         const int a0 = row0 + s0;
         // past the table, and for a chunk whose rows lie outside the operand,
         // nothing is fetched: an empty resource delivers zeros
-        const bool inside = (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
-        const bool outside = (a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in);
+        const bool inside = INNER || ((a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in));
+        const bool outside = !INNER && ((a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in));
         const bool real = (c < nchunks) & !outside;
         const sp_int4 xq = raw_rsrc(xbase, real ? x_bytes : 0u);
         if (LCK > 8 || (inside | !real)) {       // (longer chunks never come here crossing an end: see the kernel)
@@ -940,8 +942,8 @@ __device__ __forceinline__ void spmm_tile_lean(
     auto read_window = [&](SpWindow<LCK, T> &win, int b, int s0) __attribute__((always_inline)) {
         const float *buf = lds[b];
         const int a0 = row0 + s0;
-        const bool inside = (a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in);
-        const bool outside = (a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in);
+        const bool inside = INNER || ((a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in));
+        const bool outside = !INNER && ((a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in));
         if (LCK > 8 || (inside | outside)) {
             spmm_read_window<LCK, T>(win, buf + lane * SP_DPITCH + wave * T, buf + SP_DAVALS + wave * T + (lane & (T - 1)));
         } else {
@@ -1104,6 +1106,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     // the half of the buffer's diagonal block that longer chunks would need).
     const bool crossing_ok = (LCK <= 8) & ((n_in & 3) == 0);
     int crossing = 0;
+    bool inner = true;                              // every walked chunk lies wholly inside the operand
     if (!((row0 + s_min >= 0) & (row0 + s_max + STAGED <= n_in))) {
         const int lane = threadIdx.x & 63;
         c_lo = nchunks;
@@ -1124,13 +1127,18 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
         if (c_hi <= c_lo) {                          // nothing inside: one (outside) chunk keeps the pipeline fed
             c_lo = 0;
             c_hi = 1;
+            inner = false;
         }
+        inner &= crossing == 0;
         lean &= crossing == 0 || crossing_ok;
     }
-    if (lean)
-        // only the chunks inside the operand are walked; the others would add zeros
-        spmm_tile_lean<LCK, NTAB, EP>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
-                                      Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
+    // only the chunks inside the operand are walked; the others would add zeros
+    if (lean && inner)
+        spmm_tile_lean<LCK, NTAB, EP, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
+                                            Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
+    else if (lean)
+        spmm_tile_lean<LCK, NTAB, EP, false>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
+                                             Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
     else
         spmm_tile_edge<LCK, T, NTAB, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                          n_out, n_in, batch, alpha, beta, a_bytes, ep);
