@@ -871,7 +871,10 @@ __device__ __forceinline__ void spmm_tile_lean(
         }
     };
     // requests chunk c, whose entry is en, into the buffer at byte address `buf`: 3 or 2 loads
-    auto issue = [&](int c, unsigned buf, const Entry &en) __attribute__((always_inline)) {
+    // two_c: std::true_type where the caller knows that this wave issues two loads per chunk (neither a third
+    // piece of the dense rows nor diagonals), so that its copy of the loop carries no test for either
+    auto issue = [&](int c, unsigned buf, const Entry &en, auto two_c) __attribute__((always_inline)) {
+        constexpr bool TWO = decltype(two_c)::value;
         const int s0 = en.s0;
         const int a0 = row0 + s0;
         // past the table, and for a chunk whose rows lie outside the operand,
@@ -884,7 +887,7 @@ __device__ __forceinline__ void spmm_tile_lean(
             const unsigned soff = (real & inside) ? (unsigned)a0 * 4u : 0u;
             lds_load_b128(xq, buf + x_lds[0], x_off[0], soff);
             lds_load_b128(xq, buf + x_lds[1], x_off[1], soff);
-            if (x3) lds_load_b128(xq, buf + x_lds[2], x_off[2], soff);
+            if (!TWO && x3) lds_load_b128(xq, buf + x_lds[2], x_off[2], soff);
         } else {
             // The chunk's rows cross an end of the operand.  The staged block then starts at the multiple of
             // 4 at or below a0 (so that, the operand's row count being a multiple of 4 too, every 16-byte
@@ -917,10 +920,10 @@ __device__ __forceinline__ void spmm_tile_lean(
                 const int r = a0p + 4 * x_quad[it];
                 const bool ok = (r >= 0) & (r + 4 <= n_in);
                 const unsigned voff = ok ? x_off[it] + (unsigned)(a0p * 4) : OOB_OFFSET;
-                if (it < 2 || x3) lds_load_b128(xq, buf + x_lds[it], voff, 0u);
+                if (it < 2 || (!TWO && x3)) lds_load_b128(xq, buf + x_lds[it], voff, 0u);
             }
         }
-        if (a_wave) {
+        if (!TWO && a_wave) {
             // table position of this lane's diagonal, a_j: picked from the 8 scalars (each passed through an
             // empty asm so that the chain of selects stays one, and the entry stays in registers)
             constexpr int NP = LCK > 8 ? SP_CHUNK_MAX : 8;
@@ -962,9 +965,9 @@ __device__ __forceinline__ void spmm_tile_lean(
     int s_cur, s_n1, s_n2;                  // shifts of the chunk whose window is read next, and of the two after it
     {
         const Entry h0 = fetch(0), h1 = fetch(1), h2 = fetch(2);
-        issue(0, lds0, h0);
-        issue(1, lds0 + BUF_BYTES, h1);
-        issue(2, lds0 + 2 * BUF_BYTES, h2);
+        issue(0, lds0, h0, std::false_type{});
+        issue(1, lds0 + BUF_BYTES, h1, std::false_type{});
+        issue(2, lds0 + 2 * BUF_BYTES, h2, std::false_type{});
         s_cur = h0.s0;
         s_n1 = h1.s0;
         s_n2 = h2.s0;
@@ -980,17 +983,21 @@ __device__ __forceinline__ void spmm_tile_lean(
     // the entry of chunk c+4.  The FMAs of chunk c are cut in two: the wait for chunk c+1, the barrier
     // and the read of its window sit between the halves, so the second half hides the read and a chunk
     // is waited for only when its turn has come -- the product starts with one chunk in LDS, not two.
+    // The loop exists twice, for the waves that issue three loads per chunk and for those that issue two: the
+    // waits are then fixed instructions, not a choice made in every iteration.
     constexpr int JH = (LCK + 1) / 2;
+    auto run_loop = [&](auto three_c) __attribute__((always_inline)) {
+    constexpr bool THREE = decltype(three_c)::value;
     auto iteration = [&](int c, int b, int b1, SpWindow<LCK, T> &cur, SpWindow<LCK, T> &nxt, const Entry &use, Entry &next) __attribute__((always_inline)) {
         spmm_rows_range<LCK, T, 0, JH>(acc, cur);
         // chunk c+1 must be in; the loads of chunk c+2 (requested whenever c+2 < 3 or it exists) may stay out
         const bool younger = (c + 2 < 3) | (c + 2 < nchunks);
         if (!younger) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        else if (three) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
+        else if (THREE) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
         __syncthreads();                                 // also: every wave holds window(c), buffer b may be reused
         if (c + 1 < nchunks) read_window(nxt, b1, s_n1);
-        if (c + 3 < nchunks) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use);
+        if (c + 3 < nchunks) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use, std::integral_constant<bool, !THREE>{});
         s_n1 = s_n2;
         s_n2 = use.s0;
         next = fetch(c + 4);
@@ -1009,6 +1016,9 @@ __device__ __forceinline__ void spmm_tile_lean(
         iteration(c + 1, b1, b2, w1, w0, e1, e0);
         { const int t0 = b, t1 = b1; b = b2; b1 = t0; b2 = t1; }
     }
+    };
+    if (three) run_loop(std::true_type{});
+    else run_loop(std::false_type{});
     // every wave must be through with its window reads, and no load in flight, before the buffers are reused
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
