@@ -9,8 +9,10 @@
 //              each kernel below.
 //
 // Accumulation order (fp32, fused multiply-add, per output element):
-//   spmm    acc = 0; for each run chunk in ascending shift order, for each
-//           diagonal of the chunk in ascending shift order:
+//   spmm    acc = 0; for each run chunk in ascending shift order (a tile with
+//           exactly one chunk whose rows cross an end of the dense operand
+//           takes that chunk first), for each diagonal of the chunk in
+//           ascending shift order:
 //           acc = fma(a, x, acc); then dst = beta*dst + alpha*acc
 //           (dst = alpha*acc when beta == 0, dst never read).
 //           The generic kernel walks the offset table in table order instead.
@@ -772,14 +774,18 @@ constexpr int SP_DSTAGE_FLOATS = SP_DAVALS + SP_AVALS;
 static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + SP_CHUNK_MAX - 1 <= SP_DPITCH && SP_CHUNK_MAX <= SP_ADIAGS,
               "staging layout");
 
-// INNER: every chunk the call walks lies wholly inside the operand (true for all but the tiles near its ends);
+// INNER: every chunk the loop requests or reads (all but the first chunk walked) lies wholly inside the operand;
 // the loop then carries neither the tests that tell such chunks from the others nor the code for the others.
-template <int LCK, int NTAB, bool EP, bool INNER>
+// FIRST_ANY: the first chunk walked may cross an end of the operand (it is requested and read before the loop).
+// `first` is the table position (relative to `chunks`) of the chunk to walk first, the others following in table
+// order: a tile with one crossing chunk takes that one first and runs the INNER loop.  All chunks inside:
+// <INNER, !FIRST_ANY>; one crossing chunk: <INNER, FIRST_ANY>; anything else: <!INNER, FIRST_ANY>, first = 0.
+template <int LCK, int NTAB, bool EP, bool INNER, bool FIRST_ANY>
 __device__ __forceinline__ void spmm_tile_lean(
     float (&lds)[3][SP_DSTAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
-    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, SpEpilogue ep)
+    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, int first, SpEpilogue ep)
 {
     constexpr int T = 8, WAVES = 8, CPW = SP_COLS / WAVES;
     const int lane = threadIdx.x & 63;
@@ -861,7 +867,10 @@ __device__ __forceinline__ void spmm_tile_lean(
     auto fetch = [&](int c) __attribute__((always_inline)) {
         typedef int sp_i4 __attribute__((ext_vector_type(4)));
         typedef const sp_i4 __attribute__((address_space(4))) *sc_i4_ptr;
-        const sc_i4_ptr e = (sc_i4_ptr)(chunks + min(c, nchunks - 1));
+        int at = c;
+        if constexpr (FIRST_ANY) at = c == 0 ? first : (c <= first ? c - 1 : c);       // `first` moved to the front
+        at = min(at, nchunks - 1);
+        const sc_i4_ptr e = (sc_i4_ptr)(chunks + at);
         const sp_i4 e0 = e[0], e1 = e[1], e2 = e[2];
         if constexpr (LCK > 8) {
             const sp_i4 e3 = e[3];
@@ -873,14 +882,16 @@ __device__ __forceinline__ void spmm_tile_lean(
     // requests chunk c, whose entry is en, into the buffer at byte address `buf`: 3 or 2 loads
     // two_c: std::true_type where the caller knows that this wave issues two loads per chunk (neither a third
     // piece of the dense rows nor diagonals), so that its copy of the loop carries no test for either
-    auto issue = [&](int c, unsigned buf, const Entry &en, auto two_c) __attribute__((always_inline)) {
+    // inner_c: std::true_type where the caller knows the chunk to lie wholly inside the operand
+    auto issue = [&](int c, unsigned buf, const Entry &en, auto two_c, auto inner_c) __attribute__((always_inline)) {
         constexpr bool TWO = decltype(two_c)::value;
+        constexpr bool IN = decltype(inner_c)::value;
         const int s0 = en.s0;
         const int a0 = row0 + s0;
         // past the table, and for a chunk whose rows lie outside the operand,
         // nothing is fetched: an empty resource delivers zeros
-        const bool inside = INNER || ((a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in));
-        const bool outside = !INNER && ((a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in));
+        const bool inside = IN || ((a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in));
+        const bool outside = !IN && ((a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in));
         const bool real = (c < nchunks) & !outside;
         const sp_int4 xq = raw_rsrc(xbase, real ? x_bytes : 0u);
         if (LCK > 8 || (inside | !real)) {       // (longer chunks never come here crossing an end: see the kernel)
@@ -942,11 +953,12 @@ __device__ __forceinline__ void spmm_tile_lean(
     // Reads the window of the chunk whose shift is s0.  A chunk that crosses an end of the operand was staged
     // from the multiple of 4 below its first row: its window starts up to 3 rows into the column (4-byte
     // reads then), and its diagonal values sit in the wave's own corner of the buffer (see issue).
-    auto read_window = [&](SpWindow<LCK, T> &win, int b, int s0) __attribute__((always_inline)) {
+    auto read_window = [&](SpWindow<LCK, T> &win, int b, int s0, auto inner_c) __attribute__((always_inline)) {
+        constexpr bool IN = decltype(inner_c)::value;
         const float *buf = lds[b];
         const int a0 = row0 + s0;
-        const bool inside = INNER || ((a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in));
-        const bool outside = !INNER && ((a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in));
+        const bool inside = IN || ((a0 >= 0) & (a0 + 4 * SP_DQUADS <= n_in));
+        const bool outside = !IN && ((a0 + 4 * SP_DQUADS <= 0) | (a0 >= n_in));
         if (LCK > 8 || (inside | outside)) {
             spmm_read_window<LCK, T>(win, buf + lane * SP_DPITCH + wave * T, buf + SP_DAVALS + wave * T + (lane & (T - 1)));
         } else {
@@ -965,9 +977,9 @@ __device__ __forceinline__ void spmm_tile_lean(
     int s_cur, s_n1, s_n2;                  // shifts of the chunk whose window is read next, and of the two after it
     {
         const Entry h0 = fetch(0), h1 = fetch(1), h2 = fetch(2);
-        issue(0, lds0, h0, std::false_type{});
-        issue(1, lds0 + BUF_BYTES, h1, std::false_type{});
-        issue(2, lds0 + 2 * BUF_BYTES, h2, std::false_type{});
+        issue(0, lds0, h0, std::false_type{}, std::integral_constant<bool, !FIRST_ANY>{});
+        issue(1, lds0 + BUF_BYTES, h1, std::false_type{}, std::integral_constant<bool, INNER>{});
+        issue(2, lds0 + 2 * BUF_BYTES, h2, std::false_type{}, std::integral_constant<bool, INNER>{});
         s_cur = h0.s0;
         s_n1 = h1.s0;
         s_n2 = h2.s0;
@@ -978,7 +990,7 @@ __device__ __forceinline__ void spmm_tile_lean(
     if (three) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     __syncthreads();
-    read_window(w0, 0, s_cur);
+    read_window(w0, 0, s_cur, std::integral_constant<bool, !FIRST_ANY>{});
     // Iteration c: buffers b (chunk c), b1 (chunk c+1); `use` is the entry of chunk c+3, `next` receives
     // the entry of chunk c+4.  The FMAs of chunk c are cut in two: the wait for chunk c+1, the barrier
     // and the read of its window sit between the halves, so the second half hides the read and a chunk
@@ -996,8 +1008,9 @@ __device__ __forceinline__ void spmm_tile_lean(
         else if (THREE) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
         __syncthreads();                                 // also: every wave holds window(c), buffer b may be reused
-        if (c + 1 < nchunks) read_window(nxt, b1, s_n1);
-        if (c + 3 < nchunks) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use, std::integral_constant<bool, !THREE>{});
+        if (c + 1 < nchunks) read_window(nxt, b1, s_n1, std::integral_constant<bool, INNER>{});
+        if (c + 3 < nchunks) issue(c + 3, lds0 + (unsigned)b * BUF_BYTES, use, std::integral_constant<bool, !THREE>{},
+                                   std::integral_constant<bool, INNER>{});
         s_n1 = s_n2;
         s_n2 = use.s0;
         next = fetch(c + 4);
@@ -1115,7 +1128,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     // The lean body takes such chunks when they have at most 8 diagonals (their values are fetched into
     // the half of the buffer's diagonal block that longer chunks would need).
     const bool crossing_ok = (LCK <= 8) & ((n_in & 3) == 0);
-    int crossing = 0;
+    int crossing = 0, cross_at = nchunks;           // chunks crossing an end of the operand, and the first of them
     bool inner = true;                              // every walked chunk lies wholly inside the operand
     if (!((row0 + s_min >= 0) & (row0 + s_max + STAGED <= n_in))) {
         const int lane = threadIdx.x & 63;
@@ -1127,7 +1140,9 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
             const int a0 = row0 + chunks[min(idx, nchunks - 1)].s0;
             const bool inside = (a0 >= 0) & (a0 + STAGED <= n_in);
             const bool outside = (a0 + STAGED <= 0) | (a0 >= n_in);
-            crossing += (int)__builtin_popcountll(__builtin_amdgcn_ballot_w64(!(inside | outside) & (idx < nchunks)));
+            const unsigned long long cm = __builtin_amdgcn_ballot_w64(!(inside | outside) & (idx < nchunks));
+            crossing += (int)__builtin_popcountll(cm);
+            if (cm) cross_at = min(cross_at, 64 * k + (int)__builtin_ctzll(cm));
             const unsigned long long m = __builtin_amdgcn_ballot_w64(!outside & (idx < nchunks));
             if (m) {
                 c_lo = min(c_lo, 64 * k + (int)__builtin_ctzll(m));
@@ -1143,12 +1158,17 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
         lean &= crossing == 0 || crossing_ok;
     }
     // only the chunks inside the operand are walked; the others would add zeros
+    // A tile with one crossing chunk walks that chunk first: everything the loop then touches lies inside.
     if (lean && inner)
-        spmm_tile_lean<LCK, NTAB, EP, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
-                                            Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
+        spmm_tile_lean<LCK, NTAB, EP, true, false>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
+                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, ep);
+    else if (lean && crossing == 1 && c_hi > c_lo)
+        spmm_tile_lean<LCK, NTAB, EP, true, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
+                                                  ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes,
+                                                  cross_at - c_lo, ep);
     else if (lean)
-        spmm_tile_lean<LCK, NTAB, EP, false>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X, ldx,
-                                             Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, ep);
+        spmm_tile_lean<LCK, NTAB, EP, false, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
+                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, ep);
     else
         spmm_tile_edge<LCK, T, NTAB, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                          n_out, n_in, batch, alpha, beta, a_bytes, ep);
