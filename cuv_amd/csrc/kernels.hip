@@ -1370,10 +1370,11 @@ __device__ __forceinline__ void dd2dia_unit(
     // current one has gone to LDS.
     float4 bq[DD_BG][2];
     // requests column i of group g: B rows into bq, A rows into st.a
+    const unsigned rare_span = (unsigned)(rare_hi - rare_lo);
     auto issue_col = [&](int g, int i, DdStage &st) {
         const int b0 = __builtin_amdgcn_readfirstlane(g * DD_BG);   // wave-uniform: keeps column offsets scalar
         const int col = b0 + i;
-        const bool live = (col >= rare_lo) & (col < rare_hi);
+        const bool live = (unsigned)(col - rare_lo) < rare_span;      // rare_lo <= col < rare_hi in one compare
         const __amdgpu_buffer_rsrc_t br = make_rsrc(B, live ? b_bytes : 0u);
         const unsigned colb = (unsigned)col * ldb4;
         const unsigned v0 = vb_off0 + colb;
