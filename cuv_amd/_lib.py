@@ -32,7 +32,7 @@ def lib():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(
-            "libcuvdia.so is not built (%s); run `make -C cuv_amd/csrc` "
+            "libcuvdia.so is not built (%s); run `make -j6 -C cuv_amd/csrc` "
             "or __graft_entry__.build()" % LIB_PATH)
     L = ctypes.CDLL(LIB_PATH)
     c_int, c_ll, c_f, c_vp, c_char = (ctypes.c_int, ctypes.c_longlong, ctypes.c_float,

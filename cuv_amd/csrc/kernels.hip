@@ -29,6 +29,15 @@
 
 #include "kernels.hpp"
 
+// This file is compiled four times (CUVDIA_PART = 1 .. 4, see the Makefile), each translation unit
+// instantiating one share of the kernel templates, so that the shares compile in parallel: parts 1 - 3 hold
+// the tiled SpMM kernels by longest chunk (1 - 5, 6 - 9, 10 - 13), part 4 everything else.  Without the macro
+// one unit holds everything.
+#ifndef CUVDIA_PART
+#define CUVDIA_PART 0
+#endif
+#define CUVDIA_IN_PART(p) (CUVDIA_PART == 0 || CUVDIA_PART == (p))
+
 namespace cuvdia {
 namespace {
 
@@ -1585,6 +1594,7 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
 
 // ---------------------------------------------------------------- launchers --
 
+#if CUVDIA_IN_PART(4)
 hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float *B, long long ldb,
                                float *dst, long long ldd, int batch, bool trans,
                                float alpha, float beta, SpEpilogue ep, hipStream_t stream)
@@ -1618,6 +1628,85 @@ bool spmm_tiled_ok(const DiaView &A, long long ldb, long long ldd, bool trans)
            y_bytes < (long long)OOB_OFFSET && a_bytes < (long long)OOB_OFFSET;
 }
 
+#endif  // part 4
+
+// Everything a launch of the tiled SpMM kernel needs; the launch itself lives in the unit that
+// instantiates the kernel for the table's longest chunk.
+struct SpLaunch {
+    const Chunk *chunks;
+    int nchunks;
+    const float *vals;
+    int stride, ashift;
+    const float *B;
+    long long ldb;
+    float *dst;
+    long long ldd;
+    int n_out, n_in, batch;
+    float alpha, beta;
+    int col_tiles, col_group;
+    unsigned a_bytes;
+    int s_min, s_max;
+    SpEpilogue ep;
+    dim3 grid;
+    hipStream_t stream;
+    int lck;
+};
+hipError_t spmm_tiled_launch_1_5(const SpLaunch &L);
+hipError_t spmm_tiled_launch_6_9(const SpLaunch &L);
+hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
+
+// 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
+// at the sizes this path is measured on.
+#define CUVDIA_SPMM_ARGS L.chunks, L.nchunks, L.vals, L.stride, L.ashift, L.B, L.ldb, L.dst, L.ldd, L.n_out, L.n_in, \
+                         L.batch, L.alpha, L.beta, L.col_tiles, L.col_group, L.a_bytes, L.s_min, L.s_max, L.ep
+#define CUVDIA_SPMM_LAUNCH(K)                                                                                         \
+    case K:                                                                                                           \
+        if (L.nchunks <= 64 && !fused)                                                                                \
+            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 1, false>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS); \
+        else if (L.nchunks <= 64)                                                                                     \
+            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 1, true>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS);  \
+        else if (!fused)                                                                                              \
+            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 4, false>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS); \
+        else                                                                                                          \
+            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 4, true>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS);  \
+        break;
+#if CUVDIA_IN_PART(1)
+hipError_t spmm_tiled_launch_1_5(const SpLaunch &L)
+{
+    const bool fused = L.ep.bias != nullptr || L.ep.act != 0;
+    switch (L.lck) {
+        CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4) CUVDIA_SPMM_LAUNCH(5)
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+#endif
+#if CUVDIA_IN_PART(2)
+hipError_t spmm_tiled_launch_6_9(const SpLaunch &L)
+{
+    const bool fused = L.ep.bias != nullptr || L.ep.act != 0;
+    switch (L.lck) {
+        CUVDIA_SPMM_LAUNCH(6) CUVDIA_SPMM_LAUNCH(7) CUVDIA_SPMM_LAUNCH(8) CUVDIA_SPMM_LAUNCH(9)
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+#endif
+#if CUVDIA_IN_PART(3)
+hipError_t spmm_tiled_launch_10_13(const SpLaunch &L)
+{
+    const bool fused = L.ep.bias != nullptr || L.ep.act != 0;
+    switch (L.lck) {
+        CUVDIA_SPMM_LAUNCH(10) CUVDIA_SPMM_LAUNCH(11) CUVDIA_SPMM_LAUNCH(12) CUVDIA_SPMM_LAUNCH(13)
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+#endif
+#undef CUVDIA_SPMM_LAUNCH
+#undef CUVDIA_SPMM_ARGS
+
+#if CUVDIA_IN_PART(4)
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, SpEpilogue ep, hipStream_t stream)
@@ -1627,45 +1716,20 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     const long long row_tiles = (n_out + SP_ROWS - 1) / SP_ROWS;
     const long long col_tiles = (batch + SP_COLS - 1) / SP_COLS;
     if (row_tiles * col_tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-    const Chunk *chunks = trans ? A.chunks_t_dev : A.chunks_n_dev;
-    const int nchunks = trans ? A.n_chunks_t : A.n_chunks_n;
-    const int lck = trans ? A.max_len_t : A.max_len_n;
-    const unsigned a_bytes = (unsigned)((long long)A.nd * A.stride * 4);
-    const int s_min = trans ? A.s_min_t : A.s_min_n, s_max = trans ? A.s_max_t : A.s_max_n;
-    const dim3 grid((unsigned)(row_tiles * col_tiles));
     // Up to 4 column tiles form one group (the diagonals are fetched once per group and row tile); wider
     // batches are walked in groups of 2 column tiles, so that the tiles resident in an XCD stay neighbours
     // along the rows and find each other's dense rows in its L2.
-#ifndef SP_COL_GROUP
-#define SP_COL_GROUP 2
-#endif
-    const int col_group = col_tiles <= 4 ? (int)col_tiles : SP_COL_GROUP;
-    // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
-    // at the sizes this path is measured on.
-#define CUVDIA_SPMM_ARGS chunks, nchunks, vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha, \
-                         beta, (int)col_tiles, col_group, a_bytes, s_min, s_max, ep
-#define CUVDIA_SPMM_LAUNCH(L)                                                                                   \
-    case L:                                                                                                     \
-        if (nchunks <= 64 && !fused)                                                                            \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 1, false>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS); \
-        else if (nchunks <= 64)                                                                                 \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 1, true>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS);  \
-        else if (!fused)                                                                                        \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 4, false>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS); \
-        else                                                                                                    \
-            hipLaunchKernelGGL((spmm_tiled_kernel<L, 8, 4, true>), grid, dim3(512), 0, stream, CUVDIA_SPMM_ARGS);  \
-        break;
-    const bool fused = ep.bias != nullptr || ep.act != 0;
-    switch (lck) {
-        CUVDIA_SPMM_LAUNCH(1) CUVDIA_SPMM_LAUNCH(2) CUVDIA_SPMM_LAUNCH(3) CUVDIA_SPMM_LAUNCH(4)
-        CUVDIA_SPMM_LAUNCH(5) CUVDIA_SPMM_LAUNCH(6) CUVDIA_SPMM_LAUNCH(7) CUVDIA_SPMM_LAUNCH(8)
-        CUVDIA_SPMM_LAUNCH(9) CUVDIA_SPMM_LAUNCH(10) CUVDIA_SPMM_LAUNCH(11) CUVDIA_SPMM_LAUNCH(12)
-        CUVDIA_SPMM_LAUNCH(13)
-        default: return hipErrorInvalidValue;
-    }
-#undef CUVDIA_SPMM_LAUNCH
-#undef CUVDIA_SPMM_ARGS
-    return hipGetLastError();
+    const int col_group = col_tiles <= 4 ? (int)col_tiles : 2;
+    const int lck = trans ? A.max_len_t : A.max_len_n;
+    const SpLaunch L{trans ? A.chunks_t_dev : A.chunks_n_dev,
+                     trans ? A.n_chunks_t : A.n_chunks_n,
+                     vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha, beta,
+                     (int)col_tiles, col_group, (unsigned)((long long)A.nd * A.stride * 4),
+                     trans ? A.s_min_t : A.s_min_n, trans ? A.s_max_t : A.s_max_n, ep,
+                     dim3((unsigned)(row_tiles * col_tiles)), stream, lck};
+    if (lck <= 5) return spmm_tiled_launch_1_5(L);
+    if (lck <= 9) return spmm_tiled_launch_6_9(L);
+    return spmm_tiled_launch_10_13(L);
 }
 
 hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, long long lda,
@@ -1795,5 +1859,7 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
 #undef CUVDIA_DD_ARGS
     return hipGetLastError();
 }
+
+#endif  // part 4
 
 }  // namespace cuvdia
