@@ -38,7 +38,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter read for a
 # 256 MiB device copy in the same run (FETCH_SIZE 0.50 KiB per KiB copied,
 # WRITE_SIZE 1.00); commands and readings: profiles/hbm_traffic_cfg1_cfg2_cfg3.md
-MEASURED_TRAFFIC_BYTES = {"up_pass": 23_150_000, "down_pass": 31_580_000, "weight_gradient": 26_820_000}
+MEASURED_TRAFFIC_BYTES = {"up_pass": 23_170_000, "down_pass": 31_600_000, "weight_gradient": 26_820_000}
 FP32_VALU_PEAK_TFLOPS = 157.3  # published vector fp32 (packed); the kernels use no MFMA
 
 

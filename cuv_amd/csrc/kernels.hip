@@ -950,9 +950,23 @@ __device__ __forceinline__ void spmm_tile_lean(
             int p[SP_CHUNK_MAX] = {en.p0, en.p1, en.p2, en.p3, en.p4, en.p5, en.p6, en.p7, en.p8, en.p9, en.p10, en.p11, en.p12};
 #pragma unroll
             for (int k = 0; k < NP; ++k) asm("" : "+s"(p[k]));
-            int sl = p[0];
+            int sl;
+            if constexpr (LCK <= 8) {
+                // two waves fetch diagonals, four each: the wave's four candidates are chosen with scalar
+                // selects (wave is uniform), the lane's own among them with three vector selects
+                const bool up = wave != 3;
+                int q[4] = {up ? p[4] : p[0], up ? p[5] : p[1], up ? p[6] : p[2], up ? p[7] : p[3]};
 #pragma unroll
-            for (int k = 1; k < NP; ++k) sl = a_j == k ? p[k] : sl;
+                for (int k = 0; k < 4; ++k) asm("" : "+s"(q[k]));
+                const int jl = lane >> 4;
+                sl = q[0];
+#pragma unroll
+                for (int k = 1; k < 4; ++k) sl = jl == k ? q[k] : sl;
+            } else {
+                sl = p[0];
+#pragma unroll
+                for (int k = 1; k < NP; ++k) sl = a_j == k ? p[k] : sl;
+            }
             const bool ok = real & (a_j < en.len) & (sl >= 0);
             const int arow = row0 + erow + (ashift ? s0 + a_j : 0);          // first of the lane's 4 rows of its diagonal
             const unsigned voff = ok ? ((unsigned)sl * (unsigned)stride + (unsigned)arow) * 4u : OOB_OFFSET;
