@@ -19,14 +19,29 @@ def _stream_ptr():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def _check_dense(t, rows, name):
-    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.dim() == 2):
-        raise TypeError("%s must be a 2-d float32 CUDA tensor" % name)
+def _check_layout(t, rows, name):
+    """(batch, leading dimension) of a (batch, rows) tensor holding a column-major matrix; raises for layouts
+    the kernels cannot address.  Looks at shape and strides only."""
+    if t.dim() != 2:
+        raise TypeError("%s must be 2-d" % name)
     if t.stride(1) != 1:
         raise ValueError("%s must be column-major: shape (batch, rows) with unit stride along rows" % name)
     if t.shape[1] != rows:
         raise RuntimeError("%s has %d rows, expected %d" % (name, t.shape[1], rows))
-    return t.shape[0], max(t.stride(0), rows) if t.shape[0] > 1 else max(rows, 1)
+    if t.shape[0] > 1:
+        # columns closer together than their length overlap (expanded or as_strided views): the kernels
+        # would address batch*rows floats over storage that holds fewer
+        if t.stride(0) < rows:
+            raise ValueError("%s: column stride %d is smaller than its %d rows (overlapping columns)"
+                             % (name, t.stride(0), rows))
+        return t.shape[0], t.stride(0)
+    return t.shape[0], max(rows, 1)
+
+
+def _check_dense(t, rows, name):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.dim() == 2):
+        raise TypeError("%s must be a 2-d float32 CUDA tensor" % name)
+    return _check_layout(t, rows, name)
 
 
 class _dia_matrix_f:

@@ -84,6 +84,26 @@ def test_set_writes_on_band_only_and_dia_views_storage():
     assert A.get_offset(1) == 2 and A.has(0, 2)
 
 
+def test_dense_layout_rejects_overlapping_columns():
+    # an expanded (stride-0) or overlapping as_strided view would make the kernels address batch*rows floats
+    # over storage that holds fewer: for dst that is an out-of-bounds write
+    import torch
+    from cuv_amd import dia as D
+    rows = 16
+    x = torch.zeros(rows)
+    for bad in (x.expand(4, rows), torch.zeros(64).as_strided((4, rows), (8, 1))):
+        for name in ("B", "dst"):
+            with pytest.raises(ValueError, match="overlapping"):
+                D._check_layout(bad, rows, name)
+    assert D._check_layout(torch.zeros(4, rows), rows, "B") == (4, rows)
+    assert D._check_layout(torch.zeros(4, 24)[:, :rows], rows, "B") == (4, 24)       # a real leading dimension
+    assert D._check_layout(x.expand(1, rows), rows, "B") == (1, rows)                # one column: nothing to overlap
+    with pytest.raises(ValueError, match="column-major"):
+        D._check_layout(torch.zeros(rows, 4).t(), rows, "B")
+    with pytest.raises(RuntimeError, match="rows"):
+        D._check_layout(torch.zeros(4, rows + 1), rows, "B")
+
+
 def test_constructor_preconditions():
     with pytest.raises(RuntimeError, match="m_row_fact>0"):
         D.host_dia_matrix_f(4, 4, 1, 4, 0)
