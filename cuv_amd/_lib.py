@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libcuvdia.so")
 
 OK = 0
-EINVAL, ESHAPE, EHIP, ENOMEM, EUNSUPPORTED, ENODEVICE = -1, -2, -3, -4, -5, -6
+EINVAL, ESHAPE, EHIP, ENOMEM, EUNSUPPORTED, ENODEVICE, ETOOLARGE = -1, -2, -3, -4, -5, -6, -7
 ACT_NONE, ACT_SIGMOID, ACT_SIGMOID_SAMPLE = 0, 1, 2
 PATH_AUTO, PATH_GENERIC, PATH_TILED = 0, 1, 2
 
@@ -61,13 +61,15 @@ def lib():
     L.cuvdia_avg_diagonals_f32.argtypes = [c_vp, c_vp, c_vp, c_vp]
     L.cuvdia_spmm_offsets_f32.argtypes = [c_vp, ip, c_int, c_int, c_int, c_int, c_int, c_vp, c_ll,
                                           c_vp, c_ll, c_int, c_char, c_f, c_f, c_vp]
+    L.cuvdia_spmm_offsets_noalloc_f32.argtypes = L.cuvdia_spmm_offsets_f32.argtypes
     L.cuvdia_dd2dia_offsets_f32.argtypes = [c_vp, ip, c_int, c_int, c_int, c_int, c_int, c_vp, c_ll,
                                             c_vp, c_ll, c_int, c_f, c_f, c_vp]
     for name in ("cuvdia_set_path", "cuvdia_plan_chunks", "cuvdia_desc_create", "cuvdia_desc_destroy",
                  "cuvdia_desc_info", "cuvdia_spmm_f32", "cuvdia_dd2dia_f32", "cuvdia_spmm_offsets_f32",
                  "cuvdia_dd2dia_offsets_f32", "cuvdia_cache_clear", "cuvdia_spmm_bias_act_f32",
                  "cuvdia_spmm_layer_f32", "cuvdia_learn_step_weight_decay_f32", "cuvdia_avg_diagonals_f32",
-                 "cuvdia_plan_units", "cuvdia_learn_step_weight_decay_momentum_f32", "cuvdia_plan_chunks_max"):
+                 "cuvdia_plan_units", "cuvdia_learn_step_weight_decay_momentum_f32", "cuvdia_plan_chunks_max",
+                 "cuvdia_spmm_offsets_noalloc_f32"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

@@ -109,6 +109,7 @@ const char *cuvdia_strerror(int code)
         case CUVDIA_ENOMEM: return "out of memory";
         case CUVDIA_EUNSUPPORTED: return "unsupported request";
         case CUVDIA_ENODEVICE: return "no gfx950 device";
+        case CUVDIA_ETOOLARGE: return "offset table exceeds the fixed capacity of the allocation-free entry point";
         default: return "unknown cuvdia error";
     }
 }
@@ -477,6 +478,78 @@ int cuvdia_spmm_offsets_f32(const float *A_vals, const int *offsets_host, int nd
     const int rc = cached_desc(offsets_host, nd, stride, h, w, row_fact, &d);
     if (rc) return rc;
     return cuvdia_spmm_f32(d, A_vals, B, ldb, dst, ldd, batch, transA, alpha, beta, stream);
+}
+
+int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals, const int *offsets_host, int nd, int stride,
+                                    int h, int w, int row_fact, const float *B, long long ldb,
+                                    float *dst, long long ldd, int batch, char transA,
+                                    float alpha, float beta, void *stream)
+{
+    // the argument rules of cuvdia_spmm_offsets_f32 -> cuvdia_spmm_layer_f32, in the same order
+    if (!offsets_host || nd < 1) return CUVDIA_EINVAL;
+    if (const int rc = validate_shape(offsets_host, nd, h, w, stride, row_fact)) return rc;
+    if (!A_vals || batch < 0) return CUVDIA_EINVAL;
+    if (transA != 'n' && transA != 't') return CUVDIA_EINVAL;
+    if (batch == 0) return CUVDIA_OK;
+    if (!B || !dst) return CUVDIA_EINVAL;
+    const bool trans = transA == 't';
+    const int n_out = trans ? w : h, n_in = trans ? h : w;
+    if (ldb < n_in || ldd < n_out) return CUVDIA_ESHAPE;
+    if (nd > NOALLOC_MAX_DIAGONALS) return CUVDIA_ETOOLARGE;
+    if (const int rc = require_device()) return rc;
+
+    std::vector<Chunk> chunks;
+    try {
+        chunks = plan_chunks(offsets_host, nd, trans, SP_CHUNK_MAX);
+    } catch (const std::bad_alloc &) {
+        return CUVDIA_ENOMEM;
+    }
+    unsigned char *tables = nullptr;
+    hipError_t e = noalloc_scratch(&tables);
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(static table block)");
+
+    // The view a descriptor would hold, with its tables inside the static array.  Only the table of the
+    // requested traversal is described (and uploaded); the other one is left empty.
+    DiaView view{};
+    view.h = h; view.w = w; view.nd = nd; view.stride = stride; view.rf = row_fact;
+    view.offsets_dev = reinterpret_cast<const int *>(tables);
+    const Chunk *chunks_dev = reinterpret_cast<const Chunk *>(tables + NOALLOC_CHUNKS_AT);
+    int max_len = 0, s_min = chunks.front().s0, s_max = s_min;
+    for (const Chunk &c : chunks) {
+        max_len = std::max(max_len, c.len);
+        s_min = std::min(s_min, c.s0);
+        s_max = std::max(s_max, c.s0);
+    }
+    if (trans) {
+        view.chunks_t_dev = chunks_dev; view.n_chunks_t = (int)chunks.size();
+        view.max_len_t = max_len; view.s_min_t = s_min; view.s_max_t = s_max;
+    } else {
+        view.chunks_n_dev = chunks_dev; view.n_chunks_n = (int)chunks.size();
+        view.max_len_n = max_len; view.s_min_n = s_min; view.s_max_n = s_max;
+    }
+
+    // the kernel family is chosen by the rule of cuvdia_spmm_layer_f32
+    const int forced = g_path.load();
+    const bool tiled_possible = spmm_tiled_ok(view, ldb, ldd, trans);
+    bool tiled;
+    if (forced == CUVDIA_PATH_TILED) {
+        if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
+        tiled = true;
+    } else if (forced == CUVDIA_PATH_GENERIC) {
+        tiled = false;
+    } else {
+        tiled = tiled_possible && batch >= SPMM_TILED_MIN_BATCH;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // the tiled kernels read the chunk table only, the generic kernel the offset table only
+    if (tiled) e = noalloc_upload(tables + NOALLOC_CHUNKS_AT, chunks.data(), chunks.size() * sizeof(Chunk), s);
+    else e = noalloc_upload(tables, offsets_host, (size_t)nd * sizeof(int), s);
+    if (e != hipSuccess) return hip_fail(e, "table fill kernel launch");
+    const SpEpilogue ep{nullptr, CUVDIA_ACT_NONE, 0u, 0u};
+    e = tiled ? launch_spmm_tiled(view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s)
+              : launch_spmm_generic(view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s);
+    t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
+    return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "spmm kernel launch");
 }
 
 int cuvdia_dd2dia_offsets_f32(float *C_vals, const int *offsets_host, int nd, int stride,

@@ -25,6 +25,8 @@
 //           serially in ascending column order.
 #include <hip/hip_runtime.h>
 
+#include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include "kernels.hpp"
@@ -731,7 +733,11 @@ __device__ __forceinline__ void spmm_tile_edge(
 // vector-memory operations and complete in order with the wave's other loads
 // (s_waitcnt vmcnt).  Written in assembly so that the waits below can be
 // placed by hand: the loop keeps two chunks of them in flight across
-// barriers, which no automatic placement allows.
+// barriers, which no automatic placement allows.  M0 is written inside the
+// statement without appearing among its clobbers: the compiler treats M0 as a
+// reserved register (it never keeps a value there across other code, and sets
+// it immediately before each instruction of its own that reads it), and it
+// rejects reserved registers in a clobber list with a warning.
 typedef int sp_int4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ sp_int4 raw_rsrc(const void *base, unsigned bytes)
 {
@@ -1872,6 +1878,64 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
 #undef CUVDIA_DD_LAUNCH
 #undef CUVDIA_DD_ARGS
     return hipGetLastError();
+}
+
+// ------------------------------------------------- tables without allocation --
+//
+// The table block of the allocation-free entry point: the device copy of the
+// offset table and of one chunk table, which a descriptor keeps in memory it
+// allocates.  Every GPU holds its own copy of the array at its own address;
+// the name below is only the host-side handle that hipGetSymbolAddress turns
+// into that address, once per device.
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+static_assert(NOALLOC_MAX_CHUNKS >= SP_MAX_CHUNKS, "every table the tiled product accepts fits the static array");
+
+// One launch carries up to NOALLOC_PIECE_BYTES of table in its kernel
+// arguments (copied by the runtime when the launch is enqueued or captured,
+// so the host buffer may go away at once and nothing is staged or allocated).
+struct NoallocPiece {
+    unsigned w[NOALLOC_PIECE_BYTES / 4];
+};
+__global__ __launch_bounds__(256) void noalloc_fill_kernel(NoallocPiece piece, unsigned *dst, int nwords)
+{
+    for (int i = threadIdx.x; i < nwords; i += 256) dst[i] = piece.w[i];
+}
+
+hipError_t noalloc_scratch(unsigned char **out)
+{
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mutex;
+    static unsigned char *ptrs[MAX_DEVICES] = {};
+    *out = nullptr;
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    if (device < 0 || device >= MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!ptrs[device]) {
+        unsigned char *p = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        ptrs[device] = p;
+    }
+    *out = ptrs[device];
+    return hipSuccess;
+}
+
+hipError_t noalloc_upload(unsigned char *dst_dev, const void *src_host, size_t bytes, hipStream_t stream)
+{
+    const unsigned char *src = static_cast<const unsigned char *>(src_host);
+    for (size_t at = 0; at < bytes; at += NOALLOC_PIECE_BYTES) {
+        const size_t n = bytes - at < NOALLOC_PIECE_BYTES ? bytes - at : NOALLOC_PIECE_BYTES;
+        NoallocPiece piece{};
+        std::memcpy(piece.w, src + at, n);
+        hipLaunchKernelGGL(noalloc_fill_kernel, dim3(1), dim3(256), 0, stream, piece,
+                           reinterpret_cast<unsigned *>(dst_dev + at), (int)((n + 3) / 4));
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 #endif  // part 4

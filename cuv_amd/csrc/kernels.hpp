@@ -4,6 +4,8 @@
 #pragma once
 #include <hip/hip_runtime_api.h>
 
+#include <cstddef>
+
 #include "plan.hpp"
 
 namespace cuvdia {
@@ -78,6 +80,22 @@ bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch);
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream);
+
+// The allocation-free entry point keeps its device tables in a static device
+// array instead of a descriptor's allocation: the offset table at byte 0 (up
+// to NOALLOC_MAX_DIAGONALS ints), one chunk table at NOALLOC_CHUNKS_AT (up to
+// NOALLOC_MAX_CHUNKS entries of 64 bytes).
+constexpr int NOALLOC_MAX_DIAGONALS = 1024;
+constexpr int NOALLOC_MAX_CHUNKS = 256;
+constexpr size_t NOALLOC_CHUNKS_AT = (size_t)NOALLOC_MAX_DIAGONALS * sizeof(int);
+constexpr size_t NOALLOC_SCRATCH_BYTES = NOALLOC_CHUNKS_AT + (size_t)NOALLOC_MAX_CHUNKS * sizeof(Chunk);
+constexpr size_t NOALLOC_PIECE_BYTES = 3584;     // table bytes one fill launch carries in its kernel arguments
+// Address of that array on the current device (looked up once per device).
+hipError_t noalloc_scratch(unsigned char **out);
+// Enqueues the copy of `bytes` (a multiple of 4) host bytes to dst_dev, a place
+// inside the array, on `stream`: the bytes travel as kernel arguments, so no
+// staging buffer is allocated and src_host may be reused on return.
+hipError_t noalloc_upload(unsigned char *dst_dev, const void *src_host, size_t bytes, hipStream_t stream);
 
 // dst[d] = mean of diagonal d over its valid slots (row_fact == 1), dst on the device.
 hipError_t launch_avg_diagonals(const DiaView &A, const float *vals, float *dst, hipStream_t stream);

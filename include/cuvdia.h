@@ -24,7 +24,8 @@
  *     "results visible on return" behaviour (spmv.cu:99,
  *     densedense_to_sparse.cu:295);
  *   - no entry point allocates device memory except cuvdia_desc_create and
- *     the first use of a new offset table by the *_offsets_* forms;
+ *     the first use of a new offset table by the *_offsets_* forms
+ *     (cuvdia_spmm_offsets_noalloc_f32 never does);
  *   - a descriptor belongs to the device that was current when it was
  *     created; a compute call made while another device is current returns
  *     CUVDIA_EINVAL.  The *_offsets_* forms keep one descriptor per device.
@@ -43,6 +44,7 @@ extern "C" {
 #define CUVDIA_ENOMEM       -4  /* host or device allocation failed               */
 #define CUVDIA_EUNSUPPORTED -5  /* valid request this build has no kernel for     */
 #define CUVDIA_ENODEVICE    -6  /* no gfx950 device visible                       */
+#define CUVDIA_ETOOLARGE    -7  /* beyond the fixed capacity of cuvdia_spmm_offsets_noalloc_f32 */
 
 /* Kernel families, for cuvdia_set_path / cuvdia_last_path. */
 #define CUVDIA_PATH_AUTO     0  /* pick by shape (default)                        */
@@ -205,7 +207,9 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals_device,
  * declared in src/cuv/matrix_ops/diagonals.hpp:12) with the semantics of the
  * host version (diagonals.cu:24-51: the mean over the N_d = min(h - max(0,-k),
  * w - max(0,k)) valid slots, padding never read; the reference's device
- * version averages over the padded stride instead).  row_fact must be 1
+ * version averages over the padded stride instead, so ITS NUMBERS DIFFER
+ * from this entry's for every off-centre diagonal: sum/stride there,
+ * sum/N_d here).  row_fact must be 1
  * (diagonals.cu:28), else CUVDIA_EUNSUPPORTED; a diagonal without valid slots
  * yields 0. */
 int cuvdia_avg_diagonals_f32(const cuvdia_desc *desc, const float *A_vals_device,
@@ -227,6 +231,29 @@ int cuvdia_dd2dia_offsets_f32(float *C_vals_device, const int *offsets_host,
                               const float *A_device, long long lda,
                               const float *B_device, long long ldb, int batch,
                               float alpha, float beta, void *stream);
+
+/* cuvdia_spmm_offsets_f32 for callers that cannot allocate device memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  Same arguments, same
+ * argument rules, same kernels and bit-identical results; but the device copy
+ * of the offset table and of the chunk table the kernels walk -- which a
+ * descriptor keeps in memory it allocates -- lives in a static device array
+ * of 20480 bytes inside the library (one copy per GPU, held until the process
+ * ends), so the call performs no hipMalloc, no hipFree and no allocating
+ * library call, and touches neither the descriptor cache nor its lock.  Every
+ * call rewrites the part of the array it uses with one small fill kernel per
+ * 3584 bytes of table, enqueued on `stream` ahead of the product (the bytes
+ * travel as kernel arguments, so the host table may be reused on return).
+ * Capacity: nd <= 1024, else CUVDIA_ETOOLARGE (nothing is enqueued); a table
+ * of more than 256 chunks is served by the generic kernels, as everywhere.
+ * All calls on one GPU share that GPU's array: calls ordered on one stream
+ * are safe, calls that may overlap (different streams or host threads without
+ * ordering between them) race on it. */
+int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals_device, const int *offsets_host,
+                                    int nd, int stride, int h, int w, int row_fact,
+                                    const float *B_device, long long ldb,
+                                    float *dst_device, long long ldd, int batch,
+                                    char transA, float alpha, float beta, void *stream);
 
 /* Drops every descriptor held by the *_offsets_* cache. */
 int cuvdia_cache_clear(void);
