@@ -451,14 +451,127 @@ __device__ __forceinline__ void spmm_rows(float (&acc)[T], const SpWindow<LCK, T
     }
 }
 
-// the diagonals J .. J1 - 1 of a chunk
+// The FMAs of N consecutive diagonals J0 .. J0+N-1 of a chunk for a wave of 8 rows, as ONE statement:
+// acc[t] += bcast_t(a[j]) * win[j + t].  A DPP operand must not have been written by a VALU instruction in the
+// two preceding issue slots; inside the statement no FMA writes another's DPP operand (the a[j] come from LDS
+// reads), so one leading s_nop -- for whatever the compiler placed before the statement -- serves all 8*N.
+template <int J0, int N, int NA, int NW>
+__device__ __forceinline__ void fma_diagonals8(float (&acc)[8], const float (&a)[NA], const float (&win)[NW])
+{
+    static_assert(N >= 1 && N <= 4 && J0 + N <= NA && J0 + N + 7 <= NW, "one statement takes at most 30 operands");
+    if constexpr (N == 1) {
+        asm("s_nop 1\n\t"
+            "v_fmac_f32_dpp %0, %8, %9 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %8, %10 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %8, %11 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %8, %12 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %8, %13 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %8, %14 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %8, %15 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %8, %16 row_newbcast:7 row_mask:0xf bank_mask:0xf"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(a[J0 + 0]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]));
+    }     else if constexpr (N == 2) {
+        asm("s_nop 1\n\t"
+            "v_fmac_f32_dpp %0, %8, %10 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %8, %11 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %8, %12 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %8, %13 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %8, %14 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %8, %15 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %8, %16 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %8, %17 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %9, %11 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %9, %12 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %9, %13 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %9, %14 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %9, %15 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %9, %16 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %9, %17 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %9, %18 row_newbcast:7 row_mask:0xf bank_mask:0xf"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]), "v"(win[J0 + 8]));
+    }     else if constexpr (N == 3) {
+        asm("s_nop 1\n\t"
+            "v_fmac_f32_dpp %0, %8, %11 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %8, %12 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %8, %13 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %8, %14 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %8, %15 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %8, %16 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %8, %17 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %8, %18 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %9, %12 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %9, %13 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %9, %14 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %9, %15 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %9, %16 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %9, %17 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %9, %18 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %9, %19 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %10, %13 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %10, %14 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %10, %15 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %10, %16 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %10, %17 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %10, %18 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %10, %19 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %10, %20 row_newbcast:7 row_mask:0xf bank_mask:0xf"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(a[J0 + 2]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]), "v"(win[J0 + 8]), "v"(win[J0 + 9]));
+    }     else if constexpr (N == 4) {
+        asm("s_nop 1\n\t"
+            "v_fmac_f32_dpp %0, %8, %12 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %8, %13 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %8, %14 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %8, %15 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %8, %16 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %8, %17 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %8, %18 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %8, %19 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %9, %13 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %9, %14 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %9, %15 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %9, %16 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %9, %17 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %9, %18 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %9, %19 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %9, %20 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %10, %14 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %10, %15 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %10, %16 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %10, %17 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %10, %18 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %10, %19 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %10, %20 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %10, %21 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %11, %15 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %1, %11, %16 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %2, %11, %17 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %3, %11, %18 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %4, %11, %19 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %5, %11, %20 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %6, %11, %21 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %7, %11, %22 row_newbcast:7 row_mask:0xf bank_mask:0xf"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(a[J0 + 2]), "v"(a[J0 + 3]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]), "v"(win[J0 + 8]), "v"(win[J0 + 9]), "v"(win[J0 + 10]));
+    }
+}
+
+// the diagonals J .. J1 - 1 of a chunk (waves of 8 rows take them four to a statement)
 template <int LCK, int T, int J, int J1>
 __device__ __forceinline__ void spmm_rows_range(float (&acc)[T], const SpWindow<LCK, T> &win)
 {
     if constexpr (J < J1) {
-        fma_block8<J, 0>(acc, win.a[J], win.w);
-        if constexpr (T == 16) fma_block8<J, 8>(acc, win.a[J], win.w);
-        spmm_rows_range<LCK, T, J + 1, J1>(acc, win);
+        if constexpr (T == 8) {
+            constexpr int N = J1 - J < 4 ? J1 - J : 4;
+            fma_diagonals8<J, N>(acc, win.a, win.w);
+            spmm_rows_range<LCK, T, J + N, J1>(acc, win);
+        } else {
+            fma_block8<J, 0>(acc, win.a[J], win.w);
+            fma_block8<J, 8>(acc, win.a[J], win.w);
+            spmm_rows_range<LCK, T, J + 1, J1>(acc, win);
+        }
     }
 }
 
