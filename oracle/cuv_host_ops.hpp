@@ -1,10 +1,13 @@
-// host_memory_space twins of the DIA operations, for tests only.
+// host_memory_space operations backed by the C oracle, for tests only.
 //
-// TEST INFRASTRUCTURE: these overloads give C++ tests the reference's
+// TEST INFRASTRUCTURE: these functions give C++ tests the reference's
 // "run the host path and the device path on the same inputs" pattern
 // (src/tests/spmv.cpp:103-143, src/tests/densedense_to_dia.cpp:166-197).  They
 // forward to the C oracle (dia_oracle.h), which restates the reference's host
-// loops; the product headers under cuv_amd/include never include this file.
+// loops, and live in namespace cuv_oracle so that a test says which side of a
+// comparison is the checker: cuv_oracle::prod is the oracle, cuv::prod on host
+// operands is the product's own host twin (cuv/matrix_ops/host_ops.hpp).  The
+// product headers under cuv_amd/include never include this file.
 #ifndef CUV_HOST_OPS_ORACLE_HPP
 #define CUV_HOST_OPS_ORACLE_HPP
 
@@ -14,7 +17,8 @@
 
 #include "dia_oracle.h"
 
-namespace cuv {
+namespace cuv_oracle {
+using namespace cuv;
 
 // src/cuv/matrix_ops/spmv.cu:145-200 (asserts :159-160, :180-181)
 inline void spmv(tensor<float, host_memory_space> &dst, const dia_matrix<float, host_memory_space> &A,
@@ -162,5 +166,5 @@ inline void prod(tensor<float, host_memory_space, column_major> &dst,
         }
 }
 
-}  // namespace cuv
+}  // namespace cuv_oracle
 #endif

@@ -35,7 +35,7 @@ TEST_CASE(spmv_dev_correctness_trans)
     convert(C2, f.C);
     tensor<float, dev_memory_space, column_major> B2(f.B.shape());
     convert(B2, f.B);
-    prod(f.B, f.A, f.C, 't', 'n');
+    cuv_oracle::prod(f.B, f.A, f.C, 't', 'n');
     prod(B2, A2, C2, 't', 'n');
     MAT_CMP(f.B, B2, 0.1f);
 }
@@ -50,7 +50,7 @@ TEST_CASE(spmv_dev_correctness)
     tensor<float, dev_memory_space, column_major> B2(f.B.shape());
     convert(B2, f.B);
     const float factAv = 2.f, factC = 1.3f;
-    prod(f.C, f.A, f.B, 'n', 'n', factAv, factC);
+    cuv_oracle::prod(f.C, f.A, f.B, 'n', 'n', factAv, factC);
     prod(C2, A2, B2, 'n', 'n', factAv, factC);
     MAT_CMP(f.C, C2, 0.1f);
 }
@@ -70,7 +70,7 @@ TEST_CASE(spmv_dev_flat_vectors)
     for (int c = 0; c < k; c++) {
         tensor<float, host_memory_space> xv(indices[index_range(0, m)], xh.ptr() + c * m);
         tensor<float, host_memory_space> yv(indices[index_range(0, n)], yh.ptr() + c * n);
-        spmv(yv, f.A, xv, 'n', 1.f, 0.f);
+        cuv_oracle::spmv(yv, f.A, xv, 'n', 1.f, 0.f);
     }
     for (int i = 0; i < n * k; i++) CHECK((float)yd[i] == (float)yh[i]);
 }
@@ -97,7 +97,7 @@ TEST_CASE(dd2s_correctness_dev)
     tensor<float, host_memory_space, column_major> Ah(f.A.shape()), Bh(f.B.shape()), dense(DdFix::n, DdFix::m);
     convert(Ah, f.A); convert(Bh, f.B);
     fill(dense, 0);
-    prod(dense, Ah, Bh, 'n', 't');
+    cuv_oracle::prod(dense, Ah, Bh, 'n', 't');
     int seen = 0;
     for (int i = 0; i < DdFix::n; i++)
         for (int j = 0; j < DdFix::m; j++)
@@ -117,11 +117,11 @@ TEST_CASE(dd2s_cmp_dev_host)
     dev_block_descriptor<float> bd(f.C);
     host_block_descriptor<float> bdh(C2);
     densedense_to_dia(f.C, bd, f.A, f.B);
-    densedense_to_dia(C2, bdh, A2, B2);
+    cuv_oracle::densedense_to_dia(C2, bdh, A2, B2);
     MAT_CMP(f.C, C2, 0.01f);
     // documented factors, and the descriptor-free overload
     densedense_to_dia(f.C, f.A, f.B, 0.5f, 0.25f);
-    densedense_to_dia(C2, bdh, A2, B2, 0.5f, 0.25f);
+    cuv_oracle::densedense_to_dia(C2, bdh, A2, B2, 0.5f, 0.25f);
     MAT_CMP(f.C, C2, 0.01f);
 }
 
@@ -139,7 +139,7 @@ TEST_CASE(avg_diagonals_dev)
     tensor<float, dev_memory_space> avg(7);
     tensor<float, host_memory_space> avg_h(7), avg_ref(7);
     avg_diagonals(avg, wd);
-    avg_diagonals(avg_ref, w);
+    cuv_oracle::avg_diagonals(avg_ref, w);
     convert(avg_h, avg);
     for (int d = 0; d < 7; ++d) {
         const int k = off[d], i0 = std::max(0, -k), j0 = std::max(0, k);
@@ -171,7 +171,7 @@ TEST_CASE(learn_step_weight_decay_dev)
     convert(wd, w);
     convert(dwd, dw);
     learn_step_weight_decay(wd.vec(), dwd.vec(), 0.5f, 0.25f);
-    learn_step_weight_decay(w.vec(), dw.vec(), 0.5f, 0.25f);
+    cuv_oracle::learn_step_weight_decay(w.vec(), dw.vec(), 0.5f, 0.25f);
     dia_matrix<float, host_memory_space> back(32, 16, 7, 32, 1);
     convert(back, wd);
     for (unsigned i = 0; i < w.vec().size(); ++i) {
@@ -198,7 +198,7 @@ TEST_CASE(learn_step_weight_decay_momentum_dev)
     convert(md, m);
     convert(dwd, dw);
     learn_step_weight_decay_momentum(wd, md, dwd, 0.5f, 0.5f, 0.25f);
-    learn_step_weight_decay_momentum(w, m, dw, 0.5f, 0.5f, 0.25f);
+    cuv_oracle::learn_step_weight_decay_momentum(w, m, dw, 0.5f, 0.5f, 0.25f);
     tensor<float, host_memory_space> wb(n), mb(n);
     convert(wb, wd);
     convert(mb, md);
@@ -280,14 +280,14 @@ TEST_CASE(locally_connected_layer)
     tensor<float, dev_memory_space, column_major> Vd(V.shape()), Hd(H.shape()), outd(N, batch);
     convert(Vd, V); convert(Hd, H);
     prod(outd, Wd, Vd, 'n', 'n');
-    prod(Hh, *W, V, 'n', 'n');
+    cuv_oracle::prod(Hh, *W, V, 'n', 'n');
     MAT_CMP(Hh, outd, 0.01f);
     prod(outd, Wd, Hd, 't', 'n');
-    prod(Vh, *W, H, 't', 'n');
+    cuv_oracle::prod(Vh, *W, H, 't', 'n');
     MAT_CMP(Vh, outd, 0.01f);
     densedense_to_dia(Wd, Hd, Vd, 1.f / batch, 0.9f);
     host_block_descriptor<float> bdh(*W);
-    densedense_to_dia(*W, bdh, H, V, 1.f / batch, 0.9f);
+    cuv_oracle::densedense_to_dia(*W, bdh, H, V, 1.f / batch, 0.9f);
     MAT_CMP(*W, Wd, 0.01f);
     delete W;
 }

@@ -1,6 +1,7 @@
 // CPU-only checks of the C++ mirror: containers, conversions, error behaviour
-// and the host twins of the operations against the reference fixtures' closed
-// forms.  Runs without a GPU.
+// and the product's host twins of the operations (cuv/matrix_ops/host_ops.hpp)
+// against the reference fixtures' closed forms and, element for element,
+// against the oracle (namespace cuv_oracle).  Runs without a GPU.
 //
 // Re-expresses the host-side cases of the reference's tests:
 //   src/tests/dia_mat.cpp:111-119 (dia -> dense), src/tests/convert.cpp:110-129,
@@ -96,7 +97,7 @@ TEST_CASE(spmv_host_correctness)
 {
     SpmvFix f;
     prod(f.C, f.A, f.B, 'n', 'n', 2.f, 1.3f);
-    prod(f.C_, f.A_, f.B, 'n', 'n', 2.f, 1.3f);
+    cuv_oracle::prod(f.C_, f.A_, f.B, 'n', 'n', 2.f, 1.3f);
     MAT_CMP(f.C, f.C_, 0.1f);
 }
 
@@ -104,7 +105,7 @@ TEST_CASE(spmv_host_correctness_trans)
 {
     SpmvFix f;
     prod(f.B, f.A, f.C, 't', 'n', 2.f, 1.3f);
-    prod(f.B_, f.A_, f.C, 't', 'n', 2.f, 1.3f);
+    cuv_oracle::prod(f.B_, f.A_, f.C, 't', 'n', 2.f, 1.3f);
     MAT_CMP(f.B, f.B_, 0.5f);
 }
 
@@ -138,7 +139,7 @@ TEST_CASE(dd2s_correctness_host)
     host_block_descriptor<float> bdh(C);
     densedense_to_dia(C, bdh, A, B);
     fill(dense, 0);
-    prod(dense, A, B, 'n', 't');
+    cuv_oracle::prod(dense, A, B, 'n', 't');
     int seen = 0;
     for (int i = 0; i < n; i++)
         for (int j = 0; j < m; j++)
@@ -151,8 +152,62 @@ TEST_CASE(dd2s_correctness_host)
     dia_matrix<float, host_memory_space> C2(n, m, 7, 36, rf);
     C2.set_offsets(off);
     fill(C2.vec(), 0);
-    densedense_to_dia_literal(C2, A, B);
+    cuv_oracle::densedense_to_dia_literal(C2, A, B);
     MAT_CMP(C, C2, 0.0001f);
+}
+
+// The product's host twins against the oracle on the same pseudo-random operands: both restate the
+// reference's host loops in the reference's element order, so every element must agree exactly -- for
+// steep matrices, both transposes, factors that are not the defaults, unsorted and out-of-range offsets.
+TEST_CASE(host_twins_equal_the_oracle)
+{
+    unsigned state = 12345u;
+    auto rnd = [&]() { state = state * 1664525u + 1013904223u; return (float)((state >> 8) & 0xffff) / 32768.f - 1.f; };
+    const int shapes[4][3] = {{40, 40, 1}, {36, 19, 4}, {24, 50, 2}, {130, 64, 1}};
+    for (const auto &sh : shapes) {
+        const int h = sh[0], w = sh[1], rf = sh[2], batch = 5;
+        std::vector<int> off;
+        const int cand[9] = {3, -2, 0, 1, -7, w - 1, -(h / rf) + 1, w + 5, -h - 3};
+        for (int o : cand) off.push_back(o);
+        dia_matrix<float, host_memory_space> A(h, w, (int)off.size(), std::max(h, w), rf), C1(h, w, (int)off.size(), std::max(h, w), rf),
+            C2(h, w, (int)off.size(), std::max(h, w), rf);
+        A.set_offsets(off); C1.set_offsets(off); C2.set_offsets(off);
+        for (unsigned i = 0; i < A.vec().size(); i++) { A.vec()[i] = rnd(); C1.vec()[i] = C2.vec()[i] = rnd(); }
+        for (int t = 0; t < 2; t++) {
+            const char trans = t ? 't' : 'n';
+            const int n_in = t ? h : w, n_out = t ? w : h;
+            tensor<float, host_memory_space, column_major> B(n_in, batch), D1(n_out, batch), D2(n_out, batch);
+            for (int i = 0; i < n_in * batch; i++) B[i] = rnd();
+            for (int i = 0; i < n_out * batch; i++) D1[i] = D2[i] = rnd();
+            prod(D1, A, B, trans, 'n', 0.75f, -1.5f);
+            cuv_oracle::prod(D2, A, B, trans, 'n', 0.75f, -1.5f);
+            for (int i = 0; i < n_out * batch; i++) CHECK((float)D1[i] == (float)D2[i]);
+            prod(D1, A, B, trans);                                   // factC == 0 overwrites
+            cuv_oracle::prod(D2, A, B, trans);
+            for (int i = 0; i < n_out * batch; i++) CHECK((float)D1[i] == (float)D2[i]);
+            tensor<float, host_memory_space> x(indices[index_range(0, n_in)], B.ptr()), y1(n_out), y2(n_out);
+            spmv(y1, A, x, trans, 2.f, 0.f);
+            cuv_oracle::spmv(y2, A, x, trans, 2.f, 0.f);
+            for (int i = 0; i < n_out; i++) CHECK((float)y1[i] == (float)y2[i]);
+        }
+        tensor<float, host_memory_space, column_major> P(h, batch), Q(w, batch);
+        for (int i = 0; i < h * batch; i++) P[i] = rnd();
+        for (int i = 0; i < w * batch; i++) Q[i] = rnd();
+        host_block_descriptor<float> bd(C1);
+        densedense_to_dia(C1, bd, P, Q, 0.25f, 0.9f);
+        cuv_oracle::densedense_to_dia(C2, bd, P, Q, 0.25f, 0.9f);
+        for (unsigned i = 0; i < C1.vec().size(); i++) CHECK((float)C1.vec()[i] == (float)C2.vec()[i]);
+        if (rf == 1) {
+            tensor<float, host_memory_space> m1((int)off.size()), m2((int)off.size());
+            avg_diagonals(m1, A);
+            cuv_oracle::avg_diagonals(m2, A);
+            for (size_t d = 0; d < off.size(); d++) {
+                const long long k = off[d], cnt = std::min<long long>(h - std::max(0LL, -k), w - std::max(0LL, k));
+                if (cnt > 0) CHECK((float)m1[d] == (float)m2[d]);
+                else CHECK((float)m1[d] == 0.f);
+            }
+        }
+    }
 }
 
 TEST_CASE(host_preconditions_throw)

@@ -164,7 +164,7 @@ def test_leading_dimensions_and_views(oracle, gu):
     B = np.asfortranarray(rng.uniform(-1, 1, (w, batch)).astype(np.float32))
     Ad = gu.make_dev_dia(A)
     ldb, ldd = w + 12, h + 20
-    Bbig = torch.zeros(batch, ldb, device="cuda:0")
+    Bbig = torch.full((batch, ldb), float("nan"), device="cuda:0")      # the gap between columns must never be used
     Bbig[:, :w] = D.to_device_colmajor(B)
     Dbig = torch.full((batch, ldd), -7.0, device="cuda:0")
     for path in _paths(1):
@@ -176,6 +176,77 @@ def test_leading_dimensions_and_views(oracle, gu):
         got = D.to_host_colmajor(Dbig[:, :h])
         gu.assert_close_mag(got, oracle.prod(A, B), oracle.prod_mag(A, B), "ld view")
         assert torch.all(Dbig[:, h:] == -7.0)          # nothing past the rows was touched
+
+
+@pytest.mark.parametrize("offs", [
+    [dy * 128 + dx for dy in range(-1, 2) for dx in range(-3, 4)],      # chunk pairs
+    list(range(-8, -1)) + list(range(0, 8)) + [100, 101],               # single chunks
+    [dy * 96 + dx for dy in range(-1, 2) for dx in range(-6, 7)],       # long chunks (13)
+])
+def test_dd2dia_nan_in_the_gaps_around_the_operands(oracle, gu, offs):
+    """The projection stages bands of B that run past a column's ends into the neighbouring column -- or, for
+    the first and last batch column of the tiles at both ends of B, past the allocation.  With lda > h and
+    ldb > w and NaN in every gap (and before the first, behind the last column) no stored element may see one."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    rng = np.random.default_rng(77)
+    h = w = 1024                                                         # four row tiles of 256
+    batch = 40
+    C = _rand_dia(oracle, rng, h, w, offs)
+    P = np.asfortranarray(rng.uniform(-1, 1, (h, batch)).astype(np.float32))
+    Q = np.asfortranarray(rng.uniform(-1, 1, (w, batch)).astype(np.float32))
+    ref = oracle.dd2dia(C, P, Q, 0.25, 0.9)
+    mag = oracle.dd2dia_f64(oracle.Dia(h, w, offs, C.stride, 1, np.abs(np.nan_to_num(C.vals))),
+                            np.abs(P), np.abs(Q), 0.25, 0.9)
+    valid = oracle.valid_mask(C)
+
+    def gapped(host, ld, lead):
+        rows, cols = host.shape
+        flat = torch.full((lead + cols * ld + 16,), float("nan"), device="cuda:0")
+        v = flat[lead:lead + cols * ld].view(cols, ld)[:, :rows]
+        v.copy_(torch.from_numpy(np.ascontiguousarray(host.T)))
+        return flat, v
+    for path in _paths(1):
+        for lead in (0, 4, 3):                      # 16-byte aligned bases and a misaligned one
+            Cd = gu.make_dev_dia(C)
+            _, Pv = gapped(P, h + 8, lead)
+            _, Qv = gapped(Q, w + 12, lead)
+            _lib.lib().cuvdia_set_path(path)
+            try:
+                D.densedense_to_dia(Cd, None, Pv, Qv, 0.25, 0.9)
+            finally:
+                _lib.lib().cuvdia_set_path(_lib.PATH_AUTO)
+            got = Cd.pull()
+            assert np.isfinite(got[valid]).all(), "a NaN from a gap reached a stored element (path %d, lead %d)" % (path, lead)
+            gu.assert_close_mag(got[valid], ref[valid], mag[valid], "gapped operands, path %d, lead %d" % (path, lead))
+            assert np.array_equal(got[~valid].view(np.uint32), C.vals[~valid].view(np.uint32))
+
+
+def test_inf_in_the_dense_operand_reaches_only_the_rows_that_use_it(oracle, gu):
+    """One Inf in B: with a table whose chunks all have the table's longest length -- every 2-d window pattern --
+    the tiled kernels multiply exactly the elements the matrix stores, so the Inf shows up in the result rows
+    that reference its row and nowhere else, as in the generic kernels and the reference's host loop.  (A
+    table that mixes chunk lengths pads the shorter chunks with zero-valued diagonals in the tiled kernels;
+    0 * Inf then yields NaN in neighbouring rows: documented in include/cuvdia.h.)"""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(5)
+    h = w = 1024
+    offs = [dy * 32 + dx for dy in range(-2, 3) for dx in range(-2, 3)]
+    A = _rand_dia(oracle, rng, h, w, offs)
+    B = np.asfortranarray(rng.uniform(-1, 1, (w, 70)).astype(np.float32))
+    B[500, 3] = np.inf
+    for trans in ("n", "t"):
+        ref = oracle.prod(A, B, None, trans)
+        outs = {}
+        for path in _paths(1):
+            got, ran = gu.gpu_prod(A, B, None, trans, 1.0, 0.0, path)
+            assert ran == path
+            outs[path] = got
+            assert np.array_equal(np.isfinite(got), np.isfinite(ref)), "path %d, %s" % (path, trans)
+        fin = np.isfinite(ref)
+        assert (~fin).sum() == len(offs)                 # the rows that use B[500, 3], in column 3 only
+        a, b = outs[_lib.PATH_GENERIC], outs[_lib.PATH_TILED]
+        np.testing.assert_allclose(a[fin], b[fin], rtol=1e-4, atol=1e-5)
 
 
 def test_batch_zero_and_errors(oracle, gu):

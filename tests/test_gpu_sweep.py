@@ -2,8 +2,11 @@
 oracle on shapes nobody picked by hand -- ragged sizes, shuffled, duplicate and
 out-of-range offsets, steep matrices (row factor 2-4), operands that are misaligned views of wider allocations
 (any leading dimension, base address not a multiple of 16 bytes), beta == 0 over
-NaN destinations.  Tolerance as in test_gpu_parity (1e-5 of the summed
-magnitudes); bytes around the destination view must stay as they were.
+NaN destinations.  The allocations around the INPUT views hold NaN, so a kernel
+that lets a byte of the gap between columns (or before the first, after the
+last column) reach a stored result fails.  Tolerance as in test_gpu_parity
+(1e-5 of the summed magnitudes); bytes around the destination view must stay
+as they were.
 """
 import numpy as np
 import pytest
@@ -26,7 +29,7 @@ def _offsets(rng, h, w):
     return offs[:60]
 
 
-def _view(torch, rng, host, fill=0.0):
+def _view(torch, rng, host, fill=float("nan")):
     """(rows, batch) host matrix -> (flat allocation, (batch, rows) view of it with a random leading dimension
     and a base shifted by 0-3 floats, mask of the view's elements in the allocation)"""
     rows, batch = host.shape
