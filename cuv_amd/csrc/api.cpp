@@ -118,7 +118,8 @@ const char *cuvdia_last_hip_error(void) { return t_hip_error.c_str(); }
 
 int cuvdia_set_path(int path)
 {
-    if (path != CUVDIA_PATH_AUTO && path != CUVDIA_PATH_GENERIC && path != CUVDIA_PATH_TILED)
+    if (path != CUVDIA_PATH_AUTO && path != CUVDIA_PATH_GENERIC && path != CUVDIA_PATH_TILED &&
+        path != CUVDIA_PATH_TILED_NOWALK && path != CUVDIA_PATH_WALK)
         return CUVDIA_EINVAL;
     g_path.store(path);
     return CUVDIA_OK;
@@ -210,19 +211,39 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     d->dev_block = nullptr;
     if ((e = hipGetDevice(&d->device)) != hipSuccess) { delete d; return hip_fail(e, "hipGetDevice"); }
 
+    // window-table forms of the products' tables (for the walking kernel)
+    WalkPlan wn, wt;
+    try {
+        plan_walk(cn, stride, false, wn);
+        plan_walk(ct, stride, true, wt);
+    } catch (const std::bad_alloc &) {
+        delete d;
+        return CUVDIA_ENOMEM;
+    }
+    auto walk_ints = [](const WalkPlan &p) { return p.ok ? p.group_rows.size() + p.aoff4.size() : (size_t)0; };
     // one device block: offsets (padded to 64 B) | chunks_n | chunks_t | projection chunks | units | one unit per chunk
+    // | window tables
     const size_t off_bytes = ((size_t)nd * sizeof(int) + 63) / 64 * 64;
     const size_t cn_bytes = cn.size() * sizeof(Chunk), ct_bytes = ct.size() * sizeof(Chunk);
     const size_t cp_bytes = cp.size() * sizeof(Chunk);
     const size_t un_bytes = un.size() * sizeof(Unit), us_bytes = us.size() * sizeof(Unit);
     const size_t cp_at = off_bytes + cn_bytes + ct_bytes, un_at = cp_at + cp_bytes, us_at = un_at + un_bytes;
-    std::vector<unsigned char> staging(us_at + us_bytes, 0);
+    const size_t wn_at = (us_at + us_bytes + 63) / 64 * 64, wn_bytes = walk_ints(wn) * sizeof(int);
+    const size_t wt_at = (wn_at + wn_bytes + 63) / 64 * 64, wt_bytes = walk_ints(wt) * sizeof(int);
+    std::vector<unsigned char> staging(wt_at + wt_bytes + 64, 0);
     std::memcpy(staging.data(), offsets_host, (size_t)nd * sizeof(int));
     std::memcpy(staging.data() + off_bytes, cn.data(), cn_bytes);
     std::memcpy(staging.data() + off_bytes + cn_bytes, ct.data(), ct_bytes);
     std::memcpy(staging.data() + cp_at, cp.data(), cp_bytes);
     std::memcpy(staging.data() + un_at, un.data(), un_bytes);
     std::memcpy(staging.data() + us_at, us.data(), us_bytes);
+    auto put_walk = [&](const WalkPlan &p, size_t at) {
+        if (!p.ok) return;
+        std::memcpy(staging.data() + at, p.group_rows.data(), p.group_rows.size() * sizeof(int));
+        std::memcpy(staging.data() + at + p.group_rows.size() * sizeof(int), p.aoff4.data(), p.aoff4.size() * sizeof(int));
+    };
+    put_walk(wn, wn_at);
+    put_walk(wt, wt_at);
     if ((e = hipMalloc(&d->dev_block, staging.size())) != hipSuccess) {
         delete d;
         return e == hipErrorOutOfMemory ? CUVDIA_ENOMEM : hip_fail(e, "hipMalloc(descriptor)");
@@ -233,14 +254,24 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
         return hip_fail(e, "hipMemcpy(descriptor)");
     }
     unsigned char *base = static_cast<unsigned char *>(d->dev_block);
-    d->view = DiaView{h, w, nd, stride, row_fact,
-                      reinterpret_cast<const int *>(base),
-                      reinterpret_cast<const Chunk *>(base + off_bytes), d->n_chunks_n,
-                      reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes), d->n_chunks_t,
-                      0, 0, 0, 0, 0, 0,
-                      reinterpret_cast<const Chunk *>(base + cp_at), (int)cp.size(), 0,
-                      reinterpret_cast<const Unit *>(base + un_at), (int)un.size(),
-                      reinterpret_cast<const Unit *>(base + us_at)};
+    d->view = DiaView{};
+    d->view.h = h; d->view.w = w; d->view.nd = nd; d->view.stride = stride; d->view.rf = row_fact;
+    d->view.offsets_dev = reinterpret_cast<const int *>(base);
+    d->view.chunks_n_dev = reinterpret_cast<const Chunk *>(base + off_bytes);
+    d->view.n_chunks_n = d->n_chunks_n;
+    d->view.chunks_t_dev = reinterpret_cast<const Chunk *>(base + off_bytes + cn_bytes);
+    d->view.n_chunks_t = d->n_chunks_t;
+    d->view.chunks_p_dev = reinterpret_cast<const Chunk *>(base + cp_at);
+    d->view.n_chunks_p = (int)cp.size();
+    d->view.units_dev = reinterpret_cast<const Unit *>(base + un_at);
+    d->view.n_units = (int)un.size();
+    d->view.single_units_dev = reinterpret_cast<const Unit *>(base + us_at);
+    auto walk_view = [&](const WalkPlan &p, size_t at) {
+        return p.ok ? WalkView{reinterpret_cast<const int *>(base + at), p.ngroups, p.period, p.s0, p.k, p.lck, p.astep4}
+                    : WalkView{nullptr, 0, 0, 0, 0, 0, 0};
+    };
+    d->view.walk_n = walk_view(wn, wn_at);
+    d->view.walk_t = walk_view(wt, wt_at);
     auto span = [](const std::vector<Chunk> &t, int &max_len, int &s_min, int &s_max) {
         max_len = 0;
         s_min = t.empty() ? 0 : t.front().s0;
@@ -301,7 +332,7 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const fl
     const int forced = g_path.load();
     const bool tiled_possible = spmm_tiled_ok(desc->view, ldb, ldd, trans);
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {
@@ -310,10 +341,16 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const fl
         tiled = tiled_possible && batch >= SPMM_TILED_MIN_BATCH;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
+    bool walked = false;
+    const int walk = forced == CUVDIA_PATH_WALK ? 1 : forced == CUVDIA_PATH_TILED_NOWALK ? -1 : 0;
     const hipError_t e = tiled
-        ? launch_spmm_tiled(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s)
+        ? launch_spmm_tiled(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s, walk, &walked)
         : launch_spmm_generic(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s);
-    t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
+    if (tiled && walk > 0 && e == hipErrorNotSupported) {
+        (void)hipGetLastError();
+        return CUVDIA_EUNSUPPORTED;
+    }
+    t_last_path = !tiled ? CUVDIA_PATH_GENERIC : walked ? CUVDIA_PATH_WALK : CUVDIA_PATH_TILED;
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "spmm kernel launch");
 }
 
@@ -370,7 +407,7 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
     const int forced = g_path.load();
     const bool tiled_possible = dd2dia_tiled_ok(desc->view, lda, ldb, batch);
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {
@@ -530,9 +567,10 @@ int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals, const int *offsets_host
 
     // the kernel family is chosen by the rule of cuvdia_spmm_layer_f32
     const int forced = g_path.load();
+    if (forced == CUVDIA_PATH_WALK) return CUVDIA_EUNSUPPORTED;
     const bool tiled_possible = spmm_tiled_ok(view, ldb, ldd, trans);
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {

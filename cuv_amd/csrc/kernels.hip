@@ -31,10 +31,10 @@
 
 #include "kernels.hpp"
 
-// This file is compiled four times (CUVDIA_PART = 1 .. 4, see the Makefile), each translation unit
+// This file is compiled five times (CUVDIA_PART = 1 .. 5, see the Makefile), each translation unit
 // instantiating one share of the kernel templates, so that the shares compile in parallel: parts 1 - 3 hold
-// the tiled SpMM kernels by longest chunk (1 - 5, 6 - 9, 10 - 13), part 4 everything else.  Without the macro
-// one unit holds everything.
+// the tiled SpMM kernels by longest chunk (1 - 5, 6 - 9, 10 - 13), part 5 the walking SpMM kernels, part 4
+// everything else.  Without the macro one unit holds everything.
 #ifndef CUVDIA_PART
 #define CUVDIA_PART 0
 #endif
@@ -381,6 +381,8 @@ constexpr int SP_ADIAGS = 16;      // diagonals a chunk's LDS block has room for
 constexpr int SP_AVALS = SP_ADIAGS * SP_ROWS;   // diagonal values per workgroup per chunk
 constexpr int SP_DUMP = SP_XFLOATS + SP_AVALS;  // where idle lanes write
 constexpr int SP_STAGE_FLOATS = SP_DUMP + 4;
+constexpr int SP_WALK_WGS = 512;       // workgroups a walking launch aims at (two per CU)
+constexpr int SP_WALK_MIN_WGS = 384;   // below this the chip is not filled: the tile-by-tile kernels serve
 constexpr int SP_MAX_CHUNKS = 256;   // chunk-table entries a wave can keep in registers (4 sets of 64)
 
 // Per-wave shape: T rows (8 or 16, at most one DPP row of 16 lanes), so a
@@ -452,13 +454,13 @@ __device__ __forceinline__ void spmm_rows(float (&acc)[T], const SpWindow<LCK, T
 }
 
 // The FMAs of N consecutive diagonals J0 .. J0+N-1 of a chunk for a wave of 8 rows, as ONE statement:
-// acc[t] += bcast_t(a[j]) * win[j + t].  A DPP operand must not have been written by a VALU instruction in the
-// two preceding issue slots; inside the statement no FMA writes another's DPP operand (the a[j] come from LDS
-// reads), so one leading s_nop -- for whatever the compiler placed before the statement -- serves all 8*N.
-template <int J0, int N, int NA, int NW>
+// acc[t] += bcast_t(a[j]) * win[W0 + j + t].  A DPP operand must not have been written by a VALU instruction in
+// the two preceding issue slots; inside the statement no FMA writes another's DPP operand (the a[j] come from
+// LDS reads), so one leading s_nop -- for whatever the compiler placed before the statement -- serves all 8*N.
+template <int J0, int N, int W0, int NA, int NW>
 __device__ __forceinline__ void fma_diagonals8(float (&acc)[8], const float (&a)[NA], const float (&win)[NW])
 {
-    static_assert(N >= 1 && N <= 4 && J0 + N <= NA && J0 + N + 7 <= NW, "one statement takes at most 30 operands");
+    static_assert(N >= 1 && N <= 4 && J0 + N <= NA && W0 + J0 + N + 7 <= NW, "one statement takes at most 30 operands");
     if constexpr (N == 1) {
         asm("s_nop 1\n\t"
             "v_fmac_f32_dpp %0, %8, %9 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
@@ -470,7 +472,7 @@ __device__ __forceinline__ void fma_diagonals8(float (&acc)[8], const float (&a)
             "v_fmac_f32_dpp %6, %8, %15 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
             "v_fmac_f32_dpp %7, %8, %16 row_newbcast:7 row_mask:0xf bank_mask:0xf"
             : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
-            : "v"(a[J0 + 0]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]));
+            : "v"(a[J0 + 0]), "v"(win[W0 + J0 + 0]), "v"(win[W0 + J0 + 1]), "v"(win[W0 + J0 + 2]), "v"(win[W0 + J0 + 3]), "v"(win[W0 + J0 + 4]), "v"(win[W0 + J0 + 5]), "v"(win[W0 + J0 + 6]), "v"(win[W0 + J0 + 7]));
     }     else if constexpr (N == 2) {
         asm("s_nop 1\n\t"
             "v_fmac_f32_dpp %0, %8, %10 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
@@ -490,7 +492,7 @@ __device__ __forceinline__ void fma_diagonals8(float (&acc)[8], const float (&a)
             "v_fmac_f32_dpp %6, %9, %17 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
             "v_fmac_f32_dpp %7, %9, %18 row_newbcast:7 row_mask:0xf bank_mask:0xf"
             : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
-            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]), "v"(win[J0 + 8]));
+            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(win[W0 + J0 + 0]), "v"(win[W0 + J0 + 1]), "v"(win[W0 + J0 + 2]), "v"(win[W0 + J0 + 3]), "v"(win[W0 + J0 + 4]), "v"(win[W0 + J0 + 5]), "v"(win[W0 + J0 + 6]), "v"(win[W0 + J0 + 7]), "v"(win[W0 + J0 + 8]));
     }     else if constexpr (N == 3) {
         asm("s_nop 1\n\t"
             "v_fmac_f32_dpp %0, %8, %11 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
@@ -518,7 +520,7 @@ __device__ __forceinline__ void fma_diagonals8(float (&acc)[8], const float (&a)
             "v_fmac_f32_dpp %6, %10, %19 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
             "v_fmac_f32_dpp %7, %10, %20 row_newbcast:7 row_mask:0xf bank_mask:0xf"
             : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
-            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(a[J0 + 2]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]), "v"(win[J0 + 8]), "v"(win[J0 + 9]));
+            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(a[J0 + 2]), "v"(win[W0 + J0 + 0]), "v"(win[W0 + J0 + 1]), "v"(win[W0 + J0 + 2]), "v"(win[W0 + J0 + 3]), "v"(win[W0 + J0 + 4]), "v"(win[W0 + J0 + 5]), "v"(win[W0 + J0 + 6]), "v"(win[W0 + J0 + 7]), "v"(win[W0 + J0 + 8]), "v"(win[W0 + J0 + 9]));
     }     else if constexpr (N == 4) {
         asm("s_nop 1\n\t"
             "v_fmac_f32_dpp %0, %8, %12 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
@@ -554,7 +556,7 @@ __device__ __forceinline__ void fma_diagonals8(float (&acc)[8], const float (&a)
             "v_fmac_f32_dpp %6, %11, %21 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
             "v_fmac_f32_dpp %7, %11, %22 row_newbcast:7 row_mask:0xf bank_mask:0xf"
             : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
-            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(a[J0 + 2]), "v"(a[J0 + 3]), "v"(win[J0 + 0]), "v"(win[J0 + 1]), "v"(win[J0 + 2]), "v"(win[J0 + 3]), "v"(win[J0 + 4]), "v"(win[J0 + 5]), "v"(win[J0 + 6]), "v"(win[J0 + 7]), "v"(win[J0 + 8]), "v"(win[J0 + 9]), "v"(win[J0 + 10]));
+            : "v"(a[J0 + 0]), "v"(a[J0 + 1]), "v"(a[J0 + 2]), "v"(a[J0 + 3]), "v"(win[W0 + J0 + 0]), "v"(win[W0 + J0 + 1]), "v"(win[W0 + J0 + 2]), "v"(win[W0 + J0 + 3]), "v"(win[W0 + J0 + 4]), "v"(win[W0 + J0 + 5]), "v"(win[W0 + J0 + 6]), "v"(win[W0 + J0 + 7]), "v"(win[W0 + J0 + 8]), "v"(win[W0 + J0 + 9]), "v"(win[W0 + J0 + 10]));
     }
 }
 
@@ -565,7 +567,7 @@ __device__ __forceinline__ void spmm_rows_range(float (&acc)[T], const SpWindow<
     if constexpr (J < J1) {
         if constexpr (T == 8) {
             constexpr int N = J1 - J < 4 ? J1 - J : 4;
-            fma_diagonals8<J, N>(acc, win.a, win.w);
+            fma_diagonals8<J, N, 0>(acc, win.a, win.w);
             spmm_rows_range<LCK, T, J + N, J1>(acc, win);
         } else {
             fma_block8<J, 0>(acc, win.a[J], win.w);
@@ -1316,6 +1318,298 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
                                          n_out, n_in, batch, alpha, beta, a_bytes, ep);
 }
 
+#if CUVDIA_IN_PART(5)
+// ------------------------------------------------------------ walking spmm --
+//
+// The product for *window* tables (plan_walk): k window rows `period` rows apart (repeated for every
+// group).  Output tile m of a walk -- the tiles row_first + m * period, m = 0 .. S-1, of one column tile --
+// reads, for window row dy of group g, the dense rows starting at
+//     row_first + s0 + group_rows[g] + (m + dy) * period,
+// so all the (m, dy) with m + dy = u read the SAME rows: block (u, g).  A workgroup walks u = 0 .. S+k-2
+// and, for every group, stages block (u, g) ONCE -- its dense rows and the diagonal values of the up to k
+// tiles that use it -- and applies it to those tiles, which it keeps alive as k sets of running sums
+// (tile m in set m mod k).  One staged block, one window read and one barrier then serve up to k chunks
+// instead of one: the staging per FMA drops k-fold against spmm_tile_lean, and what is left is the FMAs.
+// A tile is complete when its window row k-1 has been applied (step u = m + k - 1): it is stored -- transposed
+// through LDS, so that a lane writes 4 consecutive rows and a column's rows leave as one piece -- and its set
+// starts the tile k steps on.  The walk is unrolled k steps deep so that every set has a static name.
+//
+// Workgroup = 8 waves x T rows (a tile of ROWS = 8 T output rows) x 64 batch columns, lanes <-> columns,
+// diagonal values broadcast by DPP as in spmm_tile_lean.  Two LDS buffers: while block i is applied, block
+// i+1 lands; one wait for everything in flight and one barrier per block.  Every block is staged from the
+// multiple of 4 at or below its first row (a0 - SH; SH = a0 mod 4 is the same for every block of a product
+// and a template parameter, so the window keeps static register indices): with a row count that is a
+// multiple of 4 every 16-byte piece lies wholly inside the operand or outside, and the pieces outside arrive
+// as zeros.  A block wholly outside the operand is skipped.  In a block that crosses an end of the operand
+// the diagonal values of rows whose input row does not exist are padding: such a block's values are fetched
+// element by element with that test (4-byte loads), every other block's as 16-byte pieces.
+//
+// Accumulation order per output element: window rows ascending, groups in table order within a window row
+// (for tile m: blocks (m, 0), (m, 1), .., (m+1, 0), ..), diagonals ascending within a chunk -- the order of
+// ascending shifts when there is one group, as in spmm_tile_lean.
+template <int LCK, int K, int T, int SH>
+struct WalkShape {
+    static constexpr int WAVES = 8;                                         // waves per workgroup
+    static constexpr int ROWS = WAVES * T;                                     // output rows per tile
+    static constexpr int XNEED = SH + ROWS + LCK - 1;                       // staged dense rows that are read
+    static constexpr int XQ = ((XNEED + 3) / 4) | 1;                        // 16-byte pieces per column, odd
+    static constexpr int XPITCH = 4 * XQ;                                   // floats between staged columns
+    static constexpr int XFLOATS = SP_COLS * XPITCH;
+    static constexpr int DPI = 256 / ROWS;                                  // diagonals per 16-byte-piece instruction
+    static constexpr int AI = (LCK + DPI - 1) / DPI;                        // such instructions per (tile, chunk)
+    static constexpr int ATILE = AI * 256;                                  // floats per (tile, chunk) in LDS
+    static constexpr int AFLOATS = K * ATILE;
+    static constexpr int BUF_FLOATS = XFLOATS + AFLOATS;
+    static constexpr int WIN = SH + T + LCK - 1;                            // window values a lane reads
+    static constexpr int WQ = (WIN + 3) / 4;                                // as 16-byte reads
+    static_assert(T == 8, "rows per wave");
+    static constexpr int WGS_PER_CU = (160 * 1024) / (2 * BUF_FLOATS * 4) < 4 ? (160 * 1024) / (2 * BUF_FLOATS * 4) : 4;
+    static_assert(ROWS - T + 4 * WQ <= XPITCH, "the last wave's window lies inside the staged column");
+    static_assert(2 * BUF_FLOATS * 4 <= 80 * 1024, "two workgroups share a CU's LDS");
+    static constexpr int WAVES_PER_SIMD = WGS_PER_CU * WAVES / 4 < 4 ? WGS_PER_CU * WAVES / 4 : 4;
+};
+
+// calls f(I) for I = 0 .. K-1 as compile-time constants
+template <int K, int I, class F>
+__device__ __forceinline__ void walk_for(F &&f)
+{
+    if constexpr (I < K) {
+        f(std::integral_constant<int, I>{});
+        walk_for<K, I + 1>(f);
+    }
+}
+// calls step(u0 + UU, UU) for UU = 0 .. K-1 while u0 + UU < nsteps: the step's position in its group of K
+// is a compile-time constant
+template <int K, int UU, class F>
+__device__ __forceinline__ void walk_steps(F &step, int u0, int nsteps)
+{
+    if constexpr (UU < K) {
+        if (u0 + UU < nsteps) step(u0 + UU, std::integral_constant<int, UU>{});
+        walk_steps<K, UU + 1>(step, u0, nsteps);
+    }
+}
+
+template <int LCK, int K, int T, int SH>
+__global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) void spmm_walk_kernel(
+    const int *__restrict__ tab,            // group_rows[ngroups], then aoff4[ngroups * K]
+    int ngroups, int period, int s0, int astep4, int seg_tiles, const float *__restrict__ vals,
+    const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
+    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes)
+{
+    typedef WalkShape<LCK, K, T, SH> S;
+    constexpr int WAVES = S::WAVES, ROWS = S::ROWS, XQ = S::XQ, XPITCH = S::XPITCH, AI = S::AI, ATILE = S::ATILE, WQ = S::WQ;
+    __shared__ __attribute__((aligned(16))) float lds[2][S::BUF_FLOATS];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+    // workgroup -> (segment, residue, column tile): the row tiles r, r + TP, r + 2 TP, .. (TP = period / ROWS) form
+    // the walk of residue r; it is cut into segments of seg_tiles tiles
+    const int tp = period / ROWS;
+    const int wg = xcd_tile(blockIdx.x, gridDim.x);
+    const int coltile = wg % col_tiles;
+    const int rest = wg / col_tiles;
+    const int res = rest % tp, seg = rest / tp;
+    const int n_rt = n_out / ROWS;
+    const int walk_len = (n_rt - res + tp - 1) / tp;              // tiles of this residue
+    const int m0 = seg * seg_tiles;
+    const int ntiles = min(seg_tiles, walk_len - m0);
+    if (ntiles <= 0) return;
+    const int row_first = (res + tp * m0) * ROWS;
+    const int col0 = coltile * SP_COLS;
+    const int cols_here = min(SP_COLS, batch - col0);
+    const int nsteps = ntiles + K - 1;
+    const int nblocks = nsteps * ngroups;
+
+    // dense rows: instruction i = wave + WAVES it of a block stages pieces 64 i .. 64 i + 63, piece p = XQ * column + quad
+    constexpr int XIT = (XQ + WAVES - 1) / WAVES;
+    // A lane's share of the requests is recomputed from its lane number for every block (a few integer
+    // operations) rather than kept in registers across the walk: the running sums need them.
+    auto lane_now = [&]() __attribute__((always_inline)) {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return l;
+    };
+    const unsigned x_bytes = (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4);
+    const sp_int4 xq = raw_rsrc(X + (long long)col0 * ldx, x_bytes);
+    const sp_int4 aq = raw_rsrc(vals, a_bytes);
+    const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
+    constexpr unsigned BUF_BYTES = S::BUF_FLOATS * 4u;
+
+    typedef const int __attribute__((address_space(4))) *sc_int_ptr;
+    const sc_int_ptr stab = (sc_int_ptr)tab;
+
+    // Requests block number i (step u = i / ngroups, group g = i % ngroups) into buffer i & 1: its dense
+    // rows and, for every tile m = u - dy that exists, the values of chunk (g, dy) for the tile's rows.
+    auto issue = [&](int i) __attribute__((always_inline)) {
+        const int u = i / ngroups, g = i - u * ngroups;
+        const int a0 = row_first + s0 + stab[g] + u * period;        // first dense row the block's chunks read
+        if (a0 + ROWS + LCK - 1 <= 0 || a0 >= n_in) return;          // wholly outside: nothing to stage (see apply)
+        const unsigned buf = lds0 + (unsigned)(i & 1) * BUF_BYTES;
+        const int a0p = a0 - SH;                                     // a multiple of 4
+        const int ln = lane_now();
+#pragma unroll
+        for (int it = 0; it < XIT; ++it) {
+            if (wave + WAVES * it < XQ) {
+                const int piece = 64 * (wave + WAVES * it) + ln;
+                const int col = piece / XQ;
+                const int r = a0p + 4 * (piece - col * XQ);
+                const unsigned x_col = (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u);
+                const bool ok = (r >= 0) & (r + 4 <= n_in);
+                lds_load_b128(xq, buf + 1024u * (unsigned)(wave + WAVES * it), ok ? x_col + (unsigned)(r * 4) : OOB_OFFSET, 0u);
+            }
+        }
+        const bool inside = (a0 >= 0) & (a0 + ROWS + LCK - 1 <= n_in);
+        const unsigned abuf = buf + (unsigned)S::XFLOATS * 4u;
+        if (inside) {
+            // 16-byte pieces: instruction n = dy * AI + h carries diagonals h*DPI .. of tile u - dy's chunk,
+            // lane = (ROWS/4) * diagonal + piece
+            for (int n = wave; n < K * AI; n += WAVES) {
+                const int dy = n / AI, h = n - dy * AI;
+                const int m = u - dy;
+                if (m < 0 || m >= ntiles) continue;
+                const int j = h * S::DPI + ln / (ROWS / 4), piece = ln % (ROWS / 4);
+                const int row = row_first + m * period + 4 * piece;
+                const unsigned off = (unsigned)(stab[ngroups + g * K + dy] + row * 4 + j * astep4);
+                lds_load_b128(aq, abuf + (unsigned)(n * 1024), j < LCK ? off : OOB_OFFSET, 0u);
+            }
+        } else {
+            // the block crosses an end of the operand: 4-byte loads, each lane testing its own element.
+            // Instruction n = dy * NI + h carries EPI diagonals x ROWS rows, lane = ROWS * diagonal + row.
+            constexpr int EPI = 64 / ROWS;                           // diagonals per instruction (1 or 2)
+            constexpr int NI = (LCK + EPI - 1) / EPI;
+            for (int n = wave; n < K * NI; n += WAVES) {
+                const int dy = n / NI, h = n - dy * NI;
+                const int m = u - dy;
+                if (m < 0 || m >= ntiles) continue;
+                const int j = h * EPI + ln / ROWS, i_row = ln % ROWS;
+                const int in = a0 + i_row + j;                       // the input row this value multiplies
+                const bool ok = (j < LCK) & ((unsigned)in < (unsigned)n_in);
+                const int row = row_first + m * period + i_row;
+                const unsigned off = (unsigned)(stab[ngroups + g * K + dy] + row * 4 + j * astep4);
+                lds_load_b32(aq, abuf + (unsigned)((dy * ATILE + h * EPI * ROWS) * 4), ok ? off : OOB_OFFSET);
+            }
+        }
+    };
+
+    float acc[K][T];
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[k][t] = 0.f;
+
+    // Applies block i = (u, g) to the tiles that use it; UU = u mod K gives the sets their static names:
+    // tile m = u - dy sits in set (UU - dy) mod K.
+    auto apply = [&](int i, int u, int g, auto uu_c) __attribute__((always_inline)) {
+        constexpr int UU = decltype(uu_c)::value;
+        const int a0 = row_first + s0 + stab[g] + u * period;
+        if (a0 + ROWS + LCK - 1 <= 0 || a0 >= n_in) return;
+        const float *buf = &lds[i & 1][0];
+        float win[4 * WQ];
+        {
+            const float4 *p4 = reinterpret_cast<const float4 *>(buf + lane * XPITCH + wave * T);
+#pragma unroll
+            for (int q = 0; q < WQ; ++q) {
+                const float4 v = p4[q];
+                win[4 * q + 0] = v.x; win[4 * q + 1] = v.y; win[4 * q + 2] = v.z; win[4 * q + 3] = v.w;
+            }
+        }
+        const float *abase = buf + S::XFLOATS + wave * T + (lane & (T - 1));
+        auto fma_chunk = [&](float (&set)[T], const float (&a)[LCK]) __attribute__((always_inline)) {
+            constexpr int NB = (LCK + 3) / 4;
+            if constexpr (NB >= 1) fma_diagonals8<0, (LCK < 4 ? LCK : 4), SH>(set, a, win);
+            if constexpr (NB >= 2) fma_diagonals8<4, (LCK < 8 ? LCK - 4 : 4), SH>(set, a, win);
+            if constexpr (NB >= 3) fma_diagonals8<8, (LCK < 12 ? LCK - 8 : 4), SH>(set, a, win);
+            if constexpr (NB >= 4) fma_diagonals8<12, LCK - 12, SH>(set, a, win);
+        };
+        // One path for every step: the values of chunk dy + 1 are read while chunk dy's FMAs run, whether or
+        // not tile u - dy - 1 exists (the values of a tile that does not are whatever the buffer held, and are
+        // not used); only the FMAs are skipped, so no running sum changes registers between the cases.
+        float a[2][LCK];
+#pragma unroll
+        for (int j = 0; j < LCK; ++j) a[0][j] = abase[j * ROWS];
+        walk_for<K, 0>([&](auto dy_c) __attribute__((always_inline)) {
+            constexpr int dy = decltype(dy_c)::value;
+            if constexpr (dy + 1 < K) {
+#pragma unroll
+                for (int j = 0; j < LCK; ++j) a[(dy + 1) & 1][j] = abase[(dy + 1) * ATILE + j * ROWS];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const int m = u - dy;
+            if (m >= 0 && m < ntiles) fma_chunk(acc[((UU - dy) % K + K) % K], a[dy & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    // The final store runs along the rows: 4 consecutive rows of a column per lane (LPC lanes per column, CPI
+    // columns per instruction, NST instructions for the wave's CPW columns), after a transposition through LDS.
+    constexpr int LPC = ROWS / 4, CPI = 64 / LPC, CPW = SP_COLS / WAVES, NST = CPW / CPI, OPITCH = ROWS + 4;
+    static_assert(SP_COLS * OPITCH <= S::XFLOATS, "the transposition fits the dense rows' part of a buffer");
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    // Stores the tile that step u completes (m = u - K + 1, set (UU + 1) mod K) and clears its set for the tile
+    // K steps on.  `ilast` is the step's last block: every wave is through with its buffer (the barrier that
+    // ended the block), and the next request into it comes after the second barrier below.
+    auto finish = [&](int u, int ilast, auto uu_c, const f4u (&ypre)[NST]) __attribute__((always_inline)) {
+        constexpr int SET = (decltype(uu_c)::value + 1) % K;
+        const int m = u - (K - 1);
+        if (m >= 0 && m < ntiles) {
+            const int ln = lane_now();
+            const int ecol = wave * CPW + ln / LPC, erow = 4 * (ln % LPC);
+            float *out = &lds[ilast & 1][0];
+#pragma unroll
+            for (int t = 0; t < T; ++t) out[lane * OPITCH + wave * T + t] = acc[SET][t];
+            __syncthreads();
+            f4u v[NST];
+#pragma unroll
+            for (int q = 0; q < NST; ++q) v[q] = *reinterpret_cast<const f4u *>(out + (ecol + CPI * q) * OPITCH + erow);
+#pragma unroll
+            for (int q = 0; q < NST; ++q) {
+                const int col = ecol + CPI * q;
+                if (col < cols_here) {
+                    float *y = Y + (long long)(col0 + col) * ldy + row_first + m * period + erow;
+                    float r[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) r[e] = (beta == 0.f) ? alpha * v[q][e] : beta * ypre[q][e] + alpha * v[q][e];
+                    stream_store4(y, r[0], r[1], r[2], r[3]);
+                }
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[SET][t] = 0.f;
+    };
+
+    issue(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    auto step = [&](int u, auto uu_c) __attribute__((always_inline)) {
+        // destination values of the tile this step completes (beta != 0), requested ahead of its last blocks
+        f4u ypre[NST];
+#pragma unroll
+        for (int q = 0; q < NST; ++q) ypre[q] = f4u{0.f, 0.f, 0.f, 0.f};
+        const int mf = u - (K - 1);
+        if (beta != 0.f && mf >= 0 && mf < ntiles) {
+            const int ln = lane_now();
+            const int ecol = wave * CPW + ln / LPC, erow = 4 * (ln % LPC);
+#pragma unroll
+            for (int q = 0; q < NST; ++q) {
+                const int col = ecol + CPI * q;
+                if (col < cols_here)
+                    ypre[q] = *reinterpret_cast<const f4u *>(Y + (long long)(col0 + col) * ldy + row_first + mf * period + erow);
+            }
+        }
+        int i = u * ngroups;
+        for (int g = 0; g < ngroups; ++g, ++i) {
+            if (i + 1 < nblocks) issue(i + 1);
+            apply(i, u, g, uu_c);
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+        finish(u, i - 1, uu_c, ypre);
+    };
+    for (int u0 = 0; u0 < nsteps; u0 += K) walk_steps<K, 0>(step, u0, nsteps);
+}
+#endif  // part 5
+
 // ------------------------------------------------------------ tiled dd2dia --
 //
 // Workgroup = 256 rows of ONE unit: a run chunk, or two chunks whose first
@@ -1784,6 +2078,23 @@ struct SpLaunch {
     hipStream_t stream;
     int lck;
 };
+// The walking kernel's launch (its unit instantiates the kernel); returns hipErrorNotSupported when no
+// instantiation fits the table.
+struct WalkLaunch {
+    const int *tab;
+    int ngroups, period, s0, astep4, lck, k, seg_tiles;
+    const float *vals, *B;
+    long long ldb;
+    float *dst;
+    long long ldd;
+    int n_out, n_in, batch;
+    float alpha, beta;
+    int col_tiles;
+    unsigned a_bytes;
+    hipStream_t stream;
+};
+hipError_t spmm_walk_launch(const WalkLaunch &L, bool dry_run);
+int spmm_walk_tile_rows(int lck, int k, int s0);     // output rows per tile of the instantiation that serves the window; 0: none
 hipError_t spmm_tiled_launch_1_5(const SpLaunch &L);
 hipError_t spmm_tiled_launch_6_9(const SpLaunch &L);
 hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
@@ -1803,6 +2114,38 @@ hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
         else                                                                                                          \
             hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 4, true>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS);  \
         break;
+#if CUVDIA_IN_PART(5)
+// rows per wave of the instantiation that serves a window of k rows of lck diagonals whose first shift is
+// s0 (0: none).  Instantiated: the centred 3x3, 5x5 and 7x7 windows.  (A 13x13 window needs 13 sets of running
+// sums: with the registers that leaves, two waves per SIMD, it ran slower than the tile-by-tile kernel.)
+static int walk_rows_per_wave(int lck, int k, int s0)
+{
+    const int sh = ((s0 % 4) + 4) % 4;
+    if (lck == 7 && k == 7 && sh == 1) return 8;
+    if (lck == 5 && k == 5 && sh == 2) return 8;
+    if (lck == 3 && k == 3 && sh == 3) return 8;
+    return 0;
+}
+int spmm_walk_tile_rows(int lck, int k, int s0) { return 8 * walk_rows_per_wave(lck, k, s0); }
+hipError_t spmm_walk_launch(const WalkLaunch &L, bool dry_run)
+{
+    const int rows = spmm_walk_tile_rows(L.lck, L.k, L.s0);
+    if (rows == 0) return hipErrorNotSupported;
+    if (L.n_out % rows != 0 || L.n_in % 4 != 0 || L.period % rows != 0) return hipErrorNotSupported;
+    if (dry_run) return hipSuccess;
+    const int tp = L.period / rows;
+    const int walk_len = (L.n_out / rows + tp - 1) / tp;
+    const int nseg = (walk_len + L.seg_tiles - 1) / L.seg_tiles;
+    const dim3 grid((unsigned)((long long)nseg * tp * L.col_tiles));
+#define CUVDIA_WALK_ARGS L.tab, L.ngroups, L.period, L.s0, L.astep4, L.seg_tiles, L.vals, L.B, L.ldb, L.dst, L.ldd, \
+                         L.n_out, L.n_in, L.batch, L.alpha, L.beta, L.col_tiles, L.a_bytes
+    if (L.lck == 7) hipLaunchKernelGGL((spmm_walk_kernel<7, 7, 8, 1>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
+    else if (L.lck == 5) hipLaunchKernelGGL((spmm_walk_kernel<5, 5, 8, 2>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
+    else hipLaunchKernelGGL((spmm_walk_kernel<3, 3, 8, 3>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
+#undef CUVDIA_WALK_ARGS
+    return hipGetLastError();
+}
+#endif
 #if CUVDIA_IN_PART(1)
 hipError_t spmm_tiled_launch_1_5(const SpLaunch &L)
 {
@@ -1842,8 +2185,9 @@ hipError_t spmm_tiled_launch_10_13(const SpLaunch &L)
 #if CUVDIA_IN_PART(4)
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
-                             float alpha, float beta, SpEpilogue ep, hipStream_t stream)
+                             float alpha, float beta, SpEpilogue ep, hipStream_t stream, int walk, bool *walked)
 {
+    if (walked) *walked = false;
     const int n_out = trans ? A.w : A.h;
     const int n_in = trans ? A.h : A.w;
     const long long row_tiles = (n_out + SP_ROWS - 1) / SP_ROWS;
@@ -1854,6 +2198,29 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     // along the rows and find each other's dense rows in its L2.
     const int col_group = col_tiles <= 4 ? (int)col_tiles : 2;
     const int lck = trans ? A.max_len_t : A.max_len_n;
+    // A window table on a product of many tiles: the walking kernel (plain products only).
+    const WalkView &wk = trans ? A.walk_t : A.walk_n;
+    if (walk >= 0 && wk.tab_dev != nullptr && ep.bias == nullptr && ep.act == 0) {
+        WalkLaunch W{wk.tab_dev, wk.ngroups, wk.period, wk.s0, wk.astep4, wk.lck, wk.k, 0, vals, B, ldb, dst, ldd,
+                     n_out, n_in, batch, alpha, beta, (int)col_tiles, (unsigned)((long long)A.nd * A.stride * 4), stream};
+        if (spmm_walk_launch(W, true) == hipSuccess) {
+            // Segments: as long as they can be while the launch still fills the chip (SP_WALK_WGS workgroups),
+            // but no shorter than the window has rows -- a segment of S tiles stages S + k - 1 blocks.
+            const int rows = spmm_walk_tile_rows(wk.lck, wk.k, wk.s0);
+            const long long tp = wk.period / rows;
+            const long long walk_len = (n_out / rows + tp - 1) / tp;
+            const long long walks = tp * col_tiles;
+            long long nseg = (SP_WALK_WGS + walks - 1) / walks;
+            if (nseg > walk_len / wk.k) nseg = walk_len / wk.k;
+            if (walk > 0 && nseg < 1) nseg = 1;
+            if (nseg >= 1 && (walk > 0 || nseg * walks >= SP_WALK_MIN_WGS)) {
+                W.seg_tiles = (int)((walk_len + nseg - 1) / nseg);
+                if (walked) *walked = true;
+                return spmm_walk_launch(W, false);
+            }
+        }
+    }
+    if (walk > 0) return hipErrorNotSupported;
     const SpLaunch L{trans ? A.chunks_t_dev : A.chunks_n_dev,
                      trans ? A.n_chunks_t : A.n_chunks_n,
                      vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha, beta,

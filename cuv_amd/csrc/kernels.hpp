@@ -10,6 +10,12 @@
 
 namespace cuvdia {
 
+// Device form of a window table (plan_walk) for one traversal; tab_dev == nullptr: not a window table.
+struct WalkView {
+    const int *tab_dev;          // group_rows[ngroups], then aoff4[ngroups * k]
+    int ngroups, period, s0, k, lck, astep4;
+};
+
 struct DiaView {
     int h, w, nd, stride, rf;
     const int *offsets_dev;      // nd ints, table order
@@ -20,6 +26,7 @@ struct DiaView {
     int max_len_n, max_len_t;    // longest chunk of each table
     int s_min_n, s_max_n;        // smallest / largest chunk shift of each table
     int s_min_t, s_max_t;
+    WalkView walk_n, walk_t;     // window-table form of the two products' tables
     const Chunk *chunks_p_dev;   // the projection's table (chunks of up to CHUNK_MAX): shifts = offsets
     int n_chunks_p;
     int max_len_p;
@@ -48,10 +55,15 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
 // Same contract, row_fact == 1 only: 64 output rows x 64 batch columns per
 // workgroup, dense tile staged through LDS once per run chunk, lanes own
 // batch columns and keep a sliding register window along the rows, diagonal
-// values are broadcast across each 16-lane row by DPP.
+// values are broadcast across each 16-lane row by DPP.  Window tables on
+// products of many tiles go to the walking kernel, which stages a block of
+// dense rows once for all the window rows that read it.  `walk`: 0 -- that
+// choice is made by size; 1 -- the walking kernel or hipErrorNotSupported;
+// -1 -- never the walking kernel.  *walked (if not null) tells which ran.
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
-                             float alpha, float beta, SpEpilogue ep, hipStream_t stream);
+                             float alpha, float beta, SpEpilogue ep, hipStream_t stream,
+                             int walk = 0, bool *walked = nullptr);
 
 // m = mw*M[i] - lr*(dW[i] + l2*W[i]); W[i] += m; M[i] = m, i < n.
 hipError_t launch_momentum(float *W, float *M, const float *dW, long long n, float lr, float mw, float l2,

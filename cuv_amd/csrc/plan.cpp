@@ -38,6 +38,73 @@ std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, int 
     return out;
 }
 
+namespace {
+long long gcd_ll(long long a, long long b)
+{
+    while (b) { const long long t = a % b; a = b; b = t; }
+    return a < 0 ? -a : a;
+}
+}  // namespace
+
+void plan_walk(const std::vector<Chunk> &chunks, int stride, bool transposed, WalkPlan &plan)
+{
+    plan = WalkPlan{};
+    const int n = (int)chunks.size();
+    if (n < 2) return;
+    // every chunk as long as the first, table positions in one arithmetic progression
+    const int lck = chunks.front().len;
+    long long step = 0;
+    bool have_step = false;
+    for (const Chunk &c : chunks) {
+        if (c.len != lck) return;
+        for (int j = 0; j < lck; ++j)
+            if (c.slot[j] < 0) return;
+        for (int j = 1; j < lck; ++j) {
+            const long long d = (long long)c.slot[j] - c.slot[j - 1];
+            if (!have_step) { step = d; have_step = true; }
+            else if (d != step) return;
+        }
+    }
+    const long long limit = 1LL << 29;               // 4 * value stays inside 32-bit signed arithmetic
+    const long long astep = step * stride + (transposed ? 1 : 0);
+    if (astep >= limit || astep <= -limit) return;
+    // the period: what all the shifts' distances from the first are multiples of
+    long long period = 0;
+    for (int i = 1; i < n; ++i) {
+        const long long d = (long long)chunks[i].s0 - chunks[0].s0;
+        if (d <= 0) return;                          // shifts ascend strictly
+        period = gcd_ll(period, d);
+    }
+    if (period <= 0 || period >= limit) return;
+    // window rows: the leading shifts 0, period, 2 period, ...; then whole groups of the same k rows
+    int k = 1;
+    while (k < n && (long long)chunks[k].s0 - chunks[0].s0 == (long long)k * period) ++k;
+    if (n % k != 0) return;
+    const int ngroups = n / k;
+    std::vector<int> group_rows(ngroups), aoff4(n);
+    for (int g = 0; g < ngroups; ++g) {
+        const long long base = (long long)chunks[g * k].s0 - chunks[0].s0;
+        if (base >= limit) return;
+        group_rows[g] = (int)base;
+        for (int dy = 0; dy < k; ++dy) {
+            const Chunk &c = chunks[g * k + dy];
+            if ((long long)c.s0 - chunks[0].s0 != base + (long long)dy * period) return;
+            const long long aoff = (long long)c.slot[0] * stride + (transposed ? c.s0 : 0);
+            if (aoff >= limit || aoff <= -limit) return;
+            aoff4[g * k + dy] = (int)(4 * aoff);
+        }
+    }
+    plan.ok = true;
+    plan.period = (int)period;
+    plan.k = k;
+    plan.ngroups = ngroups;
+    plan.s0 = chunks[0].s0;
+    plan.lck = lck;
+    plan.astep4 = (int)(4 * astep);
+    plan.group_rows.swap(group_rows);
+    plan.aoff4.swap(aoff4);
+}
+
 std::vector<Unit> plan_units(const std::vector<Chunk> &chunks)
 {
     std::vector<Unit> out;

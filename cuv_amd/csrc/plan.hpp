@@ -26,6 +26,24 @@ struct Chunk {
 };
 static_assert(sizeof(Chunk) == 64 && SP_CHUNK_MAX <= CHUNK_SLOTS, "Chunk layout is part of the device table");
 
+// A *window* table, the shape a 2-d (or multi-channel 2-d) local connection pattern gives a DIA matrix: every
+// chunk has `lck` diagonals at table positions in arithmetic progression (one step for the whole table), and
+// the chunks' shifts form a complete grid
+//     s(g, dy) = s0 + group_rows[g] + dy * period,    g < ngroups, dy < k,
+// -- k window rows `period` rows apart, repeated for every group (channel offset).  Output tiles `period` rows
+// apart then read the same dense rows for neighbouring window rows, which is what the products' walking kernel
+// exploits.  aoff4[g * k + dy] is 4 * the element offset of chunk (g, dy)'s first diagonal for output row 0,
+// astep4 4 * the element step between its diagonals (value of (chunk, diagonal j, output row r):
+// element aoff + r + j * astep).
+struct WalkPlan {
+    bool ok = false;
+    int period = 0, k = 0, ngroups = 0, s0 = 0, lck = 0, astep4 = 0;
+    std::vector<int> group_rows;     // ngroups, ascending, group_rows[0] == 0
+    std::vector<int> aoff4;          // ngroups * k
+};
+// `chunks`: a table from plan_chunks (shifts ascending).  plan.ok is false when the table is no window table.
+void plan_walk(const std::vector<Chunk> &chunks, int stride, bool transposed, WalkPlan &plan);
+
 // Sort shifts (stable in table position), cut into maximal runs of
 // consecutive shifts -- a repeated shift starts a new run -- and split each
 // run into near-equal chunks of at most max_len (<= CHUNK_SLOTS).  Positions

@@ -50,6 +50,8 @@ extern "C" {
 #define CUVDIA_PATH_AUTO     0  /* pick by shape (default)                        */
 #define CUVDIA_PATH_GENERIC  1  /* one-thread-per-output kernels, any row_fact    */
 #define CUVDIA_PATH_TILED    2  /* LDS-staged, register-blocked kernels (rf == 1) */
+#define CUVDIA_PATH_WALK     3  /* of the tiled family: the walking kernel for window tables (products only) */
+#define CUVDIA_PATH_TILED_NOWALK 4  /* the tiled family without its walking kernel (products only)         */
 
 /* Activation applied by cuvdia_spmm_bias_act_f32. */
 #define CUVDIA_ACT_NONE      0
@@ -244,8 +246,11 @@ int cuvdia_dd2dia_offsets_f32(float *C_vals_device, const int *offsets_host,
 /* cuvdia_spmm_offsets_f32 for callers that cannot allocate device memory:
  * code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  It has no counterpart in the reference.  Same arguments, same
- * argument rules, same kernels and bit-identical results; but the device copy
- * of the offset table and of the chunk table the kernels walk -- which a
+ * argument rules, and the generic or tile-by-tile kernels chosen as there:
+ * bit-identical results wherever cuvdia_spmm_offsets_f32 does not take its
+ * walking kernel (large products of window tables; CUVDIA_PATH_TILED_NOWALK
+ * keeps it from doing so), within rounding of them where it does.  But the
+ * device copy of the offset table and of the chunk table the kernels walk -- which a
  * descriptor keeps in memory it allocates -- lives in a static device array
  * of 20480 bytes inside the library (one copy per GPU, held until the process
  * ends), so the call performs no hipMalloc, no hipFree and no allocating
@@ -270,11 +275,16 @@ int cuvdia_cache_clear(void);
 /* Forces a kernel family for subsequent calls (process-wide; tests use it to
  * run both families on the same inputs).  CUVDIA_PATH_TILED on a request the
  * tiled kernels cannot serve (row_fact > 1) returns CUVDIA_EUNSUPPORTED from
- * the compute call. */
+ * the compute call.  CUVDIA_PATH_WALK and CUVDIA_PATH_TILED_NOWALK choose
+ * inside the tiled family for the products (cuvdia_spmm_*): the walking
+ * kernel whatever the product's size (CUVDIA_EUNSUPPORTED when the table is
+ * no window table it serves), or never; densedense_to_dia treats both as
+ * CUVDIA_PATH_TILED. */
 int cuvdia_set_path(int path);
 
 /* Which family the most recent compute call on this thread launched
- * (CUVDIA_PATH_GENERIC or CUVDIA_PATH_TILED; 0 before any call). */
+ * (CUVDIA_PATH_GENERIC, CUVDIA_PATH_TILED or -- a product served by the
+ * walking kernel -- CUVDIA_PATH_WALK; 0 before any call). */
 int cuvdia_last_path(void);
 
 /* Static string for an error code. */

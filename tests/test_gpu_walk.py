@@ -1,0 +1,111 @@
+"""The walking SpMM kernel against the CPU oracle.
+
+Window tables (k window rows of k consecutive diagonals, `period` rows apart,
+period a multiple of the 64-row tile) on products of many tiles are served by
+workgroups that walk down the rows and keep k tiles alive.  The tests force
+that kernel on sizes the oracle finishes in seconds, with NaN in every padding
+slot of the matrix and in the destination when beta == 0, and check that the
+automatic choice takes it on a product that is large enough and leaves it
+alone where its shape conditions do not hold.  Tolerance: the fp32 bar of
+_gpu_util.assert_close_mag (1e-5 of the sum of |terms| per element).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gu():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    import _gpu_util
+    return _gpu_util
+
+
+def _window_dia(o, rng, h, w, px, fs, channels=1):
+    from cuv_amd import workloads as W
+    d = o.Dia(h, w, W.window_offsets(px, fs, channels), None, 1)
+    d.vals[:] = np.nan
+    m = o.valid_mask(d)
+    d.vals[m] = rng.uniform(-1, 1, int(m.sum())).astype(np.float32)
+    return d
+
+
+def _operands(rng, A, batch, trans):
+    n_in, n_out = (A.h, A.w) if trans == "t" else (A.w, A.h)
+    B = np.asfortranarray(rng.uniform(-1, 1, (n_in, batch)).astype(np.float32))
+    dst = np.asfortranarray(rng.uniform(-1, 1, (n_out, batch)).astype(np.float32))
+    return B, dst
+
+
+# px, window, channels, batch: one and several segments per walk, a ragged last column tile, two residues
+# per period (px 128), several groups (channels)
+WALK_CASES = [
+    (64, 7, 1, 64),
+    (64, 7, 1, 70),
+    (128, 7, 1, 33),
+    (64, 5, 1, 130),
+    (64, 3, 1, 64),
+    (64, 7, 2, 64),
+    (64, 5, 3, 17),
+]
+
+
+@pytest.mark.parametrize("px,fs,channels,batch", WALK_CASES)
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_walk_matches_the_oracle(oracle, gu, px, fs, channels, batch, trans):
+    from cuv_amd import _lib
+    rng = np.random.default_rng(px * 100 + fs * 10 + channels + batch)
+    n = px * px * channels
+    A = _window_dia(oracle, rng, n, n, px, fs, channels)
+    B, dst = _operands(rng, A, batch, trans)
+    _, ran = gu.check_prod(oracle, A, B, None, trans, 1.0, 0.0, _lib.PATH_WALK, "walk beta0")
+    assert ran == _lib.PATH_WALK
+    _, ran = gu.check_prod(oracle, A, B, dst, trans, 0.75, -1.5, _lib.PATH_WALK, "walk scaled")
+    assert ran == _lib.PATH_WALK
+
+
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_walk_on_a_rectangular_matrix_with_a_short_last_segment(oracle, gu, trans):
+    """60 row tiles per walk: the last segment is shorter than the others, and the window hangs over the
+    operand's end in one direction only."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(5)
+    h, w = (64 * 60, 64 * 64) if trans == "n" else (64 * 64, 64 * 60)
+    A = _window_dia(oracle, rng, h, w, 64, 7)
+    B, dst = _operands(rng, A, 96, trans)
+    _, ran = gu.check_prod(oracle, A, B, dst, trans, 1.0, 0.5, _lib.PATH_WALK, "walk rectangular")
+    assert ran == _lib.PATH_WALK
+
+
+def test_walk_is_refused_where_its_shape_conditions_fail(oracle, gu):
+    """A 48-wide map (window rows 48 apart: not a multiple of the tile's 64 rows) and a 9x9 window have no
+    walking kernel: forcing it is an error, the automatic choice falls back to the tile-by-tile kernel."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(7)
+    for px, fs in ((48, 7), (64, 9)):
+        n = px * px
+        A = _window_dia(oracle, rng, n, n, px, fs)
+        B, dst = _operands(rng, A, 64, "n")
+        with pytest.raises(_lib.CuvDiaError):
+            gu.gpu_prod(A, B, dst, "n", 1.0, 0.0, _lib.PATH_WALK)
+        _, ran = gu.check_prod(oracle, A, B, dst, "n", 1.0, 0.0, _lib.PATH_AUTO, "fallback")
+        assert ran == _lib.PATH_TILED
+
+
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_automatic_choice_walks_a_large_product(oracle, gu, trans):
+    """128x128 map, 7x7 window, batch 1536: 6144 tiles -- the automatic choice takes the walking kernel, and
+    a small batch on the same matrix stays with the tile-by-tile kernel."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(8)
+    n = 128 * 128
+    A = _window_dia(oracle, rng, n, n, 128, 7)
+    dev = gu.make_dev_dia(A)
+    B, dst = _operands(rng, A, 1536, trans)
+    _, ran = gu.check_prod(oracle, A, B, dst, trans, 1.0, 0.5, _lib.PATH_AUTO, "auto large", dev=dev)
+    assert ran == _lib.PATH_WALK
+    B, dst = _operands(rng, A, 128, trans)
+    _, ran = gu.check_prod(oracle, A, B, dst, trans, 1.0, 0.5, _lib.PATH_AUTO, "auto small", dev=dev)
+    assert ran == _lib.PATH_TILED
