@@ -47,10 +47,12 @@ def load_traffic():
         return {"up_pass": None, "down_pass": None, "weight_gradient": None}, None
 
 
-FP32_VALU_PEAK_TFLOPS = 157.3  # published vector fp32 (packed); the kernels use no MFMA
-# What the vector units deliver without packed-fp32 instructions (switched off in this build):
-# 256 CUs x 4 SIMDs x 16 lanes x 2 FLOP x 2.4 GHz
-FP32_VALU_UNPACKED_TFLOPS = 78.6
+FP32_VALU_PEAK_TFLOPS = 157.3  # published vector fp32; the kernels use no MFMA
+# The rate of v_fmac_f32 with a DPP-broadcast or scalar operand, one wave64 instruction per SIMD per 4 clocks:
+# 256 CUs x 4 SIMDs x 16 lanes x 2 FLOP x 2.4 GHz (measured on the box: 75.7 TFLOP/s).  The products keep the
+# batch along the lanes and broadcast the diagonal's value that way, so this is the ceiling of their arithmetic;
+# only the form with three vector-register operands runs at twice that (124-137 TFLOP/s measured).
+FP32_VALU_BROADCAST_TFLOPS = 78.6
 
 
 def parse():
@@ -130,7 +132,7 @@ def measure_cfg4(steps, torch, D, W, dev, with_aux=True):
         tf = flops / (ms * 1e-3) / 1e12
         res[name] = dict(ms=ms, bytes=nbytes, flops=flops, gbs=nbytes / (ms * 1e-3) / 1e9,
                          frac_hbm=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, tflops=tf,
-                         frac_fp32_valu=tf / FP32_VALU_PEAK_TFLOPS, frac_fp32_valu_unpacked=tf / FP32_VALU_UNPACKED_TFLOPS)
+                         frac_fp32_valu=tf / FP32_VALU_PEAK_TFLOPS, frac_fp32_valu_broadcast=tf / FP32_VALU_BROADCAST_TFLOPS)
     aux = {}
     for name, (fn, nbytes) in aux_ops.items():
         ms = timed(fn)
@@ -493,7 +495,7 @@ def main():
         # what the two ceilings allow: the algorithmic bytes at the HBM peak, and the FLOPs at the vector rate
         # without packed-fp32 instructions
         per[name]["hbm_floor_us"] = per[name]["bytes"] / (HBM_PEAK_GBS * 1e9) * 1e6
-        per[name]["valu_floor_us"] = per[name]["flops"] / (FP32_VALU_UNPACKED_TFLOPS * 1e12) * 1e6
+        per[name]["valu_floor_us"] = per[name]["flops"] / (FP32_VALU_BROADCAST_TFLOPS * 1e12) * 1e6
     sp_us = (per["up_pass"]["us"] + per["down_pass"]["us"]) / 2
     sp_bytes = (per["up_pass"]["bytes"] + per["down_pass"]["bytes"]) / 2
     sp_flops = (per["up_pass"]["flops"] + per["down_pass"]["flops"]) / 2
@@ -507,7 +509,7 @@ def main():
                         kernel=kernel_names["up_pass"], op="up_pass+down_pass (mean per launch)",
                         launches_per_step=2, us_per_launch=sp_us, algorithmic_bytes=sp_bytes,
                         hbm_floor_us=sp_bytes / (HBM_PEAK_GBS * 1e9) * 1e6,
-                        valu_floor_us=sp_flops / (FP32_VALU_UNPACKED_TFLOPS * 1e12) * 1e6,
+                        valu_floor_us=sp_flops / (FP32_VALU_BROADCAST_TFLOPS * 1e12) * 1e6,
                         note="by intensity (7-10 FLOP/B) the kernel sits on the ridge of the unpacked vector rate "
                              "(9.8 FLOP/B): both floors are given")
     else:
@@ -539,9 +541,9 @@ def main():
         cfg4_config, cfg4_res, _ = measure_cfg4(20, torch, D, W, dev, with_aux=False)
         out["aux"] = dict(cfg4=dict(config=cfg4_config, ops=cfg4_res,
                                     note="bound by the fp32 vector rate (57 FLOP per algorithmic byte): "
-                                         "frac_fp32_valu is against the published 157.3 TFLOP/s (packed), "
-                                         "frac_fp32_valu_unpacked against the 78.6 TFLOP/s reachable without "
-                                         "packed-fp32 instructions"))
+                                         "frac_fp32_valu is against the published 157.3 TFLOP/s, "
+                                         "frac_fp32_valu_broadcast against the 78.6 TFLOP/s of FMAs with a "
+                                         "DPP-broadcast or scalar operand, the form these kernels use"))
 
     if not args.no_cpu:
         from oracle import oracle as O

@@ -1,0 +1,181 @@
+// Measures, on the GPU it runs on, the two rates the product kernels are laid out around:
+//   * how fast a SIMD issues fp32 FMAs in the forms a kernel can give them -- three vector-register operands, a
+//     DPP-broadcast operand (v_fmac_f32_dpp .. row_newbcast), a scalar operand;
+//   * how fast a CU's LDS answers 4-, 8- and 16-byte reads.
+// The kernels keep the batch along the lanes and broadcast a diagonal's value to them; this probe shows what that
+// form costs against the plain one, and what feeding the plain form from LDS would need.
+// Built by the Makefile into ../lib/hw_rates; prints one line per measurement.  Every wave runs a fixed number of
+// iterations and the grid is one resident round of workgroups.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <vector>
+
+#define HW_CHECK(call)                                                                      \
+    do {                                                                                    \
+        const hipError_t e_ = (call);                                                       \
+        if (e_ != hipSuccess) {                                                             \
+            std::fprintf(stderr, "%s: %s\n", #call, hipGetErrorString(e_));                 \
+            return 1;                                                                       \
+        }                                                                                   \
+    } while (0)
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+// 16 independent running sums per lane, 64 FMAs per iteration
+template <int FORM>
+__global__ __launch_bounds__(256) void fma_kernel(float *out, long long *clk, int iters, float a, float sa)
+{
+    float acc[16];
+    for (int i = 0; i < 16; ++i) acc[i] = threadIdx.x * 0.001f + i;
+    const float x = a + threadIdx.x;
+    const long long c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                if (FORM == 0) asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[i]) : "v"(x), "v"(a));
+                if (FORM == 1)
+                    asm volatile("v_fmac_f32_dpp %0, %1, %2 row_newbcast:1 row_mask:0xf bank_mask:0xf"
+                                 : "+v"(acc[i]) : "v"(x), "v"(a));
+                if (FORM == 2) asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[i]) : "s"(sa), "v"(a));
+            }
+    }
+    const long long c1 = clock64(), w1 = wall_clock64();
+    float s = 0;
+    for (int i = 0; i < 16; ++i) s += acc[i];
+    out[blockIdx.x * 256 + threadIdx.x] = s;
+    if (threadIdx.x == 0) {
+        clk[2 * blockIdx.x] = c1 - c0;
+        clk[2 * blockIdx.x + 1] = w1 - w0;
+    }
+}
+
+// every lane reads 4 W bytes per instruction at consecutive addresses (conflict-free), 8 instructions per iteration
+template <int W>
+__global__ __launch_bounds__(256) void lds_kernel(float *out, long long *clk, int iters)
+{
+    __shared__ __attribute__((aligned(16))) float buf[8192];
+    for (int i = threadIdx.x; i < 8192; i += 256) buf[i] = i;
+    __syncthreads();
+    const unsigned base =
+        (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)buf + threadIdx.x * (W * 4);
+    float sum = 0.f;
+    const long long c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            if (W == 4) {
+                f4 v;
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(base), "n"(r * 4096));
+                asm volatile("s_waitcnt lgkmcnt(4)");
+                if (r == 7) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v)); sum += v.x; }
+            }
+            if (W == 2) {
+                f2 v;
+                asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(base), "n"(r * 2048));
+                asm volatile("s_waitcnt lgkmcnt(4)");
+                if (r == 7) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v)); sum += v.x; }
+            }
+            if (W == 1) {
+                float v;
+                asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(base), "n"(r * 1024));
+                asm volatile("s_waitcnt lgkmcnt(4)");
+                if (r == 7) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v)); sum += v; }
+            }
+        }
+    }
+    const long long c1 = clock64(), w1 = wall_clock64();
+    out[blockIdx.x * 256 + threadIdx.x] = sum;
+    if (threadIdx.x == 0) {
+        clk[2 * blockIdx.x] = c1 - c0;
+        clk[2 * blockIdx.x + 1] = w1 - w0;
+    }
+}
+
+struct Probe {
+    float *out = nullptr;
+    long long *clk = nullptr;
+    int cus = 0, wgs = 0;
+    hipEvent_t e0{}, e1{};
+    std::vector<long long> host;
+};
+
+// shader clock during the kernel: s_memtime ticks per tick of the constant 100 MHz clock, averaged over workgroups
+static int finish(Probe &p, float *ms, double *mhz)
+{
+    HW_CHECK(hipEventSynchronize(p.e1));
+    HW_CHECK(hipEventElapsedTime(ms, p.e0, p.e1));
+    HW_CHECK(hipMemcpy(p.host.data(), p.clk, (size_t)p.wgs * 16, hipMemcpyDeviceToHost));
+    double cs = 0, ws = 0;
+    for (int i = 0; i < p.wgs; ++i) { cs += (double)p.host[2 * i]; ws += (double)p.host[2 * i + 1]; }
+    *mhz = ws > 0 ? cs / ws * 100.0 : 0.0;
+    return 0;
+}
+
+template <int FORM>
+static int run_fma(Probe &p, const char *name)
+{
+    const int iters = 20000;
+    float ms = 0;
+    double mhz = 0;
+    for (int rep = 0; rep < 2; ++rep) {
+        HW_CHECK(hipEventRecord(p.e0));
+        hipLaunchKernelGGL(fma_kernel<FORM>, dim3(p.wgs), dim3(256), 0, 0, p.out, p.clk, iters, 1.0001f, 0.5f);
+        HW_CHECK(hipGetLastError());
+        HW_CHECK(hipEventRecord(p.e1));
+        if (finish(p, &ms, &mhz)) return 1;
+    }
+    const double flops = 2.0 * 64 * iters * 256.0 * p.wgs;
+    const double per_simd = (double)ms * 1e-3 * mhz * 1e6 / (64.0 * iters * (256.0 / 64.0) * p.wgs / (4.0 * p.cus));
+    std::printf("fma  %-34s %8.3f ms  %6.1f TFLOP/s  %.2f clocks per wave64 FMA per SIMD  shader clock %.0f MHz\n",
+                name, ms, flops / ms / 1e9, per_simd, mhz);
+    std::fflush(stdout);
+    return 0;
+}
+
+template <int W>
+static int run_lds(Probe &p, const char *name)
+{
+    const int iters = 20000;
+    float ms = 0;
+    double mhz = 0;
+    for (int rep = 0; rep < 2; ++rep) {
+        HW_CHECK(hipEventRecord(p.e0));
+        hipLaunchKernelGGL(lds_kernel<W>, dim3(p.wgs), dim3(256), 0, 0, p.out, p.clk, iters);
+        HW_CHECK(hipGetLastError());
+        HW_CHECK(hipEventRecord(p.e1));
+        if (finish(p, &ms, &mhz)) return 1;
+    }
+    const double bytes = 8.0 * iters * 256.0 * p.wgs * W * 4;
+    std::printf("lds  %-34s %8.3f ms  %6.1f B/clk/CU  shader clock %.0f MHz\n", name, ms,
+                bytes / ((double)ms * 1e-3) / p.cus / (mhz * 1e6), mhz);
+    std::fflush(stdout);
+    return 0;
+}
+
+int main()
+{
+    hipDeviceProp_t prop;
+    HW_CHECK(hipGetDeviceProperties(&prop, 0));
+    Probe p;
+    p.cus = prop.multiProcessorCount;
+    p.wgs = p.cus * 4;                       // 16 waves per CU: one resident round
+    p.host.resize((size_t)2 * p.wgs);
+    HW_CHECK(hipMalloc(&p.out, (size_t)p.wgs * 256 * 4));
+    HW_CHECK(hipMalloc(&p.clk, (size_t)p.wgs * 16));
+    HW_CHECK(hipEventCreate(&p.e0));
+    HW_CHECK(hipEventCreate(&p.e1));
+    std::printf("%s, %d CUs\n", prop.name, p.cus);
+    if (run_fma<0>(p, "v_fmac_f32 v, v, v")) return 1;
+    if (run_fma<1>(p, "v_fmac_f32_dpp row_newbcast")) return 1;
+    if (run_fma<2>(p, "v_fmac_f32 v, s, v")) return 1;
+    if (run_lds<4>(p, "ds_read_b128")) return 1;
+    if (run_lds<2>(p, "ds_read_b64")) return 1;
+    if (run_lds<1>(p, "ds_read_b32")) return 1;
+    HW_CHECK(hipFree(p.out));
+    HW_CHECK(hipFree(p.clk));
+    return 0;
+}
