@@ -265,6 +265,7 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     d->view.n_chunks_p = (int)cp.size();
     d->view.units_dev = reinterpret_cast<const Unit *>(base + un_at);
     d->view.n_units = (int)un.size();
+    d->view.pair_delta_max = pair_delta_max(cp, un);
     d->view.single_units_dev = reinterpret_cast<const Unit *>(base + us_at);
     auto walk_view = [&](const WalkPlan &p, size_t at) {
         return p.ok ? WalkView{reinterpret_cast<const int *>(base + at), p.ngroups, p.period, p.s0, p.k, p.lck, p.astep4}

@@ -1648,19 +1648,25 @@ constexpr int DD_BG = 4;           // batch columns per step
 // keeps as many running sums as a pair but is worked by 4 waves: three such
 // workgroups share a CU (registers allow 3 waves per SIMD, and the block the
 // sums are added in is kept just under a third of the CU's LDS).
-template <int NCH, int LC>
+// WIDE: a pair whose chunks start more than PAIR_NARROW_DELTA rows apart (window rows of a map wider than 128):
+// its band takes a third 16-byte piece per lane and column.
+template <int NCH, int LC, bool WIDE = false>
 struct DdShape {
     static_assert(NCH == 1 || LC <= CHUNK_MAX, "pairs are made of short chunks");
+    static_assert(NCH == 2 || !WIDE, "only pairs are wide");
     static constexpr bool LONG = LC > CHUNK_MAX;
     static constexpr int SPAN = LONG ? SP_CHUNK_MAX : CHUNK_MAX;    // shifts a chunk can have
-    static constexpr int NQ = NCH == 1 ? 4 : 6;                 // 64-row blocks of the band
-    static constexpr int PITCH = 64 * NQ + (LONG ? 16 : 8);     // staged rows per column: 264, 272 or 392
+    static constexpr int NQ = NCH == 1 ? 4 : WIDE ? 8 : 6;      // 64-row blocks of the band
+    static constexpr int NB = WIDE ? 3 : 2;                     // 16-byte pieces a lane holds per column
+    static constexpr int PITCH = 64 * NQ + (LONG ? 16 : 8);     // staged rows per column: 264, 272, 392 or 520
     static constexpr int WAVES = NCH == 2 ? 8 : 4;
     static constexpr int RED_PAD = LONG ? 4 : 8;              // a long chunk's sums then fit a third of a CU's LDS
     static constexpr int WAVE_FLOATS = 2 * DD_BG * PITCH + 4;   // two buffers + a slot idle lanes write to
     static constexpr int STAGE_FLOATS = WAVES * WAVE_FLOATS;
 };
-static_assert(DdShape<2, CHUNK_MAX>::PITCH >= DD_ROWS + PAIR_MAX_DELTA + CHUNK_MAX, "a pair's band must fit its buffer");
+static_assert(DdShape<2, CHUNK_MAX>::PITCH >= DD_ROWS + PAIR_NARROW_DELTA + CHUNK_MAX, "a pair's band must fit its buffer");
+static_assert(DdShape<2, CHUNK_MAX, true>::PITCH >= DD_ROWS + PAIR_MAX_DELTA + CHUNK_MAX, "a wide pair's band must fit its buffer");
+static_assert(DdShape<2, CHUNK_MAX>::NB == 2 && DdShape<2, CHUNK_MAX, true>::NB == 3 && DdShape<1, CHUNK_MAX>::NB == 2, "pieces per lane");
 static_assert(DdShape<1, SP_CHUNK_MAX>::PITCH >= DD_ROWS + 4 * ((4 + SP_CHUNK_MAX - 1 + 3) / 4) - 4,
               "a long chunk's last window must fit its buffer");
 
@@ -1672,22 +1678,22 @@ struct DdStage {
 
 template <int LC, int NCH>
 constexpr int dd_red_floats() { return 4 * 4 * (NCH * LC * 64 + DdShape<NCH, LC>::RED_PAD); }
-template <int LC, int NCH>
+template <int LC, int NCH, bool WIDE = false>
 constexpr int dd_lds_floats()
 {
-    return DdShape<NCH, LC>::STAGE_FLOATS > dd_red_floats<LC, NCH>() ? DdShape<NCH, LC>::STAGE_FLOATS
-                                                                     : dd_red_floats<LC, NCH>();
+    return DdShape<NCH, LC, WIDE>::STAGE_FLOATS > dd_red_floats<LC, NCH>() ? DdShape<NCH, LC, WIDE>::STAGE_FLOATS
+                                                                           : dd_red_floats<LC, NCH>();
 }
 
-template <int LC, int NCH, bool AVEC>
+template <int LC, int NCH, bool AVEC, bool WIDE = false>
 __device__ __forceinline__ void dd2dia_unit(
     float *lds, int row0, const Chunk *ck1, const Chunk *ck2, float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
     int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
     unsigned c_bytes)
 {
-    typedef DdShape<NCH, LC> S;
-    constexpr int PITCH = S::PITCH, WAVES = S::WAVES;
+    typedef DdShape<NCH, LC, WIDE> S;
+    constexpr int PITCH = S::PITCH, WAVES = S::WAVES, NB = S::NB;
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
     constexpr int RED_T = NCH * LC * 64 + S::RED_PAD;        // floats between the 4 rows a lane owns: keeps the
@@ -1748,8 +1754,9 @@ __device__ __forceinline__ void dd2dia_unit(
     }
 
     // The band of B travels as 16-byte pieces, a lane holding rows base + 4*lane
-    // .. + 3 and, where the band reaches that far, base + 256 + 4*lane .. + 3:
-    // two loads per column, whatever the alignment of base (a load instruction
+    // .. + 3 and, where the band reaches that far, base + 256 + 4*lane .. + 3
+    // (a wide pair: and base + 512 + 4*lane .. + 3):
+    // two (three) loads per column, whatever the alignment of base (a load instruction
     // occupies the memory pipeline equally long for 4 and for 16 bytes per
     // lane).  Rows of the band outside B need no care in general: they only
     // meet sums of slots that hold no matrix element and are never stored, and
@@ -1762,8 +1769,9 @@ __device__ __forceinline__ void dd2dia_unit(
     // which answers for the piece as a whole: those columns -- [0, rare_lo) and
     // [rare_hi, batch) -- stay out of the pipelined loop and are worked row by
     // row by wave 0 before it (see below).
-    const int nquad = (need + 3) / 4;                     // pieces per column that are ever read, 66 .. 98
+    const int nquad = (need + 3) / 4;                     // pieces per column that are ever read, 66 .. 130
     const bool tail = lane < nquad - 64;
+    const bool tail2 = lane < nquad - 128;                // a wide pair's third piece
     const unsigned vb_off0 = (unsigned)(base + 4 * lane) * 4u;
     const long long b_floats = (long long)(batch - 1) * ldb + w;
     // column c's band starts c*ldb + base floats into the allocation and is 4*nquad floats long
@@ -1804,7 +1812,7 @@ __device__ __forceinline__ void dd2dia_unit(
     // B in flight: per column, rows base + 4*lane .. + 3 and base + 256 + 4*lane .. + 3 of the band.  One set
     // serves the current and the next group: column i of the next group is requested after column i of the
     // current one has gone to LDS.
-    float4 bq[DD_BG][2];
+    float4 bq[DD_BG][NB];
     // requests column i of group g: B rows into bq, A rows into st.a
     const unsigned rare_span = (unsigned)(rare_hi - rare_lo);
     auto issue_col = [&](int g, int i, DdStage &st) {
@@ -1816,6 +1824,8 @@ __device__ __forceinline__ void dd2dia_unit(
         const unsigned v0 = vb_off0 + colb;
         bq[i][0] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, v0, 0, 0));
         bq[i][1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, tail ? v0 + 1024u : OOB_OFFSET, 0, 0));
+        if constexpr (NB == 3)
+            bq[i][2] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, tail2 ? v0 + 2048u : OOB_OFFSET, 0, 0));
         const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, live ? a_bytes : 0u);
         const unsigned cola = (unsigned)col * lda4;
         if (AVEC) {
@@ -1836,6 +1846,8 @@ __device__ __forceinline__ void dd2dia_unit(
         *reinterpret_cast<float4 *>(buf + i * PITCH + 4 * lane) = bq[i][0];
         // lanes past the band's end drop their (zero) piece in the spare slot
         *reinterpret_cast<float4 *>(tail ? buf + i * PITCH + 256 + 4 * lane : mybuf + 2 * DD_BG * PITCH) = bq[i][1];
+        if constexpr (NB == 3)
+            *reinterpret_cast<float4 *>(tail2 ? buf + i * PITCH + 512 + 4 * lane : mybuf + 2 * DD_BG * PITCH) = bq[i][2];
         wave_lds_fence();
     };
     struct Windows { float w[NCH][WQ * 4]; };
@@ -1987,7 +1999,7 @@ __device__ __forceinline__ void dd2dia_unit(
 // PAIRS = false: every unit is a single chunk, 4 waves per workgroup.
 // PAIRS = true: 8 waves per workgroup; a workgroup whose unit is a single
 // chunk retires its upper four waves at once.
-template <int LC, bool AVEC, bool PAIRS>
+template <int LC, bool AVEC, bool PAIRS, bool WIDE = false>
 __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     const Chunk *__restrict__ chunks, const Unit *__restrict__ units, int nunits,
     float *__restrict__ C, int stride,
@@ -1996,8 +2008,9 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     unsigned c_bytes)
 {
     constexpr int NCH_MAX = PAIRS ? 2 : 1;
-    constexpr int LDS_FLOATS = dd_lds_floats<LC, NCH_MAX>() > dd_lds_floats<LC, 1>() ? dd_lds_floats<LC, NCH_MAX>()
-                                                                                     : dd_lds_floats<LC, 1>();
+    static_assert(PAIRS || !WIDE, "only pairs are wide");
+    constexpr int LDS_FLOATS = dd_lds_floats<LC, NCH_MAX, WIDE>() > dd_lds_floats<LC, 1>() ? dd_lds_floats<LC, NCH_MAX, WIDE>()
+                                                                                           : dd_lds_floats<LC, 1>();
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
     const int rowtile = tile / nunits;
@@ -2007,8 +2020,8 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     const int row0 = rowtile * DD_ROWS;
     if constexpr (PAIRS) {
         if (c2 >= 0) {
-            dd2dia_unit<LC, 2, AVEC>(lds, row0, chunks + c1, chunks + c2, C, stride, A, lda, B, ldb, h, w, batch,
-                                     alpha, beta, a_bytes, b_bytes, c_bytes);
+            dd2dia_unit<LC, 2, AVEC, WIDE>(lds, row0, chunks + c1, chunks + c2, C, stride, A, lda, B, ldb, h, w, batch,
+                                           alpha, beta, a_bytes, b_bytes, c_bytes);
             return;
         }
     }
@@ -2325,6 +2338,7 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     // loads and LDS traffic per FMA.  (16-byte loads of A only, as for pairs.)
     const bool long_chunks = C.max_len_n > CHUNK_MAX && a_vec;
     const bool pairs = use_units && !long_chunks;
+    const bool wide = pairs && C.pair_delta_max > PAIR_NARROW_DELTA;      // some pair needs the 520-row band
     const Unit *units = pairs ? C.units_dev : C.single_units_dev;      // the single units count 0, 1, 2, ...
     const int nunits = long_chunks ? C.n_chunks_n : pairs ? C.n_units : C.n_chunks_p;
     const Chunk *table = long_chunks ? C.chunks_n_dev : C.chunks_p_dev;
@@ -2336,7 +2350,9 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
                        a_bytes, b_bytes, c_bytes
 #define CUVDIA_DD_LAUNCH(L)                                                                              \
     case L:                                                                                              \
-        if (pairs) {                                                                                     \
+        if (wide) {                                                                                      \
+            hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, true, true>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
+        } else if (pairs) {                                                                              \
             hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, true>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
         } else {                                                                                         \
             if (a_vec) hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);  \

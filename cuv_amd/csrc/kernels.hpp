@@ -32,6 +32,7 @@ struct DiaView {
     int max_len_p;
     const Unit *units_dev;       // units of the normal table (dense x dense^T projection)
     int n_units;
+    int pair_delta_max;          // largest distance between the first shifts of a pair (0: no pairs)
     const Unit *single_units_dev;   // one unit per chunk of the normal table, in table order
 };
 

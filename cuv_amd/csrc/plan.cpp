@@ -125,6 +125,14 @@ std::vector<Unit> plan_units(const std::vector<Chunk> &chunks)
     return out;
 }
 
+int pair_delta_max(const std::vector<Chunk> &chunks, const std::vector<Unit> &units)
+{
+    int m = 0;
+    for (const Unit &u : units)
+        if (u.c2 >= 0) m = std::max(m, chunks[u.c2].s0 - chunks[u.c1].s0);
+    return m;
+}
+
 long long count_valid(const int *offsets, int nd, int h, int w, int rf)
 {
     long long total = 0;

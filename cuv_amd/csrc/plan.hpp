@@ -54,7 +54,10 @@ std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, int 
 // chunks of the normal table whose first shifts differ by a multiple of 4 of
 // at most PAIR_MAX_DELTA rows.  A wave serves both chunks of a pair from one
 // staged band of the second operand and one copy of the first operand's rows.
-constexpr int PAIR_MAX_DELTA = 128;
+// Up to PAIR_NARROW_DELTA rows apart the band fits two 16-byte pieces per lane
+// and column; a table with a wider pair runs the kernel that takes three.
+constexpr int PAIR_MAX_DELTA = 256;
+constexpr int PAIR_NARROW_DELTA = 128;
 struct Unit {
     int c1;                 // chunk index
     int c2;                 // second chunk index, or -1
@@ -62,6 +65,8 @@ struct Unit {
 // Greedy over the table in shift order: chunk c pairs with c + 1 when their
 // shifts allow it.
 std::vector<Unit> plan_units(const std::vector<Chunk> &chunks);
+// The largest distance between the first shifts of a pair (0 without pairs).
+int pair_delta_max(const std::vector<Chunk> &chunks, const std::vector<Unit> &units);
 
 // Number of matrix elements stored (slots the reference host loops touch):
 // sum over diagonals of min(h - rf*max(0,-k), rf*(w - max(0,k))), clamped at 0

@@ -104,11 +104,19 @@ SHAPES = [
     (130, 130, [1], 1, 1),
     (64, 64, [0], 1, 64),
     (700, 650, [d * 25 + e for d in range(-2, 3) for e in range(-2, 3)], 1, 96),
-    # chunk pairs of the dense x dense^T projection (first shifts a multiple of 4, at most 128, apart)
+    # chunk pairs of the dense x dense^T projection (first shifts a multiple of 4, at most 128 here, apart)
     (512, 512, [dy * 128 + dx for dy in range(-1, 2) for dx in range(-3, 4)], 1, 40),
     (300, 300, list(range(-8, -1)) + list(range(0, 8)) + [100, 101], 1, 7),
     (260, 1000, [-200, -199, -198, -72, -71, 56, 57, 58, 59, 700], 1, 131),
     (1024, 768, [dy * 64 + dx for dy in range(-2, 3) for dx in range(0, 8)], 1, 1),
+    # wide pairs (first shifts more than 128 and at most 256 apart): 256 apart on a square and on rectangular
+    # matrices both ways, 192 apart, a table that mixes a narrow pair, a wide pair and a single, and one whose
+    # rows end inside the last tile
+    (1536, 1536, [dy * 256 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 1, 72),
+    (1024, 1800, [dy * 256 + dx for dy in range(-2, 3) for dx in range(-2, 3)], 1, 33),
+    (1800, 1024, [dy * 256 + dx for dy in range(-2, 2) for dx in range(0, 7)], 1, 130),
+    (900, 900, [dy * 192 + dx for dy in range(-2, 3) for dx in range(-3, 4)], 1, 17),
+    (1111, 1300, [0, 1, 2, 64, 65, 66, 320, 321, 576, 577, 578, 1000], 1, 41),
     # window rows a multiple of the 64-row tile apart: square, rectangular both ways, a window with
     # missing rows, ragged batch
     (2048, 2048, [dy * 64 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 1, 70),
