@@ -382,6 +382,7 @@ constexpr int SP_AVALS = SP_ADIAGS * SP_ROWS;   // diagonal values per workgroup
 constexpr int SP_DUMP = SP_XFLOATS + SP_AVALS;  // where idle lanes write
 constexpr int SP_STAGE_FLOATS = SP_DUMP + 4;
 constexpr int SP_WALK_WGS = 512;       // workgroups a walking launch aims at (two per CU)
+constexpr int SP_RENUMBER_MIN_TILES = 1024;   // launches of more than two rounds renumber the row tiles of a window table
 constexpr int SP_WALK_MIN_WGS = 384;   // below this the chip is not filled: the tile-by-tile kernels serve
 constexpr int SP_MAX_CHUNKS = 256;   // chunk-table entries a wave can keep in registers (4 sets of 64)
 
@@ -1236,7 +1237,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, int col_group, unsigned a_bytes,
-    int s_min, int s_max, SpEpilogue ep)
+    int s_min, int s_max, int period_tiles, SpEpilogue ep)
 {
     static_assert(3 * SP_DSTAGE_FLOATS >= 2 * SP_STAGE_FLOATS, "the two bodies share one LDS block");
     __shared__ __attribute__((aligned(16))) float lds3[3][SP_DSTAGE_FLOATS];
@@ -1256,6 +1257,17 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
         const int width = min(col_group, col_tiles - g * col_group);
         rowtile = in / width;
         coltile = g * col_group + (in - rowtile * width);
+    }
+    // A window table (window rows period_tiles tiles apart, period_tiles > 1): the tile one period down reads,
+    // for window row dy, the dense rows this tile reads for dy + 1.  Inside every block of 16 periods the row
+    // tiles are renumbered period-major -- position 16 r + m holds tile m * period_tiles + r -- so that the row
+    // tiles an XCD holds at a time are 16 periods of one residue instead of 16 neighbours: tiles that run side
+    // by side then ask for the block a neighbour in the walk fetched a chunk earlier, and find it in the L2.
+    if (period_tiles > 1) {
+        const int blk_tiles = 16 * period_tiles;
+        const int blk = rowtile / blk_tiles, i = rowtile - blk * blk_tiles;
+        const int row_tiles = (int)(gridDim.x / (unsigned)col_tiles);
+        if ((blk + 1) * blk_tiles <= row_tiles) rowtile = blk * blk_tiles + (i & 15) * period_tiles + (i >> 4);
     }
     const int row0 = rowtile * SP_ROWS;
     const int col0 = coltile * SP_COLS;
@@ -1996,6 +2008,14 @@ __device__ __forceinline__ void dd2dia_unit(
     }
 }
 
+// Shape of the blocks the projection's tiles are numbered in (see the kernel): units per block and row tiles per
+// block, 64 positions or nearly.
+constexpr int DD_BLOCKED_MIN_TILES = 1024;   // launches of more than a few rounds number their tiles in blocks
+struct DdBlock {
+    __host__ __device__ static int units(int nunits) { return nunits < 16 ? nunits : 16; }
+    __host__ __device__ static int rows(int nunits) { return 64 / units(nunits); }
+};
+
 // PAIRS = false: every unit is a single chunk, 4 waves per workgroup.
 // PAIRS = true: 8 waves per workgroup; a workgroup whose unit is a single
 // chunk retires its upper four waves at once.
@@ -2005,7 +2025,7 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
     int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
-    unsigned c_bytes)
+    unsigned c_bytes, int blocked)
 {
     constexpr int NCH_MAX = PAIRS ? 2 : 1;
     static_assert(PAIRS || !WIDE, "only pairs are wide");
@@ -2013,9 +2033,33 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
                                                                                            : dd_lds_floats<LC, 1>();
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int rowtile = tile / nunits;
+    // Tiles are numbered block by block: a block is DdBlock::rows(nunits) neighbouring row tiles x up to 16
+    // units, the unit running fastest -- the 64 workgroups an XCD receives together.  The units of a row tile
+    // share its 256 rows of A; the unit one window row up of the row tile one period down reads the same band of
+    // B: a block of 4 x 16 touches 4 copies of A's rows and about 19 bands where 64 units of one row tile would
+    // touch 64 bands.  Positions past the last row tile or unit do nothing.
+    // (Launches of one or two rounds keep the plain numbering, unit fastest: every workgroup is resident at
+    // once or nearly, and the index arithmetic below -- integer divisions -- would cost them half a microsecond.)
+    int rowtile, unit;
+    if (!blocked) {
+        rowtile = tile / nunits;
+        unit = tile - rowtile * nunits;
+    } else {
+    const int ub = DdBlock::units(nunits), rb = DdBlock::rows(nunits), nub = (nunits + ub - 1) / ub;
+    const int per_rblk = nub * rb * ub;
+    const int rblk = tile / per_rblk, rem = tile - rblk * per_rblk;
+    // Workgroup ids go to the XCDs round-robin by spans of 64: with the unit blocks of a row block always in the
+    // same order an XCD would meet the same unit block again and again -- and the unit blocks of a multi-channel
+    // table differ in how many of their units lie inside the operand.  The order is therefore turned by one
+    // place every time the spans have gone round the XCDs.
+    const int turn = rblk / (nub < 8 ? 8 / nub : 1);
+    const int ublk = (rem / (rb * ub) + turn) % nub, pos = rem % (rb * ub);
+    rowtile = rblk * rb + pos / ub;
+    unit = ublk * ub + pos % ub;
+    }
+    if (rowtile * DD_ROWS >= h || unit >= nunits) return;
     typedef const Unit __attribute__((address_space(4))) *sc_unit_ptr;
-    const sc_unit_ptr u = (sc_unit_ptr)units + (tile - rowtile * nunits);
+    const sc_unit_ptr u = (sc_unit_ptr)units + unit;
     const int c1 = u->c1, c2 = u->c2;
     const int row0 = rowtile * DD_ROWS;
     if constexpr (PAIRS) {
@@ -2086,6 +2130,7 @@ struct SpLaunch {
     int col_tiles, col_group;
     unsigned a_bytes;
     int s_min, s_max;
+    int period_tiles;           // window tables: tiles between window rows (0: no renumbering of the row tiles)
     SpEpilogue ep;
     dim3 grid;
     hipStream_t stream;
@@ -2115,7 +2160,7 @@ hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
 // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
 // at the sizes this path is measured on.
 #define CUVDIA_SPMM_ARGS L.chunks, L.nchunks, L.vals, L.stride, L.ashift, L.B, L.ldb, L.dst, L.ldd, L.n_out, L.n_in, \
-                         L.batch, L.alpha, L.beta, L.col_tiles, L.col_group, L.a_bytes, L.s_min, L.s_max, L.ep
+                         L.batch, L.alpha, L.beta, L.col_tiles, L.col_group, L.a_bytes, L.s_min, L.s_max, L.period_tiles, L.ep
 #define CUVDIA_SPMM_LAUNCH(K)                                                                                         \
     case K:                                                                                                           \
         if (L.nchunks <= 64 && !fused)                                                                                \
@@ -2238,7 +2283,10 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
                      trans ? A.n_chunks_t : A.n_chunks_n,
                      vals, A.stride, trans ? 1 : 0, B, ldb, dst, ldd, n_out, n_in, batch, alpha, beta,
                      (int)col_tiles, col_group, (unsigned)((long long)A.nd * A.stride * 4),
-                     trans ? A.s_min_t : A.s_min_n, trans ? A.s_max_t : A.s_max_n, ep,
+                     trans ? A.s_min_t : A.s_min_n, trans ? A.s_max_t : A.s_max_n,
+                     (wk.tab_dev != nullptr && wk.period % SP_ROWS == 0 && row_tiles * col_tiles > SP_RENUMBER_MIN_TILES)
+                         ? wk.period / SP_ROWS : 0,
+                     ep,
                      dim3((unsigned)(row_tiles * col_tiles)), stream, lck};
     if (lck <= 5) return spmm_tiled_launch_1_5(L);
     if (lck <= 9) return spmm_tiled_launch_6_9(L);
@@ -2343,11 +2391,14 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     const int nunits = long_chunks ? C.n_chunks_n : pairs ? C.n_units : C.n_chunks_p;
     const Chunk *table = long_chunks ? C.chunks_n_dev : C.chunks_p_dev;
     const int lc = long_chunks ? C.max_len_n : C.max_len_p;
-    const long long blocks = row_tiles * nunits;
+    const int ub = DdBlock::units(nunits), rb = DdBlock::rows(nunits);
+    const int blocked = row_tiles * nunits > DD_BLOCKED_MIN_TILES ? 1 : 0;
+    const long long blocks = blocked ? ((row_tiles + rb - 1) / rb) * ((nunits + ub - 1) / ub) * (long long)(rb * ub)
+                                     : row_tiles * nunits;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks);
 #define CUVDIA_DD_ARGS table, units, nunits, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
-                       a_bytes, b_bytes, c_bytes
+                       a_bytes, b_bytes, c_bytes, blocked
 #define CUVDIA_DD_LAUNCH(L)                                                                              \
     case L:                                                                                              \
         if (wide) {                                                                                      \
