@@ -492,8 +492,8 @@ def main():
     for name in per:
         per[name]["kernel"] = kernel_names[name]
         per[name]["traffic"] = traffic[name]
-        # what the two ceilings allow: the algorithmic bytes at the HBM peak, and the FLOPs at the vector rate
-        # without packed-fp32 instructions
+        # what the two ceilings allow: the algorithmic bytes at the HBM peak, and the FLOPs at the rate of
+        # broadcast-operand FMAs (the products' form; the projection's plain FMAs could run at twice that)
         per[name]["hbm_floor_us"] = per[name]["bytes"] / (HBM_PEAK_GBS * 1e9) * 1e6
         per[name]["valu_floor_us"] = per[name]["flops"] / (FP32_VALU_BROADCAST_TFLOPS * 1e12) * 1e6
     sp_us = (per["up_pass"]["us"] + per["down_pass"]["us"]) / 2
@@ -510,8 +510,8 @@ def main():
                         launches_per_step=2, us_per_launch=sp_us, algorithmic_bytes=sp_bytes,
                         hbm_floor_us=sp_bytes / (HBM_PEAK_GBS * 1e9) * 1e6,
                         valu_floor_us=sp_flops / (FP32_VALU_BROADCAST_TFLOPS * 1e12) * 1e6,
-                        note="by intensity (7-10 FLOP/B) the kernel sits on the ridge of the unpacked vector rate "
-                             "(9.8 FLOP/B): both floors are given")
+                        note="by intensity (7-10 FLOP/B) the kernel sits on the ridge of the rate its broadcast-operand "
+                             "FMAs issue at (78.6 TFLOP/s / 8 TB/s = 9.8 FLOP/B): both floors are given")
     else:
         g = per["weight_gradient"]
         roofline = dict(bound="hbm", achieved=g["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=g["gbs"] / HBM_PEAK_GBS,

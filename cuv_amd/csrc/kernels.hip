@@ -1697,7 +1697,13 @@ constexpr int dd_lds_floats()
                                                                            : dd_red_floats<LC, NCH>();
 }
 
-template <int LC, int NCH, bool AVEC, bool WIDE = false>
+// Rows of a tile.  A launch of single chunks only (no pairs) cuts its tiles 8 (long chunks: 16) rows short of
+// 256: the band of B a tile needs -- its rows plus the chunk's span -- then fits the 256 rows that one 16-byte
+// piece per lane covers, and a column costs two load instructions (B, A) instead of three.
+template <int LC>
+constexpr int dd_short_rows() { return DD_ROWS - (LC > CHUNK_MAX ? 16 : 8); }
+
+template <int LC, int NCH, bool AVEC, bool WIDE = false, bool SHORT = false>
 __device__ __forceinline__ void dd2dia_unit(
     float *lds, int row0, const Chunk *ck1, const Chunk *ck2, float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
@@ -1705,7 +1711,10 @@ __device__ __forceinline__ void dd2dia_unit(
     unsigned c_bytes)
 {
     typedef DdShape<NCH, LC, WIDE> S;
-    constexpr int PITCH = S::PITCH, WAVES = S::WAVES, NB = S::NB;
+    static_assert(!SHORT || NCH == 1, "only launches of single chunks use short tiles");
+    constexpr int TR = SHORT ? dd_short_rows<LC>() : DD_ROWS;             // rows of the tile
+    constexpr int PITCH = S::PITCH, WAVES = S::WAVES, NB = SHORT ? 1 : S::NB;
+    static_assert(!SHORT || TR + S::SPAN <= 256 || (S::LONG && TR + 16 <= 256), "a short tile's band is one piece per lane");
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
     constexpr int RED_T = NCH * LC * 64 + S::RED_PAD;        // floats between the 4 rows a lane owns: keeps the
@@ -1731,7 +1740,7 @@ __device__ __forceinline__ void dd2dia_unit(
         }
     }
     const int delta = NCH == 2 ? s0[NCH - 1] - s0[0] : 0;      // rows between the two windows
-    const int need = DD_ROWS + delta + S::SPAN;                 // staged rows that are ever read
+    const int need = TR + delta + S::SPAN;                      // staged rows that are ever read
     const int base = row0 + s0[0];                              // first staged row of B
     // Every slot of the unit pairs row i with row i + s0 + j of B: with the
     // whole band outside B the unit stores no matrix element, and there is
@@ -1747,7 +1756,7 @@ __device__ __forceinline__ void dd2dia_unit(
         const int sl = slots[n][j];
         const int o = row0 + 64 * wave + lane;
         const int in = o + s0[n] + j;
-        const bool ok = (wave < 4) & (sl >= 0) & (o < h) & (in >= 0) & (in < w);
+        const bool ok = (wave < 4) & (sl >= 0) & (o < h) & (in >= 0) & (in < w) & (64 * wave + lane < TR);
         return ok ? ((unsigned)sl * (unsigned)stride + (unsigned)o) * 4u : OOB_OFFSET;
     };
     float cpre[NCH][LC];
@@ -1796,10 +1805,10 @@ __device__ __forceinline__ void dd2dia_unit(
     }
     unsigned a_off[4];
     if (AVEC) {
-        a_off[0] = (myrow + 3 < h) ? (unsigned)myrow * 4u : OOB_OFFSET;
+        a_off[0] = ((myrow + 3 < h) & (4 * lane + 3 < TR)) ? (unsigned)myrow * 4u : OOB_OFFSET;
     } else {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) a_off[t] = (myrow + t < h) ? (unsigned)(myrow + t) * 4u : OOB_OFFSET;
+        for (int t = 0; t < 4; ++t) a_off[t] = ((myrow + t < h) & (4 * lane + t < TR)) ? (unsigned)(myrow + t) * 4u : OOB_OFFSET;
     }
     // Column strides in bytes, pinned to scalar registers: they feed the loads'
     // scalar offsets, and left alone the compiler derives them from a vector
@@ -1835,7 +1844,8 @@ __device__ __forceinline__ void dd2dia_unit(
         const unsigned colb = (unsigned)col * ldb4;
         const unsigned v0 = vb_off0 + colb;
         bq[i][0] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, v0, 0, 0));
-        bq[i][1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, tail ? v0 + 1024u : OOB_OFFSET, 0, 0));
+        if constexpr (NB >= 2)
+            bq[i][1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, tail ? v0 + 1024u : OOB_OFFSET, 0, 0));
         if constexpr (NB == 3)
             bq[i][2] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(br, tail2 ? v0 + 2048u : OOB_OFFSET, 0, 0));
         const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, live ? a_bytes : 0u);
@@ -1857,7 +1867,8 @@ __device__ __forceinline__ void dd2dia_unit(
         float *buf = mybuf + par * (DD_BG * PITCH);
         *reinterpret_cast<float4 *>(buf + i * PITCH + 4 * lane) = bq[i][0];
         // lanes past the band's end drop their (zero) piece in the spare slot
-        *reinterpret_cast<float4 *>(tail ? buf + i * PITCH + 256 + 4 * lane : mybuf + 2 * DD_BG * PITCH) = bq[i][1];
+        if constexpr (NB >= 2)
+            *reinterpret_cast<float4 *>(tail ? buf + i * PITCH + 256 + 4 * lane : mybuf + 2 * DD_BG * PITCH) = bq[i][1];
         if constexpr (NB == 3)
             *reinterpret_cast<float4 *>(tail2 ? buf + i * PITCH + 512 + 4 * lane : mybuf + 2 * DD_BG * PITCH) = bq[i][2];
         wave_lds_fence();
@@ -1944,7 +1955,7 @@ __device__ __forceinline__ void dd2dia_unit(
 #pragma unroll
             for (int t = 0; t < 4; ++t)
                 a[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    ar, (myrow + t < h) ? (unsigned)(myrow + t) * 4u + cola : OOB_OFFSET, 0, 0));
+                    ar, ((myrow + t < h) & (4 * lane + t < TR)) ? (unsigned)(myrow + t) * 4u + cola : OOB_OFFSET, 0, 0));
             fmas(a, win);
         }
     }
@@ -2057,11 +2068,12 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     rowtile = rblk * rb + pos / ub;
     unit = ublk * ub + pos % ub;
     }
-    if (rowtile * DD_ROWS >= h || unit >= nunits) return;
+    constexpr int TR = PAIRS ? DD_ROWS : dd_short_rows<LC>();        // rows of a tile
+    if (rowtile * TR >= h || unit >= nunits) return;
     typedef const Unit __attribute__((address_space(4))) *sc_unit_ptr;
     const sc_unit_ptr u = (sc_unit_ptr)units + unit;
     const int c1 = u->c1, c2 = u->c2;
-    const int row0 = rowtile * DD_ROWS;
+    const int row0 = rowtile * TR;
     if constexpr (PAIRS) {
         if (c2 >= 0) {
             dd2dia_unit<LC, 2, AVEC, WIDE>(lds, row0, chunks + c1, chunks + c2, C, stride, A, lda, B, ldb, h, w, batch,
@@ -2070,7 +2082,7 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
         }
     }
     if (PAIRS && threadIdx.x >= 256) return;
-    dd2dia_unit<LC, 1, AVEC>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
+    dd2dia_unit<LC, 1, AVEC, false, !PAIRS>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
                              alpha, beta, a_bytes, b_bytes, c_bytes);
 }
 
@@ -2368,7 +2380,6 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream)
 {
-    const long long row_tiles = (C.h + DD_ROWS - 1) / DD_ROWS;
     // 16-byte loads of A need an aligned base and leading dimension and whole
     // groups of 4 rows; row tiles start at multiples of 256 and lanes at
     // multiples of 4 rows.
@@ -2391,6 +2402,8 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     const int nunits = long_chunks ? C.n_chunks_n : pairs ? C.n_units : C.n_chunks_p;
     const Chunk *table = long_chunks ? C.chunks_n_dev : C.chunks_p_dev;
     const int lc = long_chunks ? C.max_len_n : C.max_len_p;
+    const int tile_rows = pairs ? DD_ROWS : lc > CHUNK_MAX ? dd_short_rows<SP_CHUNK_MAX>() : dd_short_rows<CHUNK_MAX>();
+    const long long row_tiles = (C.h + tile_rows - 1) / tile_rows;
     const int ub = DdBlock::units(nunits), rb = DdBlock::rows(nunits);
     const int blocked = row_tiles * nunits > DD_BLOCKED_MIN_TILES ? 1 : 0;
     const long long blocks = blocked ? ((row_tiles + rb - 1) / rb) * ((nunits + ub - 1) / ub) * (long long)(rb * ub)
