@@ -47,6 +47,7 @@ def lib():
     L.cuvdia_plan_chunks.argtypes = [ip, c_int, c_int, ip, ip, ip, c_int]
     L.cuvdia_plan_chunks_max.argtypes = [ip, c_int, c_int, c_int, ip, ip, ip, c_int]
     L.cuvdia_plan_units.argtypes = [ip, c_int, ip, ip, c_int]
+    L.cuvdia_plan_walk.argtypes = [ip, c_int, c_int, c_int, ip, ip, ip, ip]
     L.cuvdia_desc_create.argtypes = [ctypes.POINTER(c_vp), ip, c_int, c_int, c_int, c_int, c_int]
     L.cuvdia_desc_destroy.argtypes = [c_vp]
     L.cuvdia_desc_info.argtypes = [c_vp, ip, ip, ctypes.POINTER(c_ll)]
@@ -68,7 +69,7 @@ def lib():
                  "cuvdia_desc_info", "cuvdia_spmm_f32", "cuvdia_dd2dia_f32", "cuvdia_spmm_offsets_f32",
                  "cuvdia_dd2dia_offsets_f32", "cuvdia_cache_clear", "cuvdia_spmm_bias_act_f32",
                  "cuvdia_spmm_layer_f32", "cuvdia_learn_step_weight_decay_f32", "cuvdia_avg_diagonals_f32",
-                 "cuvdia_plan_units", "cuvdia_learn_step_weight_decay_momentum_f32", "cuvdia_plan_chunks_max",
+                 "cuvdia_plan_units", "cuvdia_plan_walk", "cuvdia_learn_step_weight_decay_momentum_f32", "cuvdia_plan_chunks_max",
                  "cuvdia_spmm_offsets_noalloc_f32"):
         getattr(L, name).restype = c_int
     _lib = L

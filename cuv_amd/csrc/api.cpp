@@ -154,6 +154,25 @@ int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
     return cuvdia_plan_chunks_max(offsets_host, nd, transposed, CHUNK_MAX, s0, len, slot, cap);
 }
 
+int cuvdia_plan_walk(const int *offsets_host, int nd, int stride, int transposed,
+                     int *period, int *k, int *ngroups, int *lck)
+{
+    if (!offsets_host || nd < 1 || stride < 1) return CUVDIA_EINVAL;
+    WalkPlan wp;
+    try {
+        plan_walk(plan_chunks(offsets_host, nd, transposed != 0, SP_CHUNK_MAX), stride, transposed != 0, wp);
+    } catch (const std::bad_alloc &) {
+        return CUVDIA_ENOMEM;
+    }
+    if (!wp.ok) return 0;
+    if (period) *period = wp.period;
+    if (k) *k = wp.k;
+    if (ngroups) *ngroups = wp.ngroups;
+    if (lck) *lck = wp.lck;
+    const int rows = spmm_walk_tile_rows(wp.lck, wp.k, wp.s0);
+    return rows > 0 && wp.period % rows == 0 ? 2 : 1;
+}
+
 int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap)
 {
     if (!offsets_host || nd < 1) return CUVDIA_EINVAL;

@@ -61,6 +61,9 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
 // dense rows once for all the window rows that read it.  `walk`: 0 -- that
 // choice is made by size; 1 -- the walking kernel or hipErrorNotSupported;
 // -1 -- never the walking kernel.  *walked (if not null) tells which ran.
+// Output rows per tile of the walking kernel's instantiation for a window of k rows of lck diagonals whose first
+// shift is s0; 0 when there is none.
+int spmm_walk_tile_rows(int lck, int k, int s0);
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, SpEpilogue ep, hipStream_t stream,

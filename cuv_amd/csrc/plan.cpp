@@ -79,7 +79,7 @@ void plan_walk(const std::vector<Chunk> &chunks, int stride, bool transposed, Wa
     // window rows: the leading shifts 0, period, 2 period, ...; then whole groups of the same k rows
     int k = 1;
     while (k < n && (long long)chunks[k].s0 - chunks[0].s0 == (long long)k * period) ++k;
-    if (n % k != 0) return;
+    if (k < 2 || n % k != 0) return;                 // a window has at least two rows
     const int ngroups = n / k;
     std::vector<int> group_rows(ngroups), aoff4(n);
     for (int g = 0; g < ngroups; ++g) {

@@ -111,6 +111,21 @@ int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
  * the block list built in src/cuv/matrix_ops/densedense_to_sparse.cu:123-171. */
 int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap);
 
+/* Pure host function: is the offset table a *window table* -- k window rows of
+ * lck consecutive offsets, `period` rows apart, repeated for every one of
+ * ngroups groups (channel shifts); the pattern filter_factory builds
+ * (src/cuv/basics/filter_factory.hpp:43-91) -- and does the walking product
+ * kernel serve it?  transposed selects the table of the transposed product.
+ * Writes period, k, ngroups and lck (each pointer may be NULL) when the answer
+ * is not 0.  Returns 0: no window table; 1: a window table that the products
+ * walk tile by tile (with their row tiles numbered period-major on launches of
+ * many rounds); 2: a window table with a walking kernel (centred 3x3, 5x5 or
+ * 7x7 window, period a multiple of 64: the kernel the automatic choice takes
+ * on products of many tiles whose row counts are multiples of 64); negative:
+ * an error.  No counterpart in the reference. */
+int cuvdia_plan_walk(const int *offsets_host, int nd, int stride, int transposed,
+                     int *period, int *k, int *ngroups, int *lck);
+
 /* dst = beta*dst + alpha*op(A)*B for a batch of dense columns.
  * Replaces prod<float,dev_memory_space,column_major>(dst, dia A, B, transA,
  * 'n', factAB, factC) (src/cuv/matrix_ops/spmv.cu:221-247), the spmv it

@@ -217,3 +217,48 @@ def test_dia_file_round_trip(tmp_path):
         io.check_fields(dict(f, m_vec=f["m_vec"][:-1]))
     with pytest.raises(ValueError):
         io.check_fields({k: v for k, v in f.items() if k != "m_offsets"})
+
+
+def _walk(offs, stride, transposed=0):
+    from cuv_amd import _lib
+    L = _lib.lib()
+    ip = ctypes.POINTER(ctypes.c_int)
+    offs = np.ascontiguousarray(offs, np.int32)
+    out = [ctypes.c_int(-1) for _ in range(4)]
+    rc = L.cuvdia_plan_walk(offs.ctypes.data_as(ip), offs.size, stride, transposed, *[ctypes.byref(o) for o in out])
+    return rc, tuple(o.value for o in out)
+
+
+def test_window_tables_are_recognised():
+    from cuv_amd import workloads as W
+    # 7x7 window on a 128-wide map: 7 window rows of 7 offsets, 128 rows apart, one group; both transposes
+    offs = W.window_offsets(128, 7)
+    for tr in (0, 1):
+        assert _walk(offs, 128 * 128, tr) == (2, (128, 7, 1, 7))
+    # the same offsets in scrambled table order: the diagonals of a window row no longer sit at evenly spaced
+    # table positions, which the walking kernel's addressing needs -- no window table (the products then run
+    # tile by tile, as for any table)
+    rng = np.random.default_rng(0)
+    assert _walk(rng.permutation(offs), 128 * 128)[0] == 0
+    # 5x5 window, three channel groups 64*64 rows apart; 3x3
+    assert _walk(W.window_offsets(64, 5, 3), 3 * 64 * 64) == (2, (64, 5, 3, 5))
+    assert _walk(W.window_offsets(192, 3), 192 * 192) == (2, (192, 3, 1, 3))
+    # window tables without a walking kernel: 13x13 (the large layer), 9x9, and a 7x7 window on a map whose
+    # width is no multiple of the 64-row tile
+    assert _walk(W.window_offsets(256, 13, 4), 4 * 256 * 256) == (1, (256, 13, 4, 13))
+    assert _walk(W.window_offsets(64, 9), 64 * 64) == (1, (64, 9, 1, 9))
+    assert _walk(W.window_offsets(48, 7), 48 * 48) == (1, (48, 7, 1, 7))
+    # a window that is not centred (first offset not congruent 1 mod 4 for 7 wide)
+    assert _walk([dy * 128 + dx for dy in range(7) for dx in range(7)], 128 * 128)[0] == 1
+
+
+def test_tables_that_are_no_window_tables():
+    # a single run, runs of different lengths, a grid with a missing row, window rows at uneven distances
+    assert _walk(list(range(-3, 4)), 4096)[0] == 0
+    assert _walk(list(range(-3, 4)) + [100, 101], 4096)[0] == 0
+    assert _walk([dy * 128 + dx for dy in (0, 1, 3) for dx in range(7)], 128 * 128)[0] == 0
+    assert _walk([dy + dx for dy in (0, 128, 300) for dx in range(7)], 128 * 128)[0] == 0
+    # two groups with different numbers of window rows
+    assert _walk([dx for dx in range(3)] + [64 + dx for dx in range(3)] + [5000 + dx for dx in range(3)], 8192)[0] == 0
+    from cuv_amd import _lib
+    assert _lib.lib().cuvdia_plan_walk(None, 3, 16, 0, None, None, None, None) == _lib.EINVAL
