@@ -304,6 +304,8 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     };
     span(cn, d->view.max_len_n, d->view.s_min_n, d->view.s_max_n);
     span(ct, d->view.max_len_t, d->view.s_min_t, d->view.s_max_t);
+    d->view.slot_step_n = common_slot_step(cn);
+    d->view.slot_step_t = common_slot_step(ct);
     int unused_min = 0, unused_max = 0;
     span(cp, d->view.max_len_p, unused_min, unused_max);
     *out = d;
@@ -580,9 +582,11 @@ int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals, const int *offsets_host
     if (trans) {
         view.chunks_t_dev = chunks_dev; view.n_chunks_t = (int)chunks.size();
         view.max_len_t = max_len; view.s_min_t = s_min; view.s_max_t = s_max;
+        view.slot_step_t = common_slot_step(chunks);
     } else {
         view.chunks_n_dev = chunks_dev; view.n_chunks_n = (int)chunks.size();
         view.max_len_n = max_len; view.s_min_n = s_min; view.s_max_n = s_max;
+        view.slot_step_n = common_slot_step(chunks);
     }
 
     // the kernel family is chosen by the rule of cuvdia_spmm_layer_f32

@@ -916,7 +916,8 @@ __device__ __forceinline__ void spmm_tile_lean(
     float (&lds)[3][SP_DSTAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
-    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, int first, SpEpilogue ep)
+    int n_out, int n_in, int batch, float alpha, float beta, unsigned a_bytes, int first, int slot_step,
+    SpEpilogue ep)
 {
     constexpr int T = 8, WAVES = 8, CPW = SP_COLS / WAVES;
     const int lane = threadIdx.x & 63;
@@ -1073,7 +1074,10 @@ __device__ __forceinline__ void spmm_tile_lean(
 #pragma unroll
             for (int k = 0; k < NP; ++k) asm("" : "+s"(p[k]));
             int sl;
-            if constexpr (LCK <= 8) {
+            if (slot_step != 0) {
+                // the table's diagonals sit at evenly spaced positions inside every chunk: no picking
+                sl = p[0] + a_j * slot_step;
+            } else if constexpr (LCK <= 8) {
                 // two waves fetch diagonals, four each: the wave's four candidates are chosen with scalar
                 // selects (wave is uniform), the lane's own among them with three vector selects
                 const bool up = wave != 3;
@@ -1237,7 +1241,7 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, int col_group, unsigned a_bytes,
-    int s_min, int s_max, int period_tiles, SpEpilogue ep)
+    int s_min, int s_max, int period_tiles, int slot_step, SpEpilogue ep)
 {
     static_assert(3 * SP_DSTAGE_FLOATS >= 2 * SP_STAGE_FLOATS, "the two bodies share one LDS block");
     __shared__ __attribute__((aligned(16))) float lds3[3][SP_DSTAGE_FLOATS];
@@ -1317,14 +1321,14 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     // A tile with one crossing chunk walks that chunk first: everything the loop then touches lies inside.
     if (lean && inner)
         spmm_tile_lean<LCK, NTAB, EP, true, false>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
-                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, ep);
+                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, slot_step, ep);
     else if (lean && crossing == 1 && c_hi > c_lo)
         spmm_tile_lean<LCK, NTAB, EP, true, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes,
-                                                  cross_at - c_lo, ep);
+                                                  cross_at - c_lo, slot_step, ep);
     else if (lean)
         spmm_tile_lean<LCK, NTAB, EP, false, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
-                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, ep);
+                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, slot_step, ep);
     else
         spmm_tile_edge<LCK, T, NTAB, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                          n_out, n_in, batch, alpha, beta, a_bytes, ep);
@@ -2143,6 +2147,7 @@ struct SpLaunch {
     unsigned a_bytes;
     int s_min, s_max;
     int period_tiles;           // window tables: tiles between window rows (0: no renumbering of the row tiles)
+    int slot_step;              // table positions between neighbouring diagonals of a chunk, if common (else 0)
     SpEpilogue ep;
     dim3 grid;
     hipStream_t stream;
@@ -2172,7 +2177,7 @@ hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
 // 8 rows per wave (8 waves per workgroup) keeps four waves on every SIMD
 // at the sizes this path is measured on.
 #define CUVDIA_SPMM_ARGS L.chunks, L.nchunks, L.vals, L.stride, L.ashift, L.B, L.ldb, L.dst, L.ldd, L.n_out, L.n_in, \
-                         L.batch, L.alpha, L.beta, L.col_tiles, L.col_group, L.a_bytes, L.s_min, L.s_max, L.period_tiles, L.ep
+                         L.batch, L.alpha, L.beta, L.col_tiles, L.col_group, L.a_bytes, L.s_min, L.s_max, L.period_tiles, L.slot_step, L.ep
 #define CUVDIA_SPMM_LAUNCH(K)                                                                                         \
     case K:                                                                                                           \
         if (L.nchunks <= 64 && !fused)                                                                                \
@@ -2298,7 +2303,7 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
                      trans ? A.s_min_t : A.s_min_n, trans ? A.s_max_t : A.s_max_n,
                      (wk.tab_dev != nullptr && wk.period % SP_ROWS == 0 && row_tiles * col_tiles > SP_RENUMBER_MIN_TILES)
                          ? wk.period / SP_ROWS : 0,
-                     ep,
+                     trans ? A.slot_step_t : A.slot_step_n, ep,
                      dim3((unsigned)(row_tiles * col_tiles)), stream, lck};
     if (lck <= 5) return spmm_tiled_launch_1_5(L);
     if (lck <= 9) return spmm_tiled_launch_6_9(L);

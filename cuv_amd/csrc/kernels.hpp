@@ -26,6 +26,7 @@ struct DiaView {
     int max_len_n, max_len_t;    // longest chunk of each table
     int s_min_n, s_max_n;        // smallest / largest chunk shift of each table
     int s_min_t, s_max_t;
+    int slot_step_n, slot_step_t; // common_slot_step of each table (0: none)
     WalkView walk_n, walk_t;     // window-table form of the two products' tables
     const Chunk *chunks_p_dev;   // the projection's table (chunks of up to CHUNK_MAX): shifts = offsets
     int n_chunks_p;

@@ -125,6 +125,23 @@ std::vector<Unit> plan_units(const std::vector<Chunk> &chunks)
     return out;
 }
 
+int common_slot_step(const std::vector<Chunk> &chunks)
+{
+    long long step = 0;
+    bool have = false;
+    for (const Chunk &c : chunks) {
+        for (int j = 0; j < c.len; ++j)
+            if (c.slot[j] < 0) return 0;
+        for (int j = 1; j < c.len; ++j) {
+            const long long d = (long long)c.slot[j] - c.slot[j - 1];
+            if (!have) { step = d; have = true; }
+            else if (d != step) return 0;
+        }
+    }
+    // the kernels add j * step to a position below 2^31 / stride: keep it small
+    return have && step != 0 && step > -(1 << 20) && step < (1 << 20) ? (int)step : 0;
+}
+
 int pair_delta_max(const std::vector<Chunk> &chunks, const std::vector<Unit> &units)
 {
     int m = 0;

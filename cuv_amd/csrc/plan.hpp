@@ -65,6 +65,10 @@ struct Unit {
 // Greedy over the table in shift order: chunk c pairs with c + 1 when their
 // shifts allow it.
 std::vector<Unit> plan_units(const std::vector<Chunk> &chunks);
+// The distance in table positions between neighbouring diagonals of a chunk when it is the same for every chunk
+// of the table (1 for a table listed in ascending order of its offsets), else 0.  The products' kernels then
+// compute a diagonal's table position instead of picking it out of the chunk's entry.
+int common_slot_step(const std::vector<Chunk> &chunks);
 // The largest distance between the first shifts of a pair (0 without pairs).
 int pair_delta_max(const std::vector<Chunk> &chunks, const std::vector<Unit> &units);
 
