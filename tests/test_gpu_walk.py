@@ -109,3 +109,72 @@ def test_automatic_choice_walks_a_large_product(oracle, gu, trans):
     B, dst = _operands(rng, A, 128, trans)
     _, ran = gu.check_prod(oracle, A, B, dst, trans, 1.0, 0.5, _lib.PATH_AUTO, "auto small", dev=dev)
     assert ran == _lib.PATH_TILED
+
+
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_walk_on_column_slices_of_wider_allocations(oracle, gu, trans):
+    """ld > rows for both dense operands, NaN in every gap of the input (and before its first and behind its last
+    column), a sentinel in the gaps of the destination: the walking kernel's staged blocks run 6 rows past a
+    tile and start up to 3 rows before it -- nothing of that may come from a gap, and nothing but the
+    destination's own rows may be written.  beta != 0 also reads the destination through the view."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    rng = np.random.default_rng(11)
+    px, batch = 64, 70
+    n = px * px
+    A = _window_dia(oracle, rng, n, n, px, 7)
+    B, dst = _operands(rng, A, batch, trans)
+    Ad = gu.make_dev_dia(A)
+    ldb, ldd = n + 12, n + 20
+    Bbig = torch.full((batch + 2, ldb), float("nan"), device="cuda:0")
+    Bbig[1:batch + 1, :n] = D.to_device_colmajor(B)
+    Dbig = torch.full((batch + 2, ldd), -7.0, device="cuda:0")
+    Dbig[1:batch + 1, :n] = D.to_device_colmajor(dst)
+    L = _lib.lib()
+    L.cuvdia_set_path(_lib.PATH_WALK)
+    try:
+        D.prod(Dbig[1:batch + 1, :n], Ad, Bbig[1:batch + 1, :n], trans, "n", 0.75, -1.5)
+        assert L.cuvdia_last_path() == _lib.PATH_WALK
+    finally:
+        L.cuvdia_set_path(_lib.PATH_AUTO)
+    got = D.to_host_colmajor(Dbig[1:batch + 1, :n])
+    gu.assert_close_mag(got, oracle.prod(A, B, dst, trans, 0.75, -1.5), oracle.prod_mag(A, B, dst, trans, 0.75, -1.5), "walk ld view")
+    assert torch.all(Dbig[:, n:] == -7.0) and torch.all(Dbig[0] == -7.0) and torch.all(Dbig[batch + 1] == -7.0)
+
+
+def test_walk_under_graph_capture_and_replay(oracle, gu):
+    """The walking kernel recorded into a HIP graph and replayed with the program's own eager work between the
+    replays: every replay equals the eager result."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    rng = np.random.default_rng(12)
+    px, batch = 64, 96
+    n = px * px
+    A = _window_dia(oracle, rng, n, n, px, 5)
+    B, dst0 = _operands(rng, A, batch, "n")
+    Ad = gu.make_dev_dia(A)
+    Bd = D.to_device_colmajor(B)
+    L = _lib.lib()
+    L.cuvdia_set_path(_lib.PATH_WALK)
+    try:
+        eager = torch.zeros(batch, n, device="cuda:0")
+        D.prod(eager, Ad, Bd, "n", "n", 1.0, 0.0)
+        assert L.cuvdia_last_path() == _lib.PATH_WALK
+        out = torch.zeros(batch, n, device="cuda:0")
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            D.prod(out, Ad, Bd, "n", "n", 1.0, 0.0, sync=False)          # warm-up on a side stream
+        torch.cuda.current_stream().wait_stream(s)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            D.prod(out, Ad, Bd, "n", "n", 1.0, 0.0, sync=False)          # (a synchronisation would end the capture)
+        for rep in range(3):
+            out.fill_(float("nan"))
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), "replay %d differs from the eager call" % rep
+    finally:
+        L.cuvdia_set_path(_lib.PATH_AUTO)
+    gu.assert_close_mag(D.to_host_colmajor(eager), oracle.prod(A, B), oracle.prod_mag(A, B), "walk eager")
