@@ -1561,6 +1561,25 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
     constexpr int LPC = ROWS / 4, CPI = 64 / LPC, CPW = SP_COLS / WAVES, NST = CPW / CPI, OPITCH = ROWS + 4;
     static_assert(SP_COLS * OPITCH <= S::XFLOATS, "the transposition fits the dense rows' part of a buffer");
     typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    typedef unsigned sp_u4 __attribute__((ext_vector_type(4)));
+    // What a lane contributes to the addresses of a tile's final store, kept for the whole walk: where it writes
+    // its sums in the transposition block and reads its 4 rows back (floats), and the byte offset of those rows in
+    // the destination's column tile (the out-of-range marker for a column past the batch: the buffer store then
+    // drops it).  A finished tile then costs its multiplications and two stores, no address arithmetic.
+    const int o_write = lane * OPITCH + wave * T;
+    int o_read[NST];
+    unsigned y_lane[NST];
+    {
+        const int ecol = wave * CPW + lane / LPC, erow = 4 * (lane % LPC);
+#pragma unroll
+        for (int q = 0; q < NST; ++q) {
+            const int col = ecol + CPI * q;
+            o_read[q] = col * OPITCH + erow;
+            y_lane[q] = col < cols_here ? (unsigned)(col * ldy + erow) * 4u : OOB_OFFSET;
+        }
+    }
+    const __amdgpu_buffer_rsrc_t yr = make_rsrc(
+        Y + (long long)col0 * ldy, (unsigned)(((long long)(cols_here - 1) * ldy + n_out) * 4));
     // Stores the tile that step u completes (m = u - K + 1, set (UU + 1) mod K) and clears its set for the tile
     // K steps on.  `ilast` is the step's last block: every wave is through with its buffer (the barrier that
     // ended the block), and the next request into it comes after the second barrier below.
@@ -1568,26 +1587,27 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         constexpr int SET = (decltype(uu_c)::value + 1) % K;
         const int m = u - (K - 1);
         if (m >= 0 && m < ntiles) {
-            const int ln = lane_now();
-            const int ecol = wave * CPW + ln / LPC, erow = 4 * (ln % LPC);
             float *out = &lds[ilast & 1][0];
+            static_assert(OPITCH % 4 == 0 && T % 4 == 0, "the sums leave as 16-byte LDS writes");
 #pragma unroll
-            for (int t = 0; t < T; ++t) out[lane * OPITCH + wave * T + t] = acc[SET][t];
+            for (int t = 0; t < T; t += 4)
+                *reinterpret_cast<float4 *>(out + o_write + t) =
+                    make_float4(acc[SET][t], acc[SET][t + 1], acc[SET][t + 2], acc[SET][t + 3]);
             __syncthreads();
             f4u v[NST];
 #pragma unroll
-            for (int q = 0; q < NST; ++q) v[q] = *reinterpret_cast<const f4u *>(out + (ecol + CPI * q) * OPITCH + erow);
+            for (int q = 0; q < NST; ++q) v[q] = *reinterpret_cast<const f4u *>(out + o_read[q]);
+            const unsigned tile_off = (unsigned)(row_first + m * period) * 4u;      // wave-uniform
+            if (beta == 0.f) {
 #pragma unroll
-            for (int q = 0; q < NST; ++q) {
-                const int col = ecol + CPI * q;
-                if (col < cols_here) {
-                    float *y = Y + (long long)(col0 + col) * ldy + row_first + m * period + erow;
-                    float r[4];
+                for (int q = 0; q < NST; ++q) v[q] = alpha * v[q];
+            } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) r[e] = (beta == 0.f) ? alpha * v[q][e] : beta * ypre[q][e] + alpha * v[q][e];
-                    stream_store4(y, r[0], r[1], r[2], r[3]);
-                }
+                for (int q = 0; q < NST; ++q) v[q] = beta * ypre[q] + alpha * v[q];
             }
+#pragma unroll
+            for (int q = 0; q < NST; ++q)       // non-temporal, like every result of the library
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(sp_u4, v[q]), yr, y_lane[q], tile_off, 2);
             __syncthreads();
         }
 #pragma unroll
@@ -1604,14 +1624,10 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         for (int q = 0; q < NST; ++q) ypre[q] = f4u{0.f, 0.f, 0.f, 0.f};
         const int mf = u - (K - 1);
         if (beta != 0.f && mf >= 0 && mf < ntiles) {
-            const int ln = lane_now();
-            const int ecol = wave * CPW + ln / LPC, erow = 4 * (ln % LPC);
+            const unsigned tile_off = (unsigned)(row_first + mf * period) * 4u;
 #pragma unroll
-            for (int q = 0; q < NST; ++q) {
-                const int col = ecol + CPI * q;
-                if (col < cols_here)
-                    ypre[q] = *reinterpret_cast<const f4u *>(Y + (long long)(col0 + col) * ldy + row_first + mf * period + erow);
-            }
+            for (int q = 0; q < NST; ++q)
+                ypre[q] = __builtin_bit_cast(f4u, __builtin_amdgcn_raw_buffer_load_b128(yr, y_lane[q], tile_off, 0));
         }
         int i = u * ngroups;
         for (int g = 0; g < ngroups; ++g, ++i) {
