@@ -1,7 +1,10 @@
 // Measures, on the GPU it runs on, the two rates the product kernels are laid out around:
 //   * how fast a SIMD issues fp32 FMAs in the forms a kernel can give them -- three vector-register operands, a
 //     DPP-broadcast operand (v_fmac_f32_dpp .. row_newbcast), a scalar operand;
-//   * how fast a CU's LDS answers 4-, 8- and 16-byte reads.
+//   * how fast a CU's LDS answers 4-, 8- and 16-byte reads;
+//   * what one launch that only moves the headline up-pass's bytes costs -- 8.4 MB + 3.2 MB read, 8.4 MB written,
+//     no arithmetic to speak of -- launched back to back from a HIP graph, with its operands in HBM (31 rotating
+//     buffer sets) and in the caches (one set): the time no kernel of that traffic can go below on this machine.
 // The kernels keep the batch along the lanes and broadcast a diagonal's value to them; this probe shows what that
 // form costs against the plain one, and what feeding the plain form from LDS would need.
 // Built by the Makefile into ../lib/hw_rates; prints one line per measurement.  Every wave runs a fixed number of
@@ -95,6 +98,26 @@ __global__ __launch_bounds__(256) void lds_kernel(float *out, long long *clk, in
     }
 }
 
+// y[i] = x[i] (+ a[i] for i < na4), 16-byte pieces, PT pieces per lane all requested before the first is stored
+template <int PT>
+__global__ __launch_bounds__(256) void stream_kernel(const f4 *__restrict__ x, const f4 *__restrict__ a,
+                                                     f4 *__restrict__ y, int n4, int na4)
+{
+    const int t = blockIdx.x * 256 + threadIdx.x, stride = gridDim.x * 256;
+    f4 v[PT];
+#pragma unroll
+    for (int k = 0; k < PT; ++k) {
+        const int i = t + k * stride;
+        v[k] = i < n4 ? x[i] : f4{0.f, 0.f, 0.f, 0.f};
+        if (i < na4) v[k] += a[i];
+    }
+#pragma unroll
+    for (int k = 0; k < PT; ++k) {
+        const int i = t + k * stride;
+        if (i < n4) __builtin_nontemporal_store(v[k], &y[i]);
+    }
+}
+
 struct Probe {
     float *out = nullptr;
     long long *clk = nullptr;
@@ -156,6 +179,60 @@ static int run_lds(Probe &p, const char *name)
     return 0;
 }
 
+// One launch per buffer set, `sets` launches recorded into a HIP graph and replayed.
+template <int PT>
+static int run_stream(int sets, const char *name)
+{
+    const int n4 = 16384 * 128 / 4, na4 = 49 * 16384 / 4;          // the headline layer: batch 128, 49 diagonals
+    const int total_sets = 31;
+    static f4 *x[31], *a[31], *y[31];
+    static bool ready = false;
+    if (!ready) {
+        for (int s = 0; s < total_sets; ++s) {
+            HW_CHECK(hipMalloc(&x[s], (size_t)n4 * 16));
+            HW_CHECK(hipMalloc(&a[s], (size_t)na4 * 16));
+            HW_CHECK(hipMalloc(&y[s], (size_t)n4 * 16));
+            HW_CHECK(hipMemset(x[s], 0, (size_t)n4 * 16));
+            HW_CHECK(hipMemset(a[s], 0, (size_t)na4 * 16));
+        }
+        ready = true;
+    }
+    hipStream_t st;
+    HW_CHECK(hipStreamCreate(&st));
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    const int wgs = (n4 + 256 * PT - 1) / (256 * PT);
+    HW_CHECK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+    for (int s = 0; s < total_sets; ++s) {
+        const int b = s % sets;
+        hipLaunchKernelGGL(stream_kernel<PT>, dim3(wgs), dim3(256), 0, st, x[b], a[b], y[b], n4, na4);
+    }
+    HW_CHECK(hipStreamEndCapture(st, &graph));
+    HW_CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    hipEvent_t e0, e1;
+    HW_CHECK(hipEventCreate(&e0));
+    HW_CHECK(hipEventCreate(&e1));
+    const int reps = 40;
+    for (int r = 0; r < 5; ++r) HW_CHECK(hipGraphLaunch(exec, st));
+    HW_CHECK(hipEventRecord(e0, st));
+    for (int r = 0; r < reps; ++r) HW_CHECK(hipGraphLaunch(exec, st));
+    HW_CHECK(hipEventRecord(e1, st));
+    HW_CHECK(hipEventSynchronize(e1));
+    float ms = 0;
+    HW_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    const double us = (double)ms * 1e3 / (reps * total_sets);
+    const double bytes = 16.0 * (2.0 * n4 + na4);
+    std::printf("move %-34s %6.2f us per launch  %6.0f GB/s  (%d workgroups, %.2f MB per launch)\n", name, us,
+                bytes / us / 1e3, wgs, bytes / 1e6);
+    std::fflush(stdout);
+    HW_CHECK(hipGraphExecDestroy(exec));
+    HW_CHECK(hipGraphDestroy(graph));
+    HW_CHECK(hipEventDestroy(e0));
+    HW_CHECK(hipEventDestroy(e1));
+    HW_CHECK(hipStreamDestroy(st));
+    return 0;
+}
+
 int main()
 {
     hipDeviceProp_t prop;
@@ -175,6 +252,14 @@ int main()
     if (run_lds<4>(p, "ds_read_b128")) return 1;
     if (run_lds<2>(p, "ds_read_b64")) return 1;
     if (run_lds<1>(p, "ds_read_b32")) return 1;
+    if (run_stream<1>(31, "operands in HBM, 1 piece per lane")) return 1;
+    if (run_stream<2>(31, "operands in HBM, 2 pieces per lane")) return 1;
+    if (run_stream<4>(31, "operands in HBM, 4 pieces per lane")) return 1;
+    if (run_stream<8>(31, "operands in HBM, 8 pieces per lane")) return 1;
+    if (run_stream<1>(1, "operands cached,  1 piece per lane")) return 1;
+    if (run_stream<2>(1, "operands cached,  2 pieces per lane")) return 1;
+    if (run_stream<4>(1, "operands cached,  4 pieces per lane")) return 1;
+    if (run_stream<8>(1, "operands cached,  8 pieces per lane")) return 1;
     HW_CHECK(hipFree(p.out));
     HW_CHECK(hipFree(p.clk));
     return 0;

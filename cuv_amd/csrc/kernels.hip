@@ -1385,6 +1385,14 @@ struct WalkShape {
     static constexpr int WAVES_PER_SIMD = WGS_PER_CU * WAVES / 4 < 4 ? WGS_PER_CU * WAVES / 4 : 4;
 };
 
+// x / d == (x * m) >> 16 for every 0 <= x < limit
+constexpr bool recip16_exact(unsigned d, unsigned m, unsigned limit)
+{
+    for (unsigned x = 0; x < limit; ++x)
+        if (x / d != ((x * m) >> 16)) return false;
+    return true;
+}
+
 // calls f(I) for I = 0 .. K-1 as compile-time constants
 template <int K, int I, class F>
 __device__ __forceinline__ void walk_for(F &&f)
@@ -1454,10 +1462,13 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
     typedef const int __attribute__((address_space(4))) *sc_int_ptr;
     const sc_int_ptr stab = (sc_int_ptr)tab;
 
-    // Requests block number i (step u = i / ngroups, group g = i % ngroups) into buffer i & 1: its dense
+    // piece -> column without an integer division: pieces number fewer than 2^11, and for those
+    // piece / XQ == (piece * XQ_RECIP) >> 16 (checked below), a 24-bit multiplication at full rate
+    constexpr unsigned XQ_RECIP = (65536u + XQ - 1) / XQ;
+    static_assert(64 * XIT * WAVES <= 2048 && recip16_exact(XQ, XQ_RECIP, 2048), "piece / XQ by multiplication");
+    // Requests block number i = u * ngroups + g (step u, group g) into buffer i & 1: its dense
     // rows and, for every tile m = u - dy that exists, the values of chunk (g, dy) for the tile's rows.
-    auto issue = [&](int i) __attribute__((always_inline)) {
-        const int u = i / ngroups, g = i - u * ngroups;
+    auto issue = [&](int i, int u, int g) __attribute__((always_inline)) {
         const int a0 = row_first + s0 + stab[g] + u * period;        // first dense row the block's chunks read
         if (a0 + ROWS + LCK - 1 <= 0 || a0 >= n_in) return;          // wholly outside: nothing to stage (see apply)
         const unsigned buf = lds0 + (unsigned)(i & 1) * BUF_BYTES;
@@ -1467,7 +1478,7 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         for (int it = 0; it < XIT; ++it) {
             if (wave + WAVES * it < XQ) {
                 const int piece = 64 * (wave + WAVES * it) + ln;
-                const int col = piece / XQ;
+                const int col = (int)(__umul24((unsigned)piece, XQ_RECIP) >> 16);
                 const int r = a0p + 4 * (piece - col * XQ);
                 const unsigned x_col = (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u);
                 const bool ok = (r >= 0) & (r + 4 <= n_in);
@@ -1614,7 +1625,7 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         for (int t = 0; t < T; ++t) acc[SET][t] = 0.f;
     };
 
-    issue(0);
+    issue(0, 0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     auto step = [&](int u, auto uu_c) __attribute__((always_inline)) {
@@ -1631,7 +1642,10 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         }
         int i = u * ngroups;
         for (int g = 0; g < ngroups; ++g, ++i) {
-            if (i + 1 < nblocks) issue(i + 1);
+            if (i + 1 < nblocks) {
+                const bool last = g + 1 == ngroups;
+                issue(i + 1, last ? u + 1 : u, last ? 0 : g + 1);
+            }
             apply(i, u, g, uu_c);
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __syncthreads();
