@@ -1,7 +1,8 @@
 // Measures, on the GPU it runs on, the two rates the product kernels are laid out around:
-//   * how fast a SIMD issues fp32 FMAs in the forms a kernel can give them -- three vector-register operands, a
-//     DPP-broadcast operand (v_fmac_f32_dpp .. row_newbcast), a scalar operand;
-//   * how fast a CU's LDS answers 4-, 8- and 16-byte reads;
+//   * how fast a SIMD issues fp32 FMAs in the forms a kernel can give them -- three vector-register operands (with
+//     the two multiplicands in different banks of the register file or in the same one), a DPP-broadcast operand
+//     (v_fmac_f32_dpp .. row_newbcast), a scalar operand;
+//   * how fast a CU's LDS answers 4-, 8- and 16-byte reads, with an address per lane and with one per wave;
 //   * what one launch that only moves the headline up-pass's bytes costs -- 8.4 MB + 3.2 MB read, 8.4 MB written,
 //     no arithmetic to speak of -- launched back to back from a HIP graph, with its operands in HBM (31 rotating
 //     buffer sets) and in the caches (one set): the time no kernel of that traffic can go below on this machine.
@@ -33,13 +34,133 @@ __global__ __launch_bounds__(256) void fma_kernel(float *out, long long *clk, in
     float acc[16];
     for (int i = 0; i < 16; ++i) acc[i] = threadIdx.x * 0.001f + i;
     const float x = a + threadIdx.x;
+    // FORM 3 and 4: three vector registers of the compiler's choosing, no two FMAs in a row sharing an operand
+    // register -- 8 + 8 (FORM 4: 4 + 16) different ones, as in a tile's inner loop
+    float xs[16], as[16];
+    for (int i = 0; i < 16; ++i) {
+        xs[i] = x + i;
+        as[i] = a * (i + 1);
+        asm volatile("" : "+v"(xs[i]), "+v"(as[i]));
+    }
     const long long c0 = clock64(), w0 = wall_clock64();
-    for (int it = 0; it < iters; ++it) {
+    // FORM 5 .. 9: the same FMAs on registers named outright, to place the three operands in the register file's four
+    // banks (a register's bank is its number modulo 4):
+    //   5 -- sums in consecutive registers, multiplicands in banks 0 and 1
+    //   6 -- sums in banks 2 and 3, multiplicands in banks 0 and 1: no two operands share a bank
+    //   7 -- sums in consecutive registers, both multiplicands in bank 0
+    //   8 -- sums in banks 2 and 3, both multiplicands in bank 0
+    //   9 -- all three operands in bank 0
+    if (FORM >= 5) {
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (FORM == 5)
+                asm volatile(
+                    "v_fmac_f32 v108, v100, v101\n\t"
+                    "v_fmac_f32 v109, v100, v101\n\t"
+                    "v_fmac_f32 v110, v100, v101\n\t"
+                    "v_fmac_f32 v111, v100, v101\n\t"
+                    "v_fmac_f32 v112, v100, v101\n\t"
+                    "v_fmac_f32 v113, v100, v101\n\t"
+                    "v_fmac_f32 v114, v100, v101\n\t"
+                    "v_fmac_f32 v115, v100, v101\n\t"
+                    "v_fmac_f32 v116, v100, v101\n\t"
+                    "v_fmac_f32 v117, v100, v101\n\t"
+                    "v_fmac_f32 v118, v100, v101\n\t"
+                    "v_fmac_f32 v119, v100, v101\n\t"
+                    "v_fmac_f32 v120, v100, v101\n\t"
+                    "v_fmac_f32 v121, v100, v101\n\t"
+                    "v_fmac_f32 v122, v100, v101\n\t"
+                    "v_fmac_f32 v123, v100, v101\n\t"
+                    ::: "v100", "v101", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123");
+                if (FORM == 6)
+                asm volatile(
+                    "v_fmac_f32 v110, v100, v101\n\t"
+                    "v_fmac_f32 v111, v100, v101\n\t"
+                    "v_fmac_f32 v114, v100, v101\n\t"
+                    "v_fmac_f32 v115, v100, v101\n\t"
+                    "v_fmac_f32 v118, v100, v101\n\t"
+                    "v_fmac_f32 v119, v100, v101\n\t"
+                    "v_fmac_f32 v122, v100, v101\n\t"
+                    "v_fmac_f32 v123, v100, v101\n\t"
+                    "v_fmac_f32 v126, v100, v101\n\t"
+                    "v_fmac_f32 v127, v100, v101\n\t"
+                    "v_fmac_f32 v130, v100, v101\n\t"
+                    "v_fmac_f32 v131, v100, v101\n\t"
+                    "v_fmac_f32 v134, v100, v101\n\t"
+                    "v_fmac_f32 v135, v100, v101\n\t"
+                    "v_fmac_f32 v138, v100, v101\n\t"
+                    "v_fmac_f32 v139, v100, v101\n\t"
+                    ::: "v100", "v101", "v110", "v111", "v114", "v115", "v118", "v119", "v122", "v123", "v126", "v127", "v130", "v131", "v134", "v135", "v138", "v139");
+                if (FORM == 7)
+                asm volatile(
+                    "v_fmac_f32 v108, v100, v104\n\t"
+                    "v_fmac_f32 v109, v100, v104\n\t"
+                    "v_fmac_f32 v110, v100, v104\n\t"
+                    "v_fmac_f32 v111, v100, v104\n\t"
+                    "v_fmac_f32 v112, v100, v104\n\t"
+                    "v_fmac_f32 v113, v100, v104\n\t"
+                    "v_fmac_f32 v114, v100, v104\n\t"
+                    "v_fmac_f32 v115, v100, v104\n\t"
+                    "v_fmac_f32 v116, v100, v104\n\t"
+                    "v_fmac_f32 v117, v100, v104\n\t"
+                    "v_fmac_f32 v118, v100, v104\n\t"
+                    "v_fmac_f32 v119, v100, v104\n\t"
+                    "v_fmac_f32 v120, v100, v104\n\t"
+                    "v_fmac_f32 v121, v100, v104\n\t"
+                    "v_fmac_f32 v122, v100, v104\n\t"
+                    "v_fmac_f32 v123, v100, v104\n\t"
+                    ::: "v100", "v104", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123");
+                if (FORM == 8)
+                asm volatile(
+                    "v_fmac_f32 v110, v100, v104\n\t"
+                    "v_fmac_f32 v111, v100, v104\n\t"
+                    "v_fmac_f32 v114, v100, v104\n\t"
+                    "v_fmac_f32 v115, v100, v104\n\t"
+                    "v_fmac_f32 v118, v100, v104\n\t"
+                    "v_fmac_f32 v119, v100, v104\n\t"
+                    "v_fmac_f32 v122, v100, v104\n\t"
+                    "v_fmac_f32 v123, v100, v104\n\t"
+                    "v_fmac_f32 v126, v100, v104\n\t"
+                    "v_fmac_f32 v127, v100, v104\n\t"
+                    "v_fmac_f32 v130, v100, v104\n\t"
+                    "v_fmac_f32 v131, v100, v104\n\t"
+                    "v_fmac_f32 v134, v100, v104\n\t"
+                    "v_fmac_f32 v135, v100, v104\n\t"
+                    "v_fmac_f32 v138, v100, v104\n\t"
+                    "v_fmac_f32 v139, v100, v104\n\t"
+                    ::: "v100", "v104", "v110", "v111", "v114", "v115", "v118", "v119", "v122", "v123", "v126", "v127", "v130", "v131", "v134", "v135", "v138", "v139");
+                if (FORM == 9)
+                asm volatile(
+                    "v_fmac_f32 v108, v100, v104\n\t"
+                    "v_fmac_f32 v112, v100, v104\n\t"
+                    "v_fmac_f32 v116, v100, v104\n\t"
+                    "v_fmac_f32 v120, v100, v104\n\t"
+                    "v_fmac_f32 v124, v100, v104\n\t"
+                    "v_fmac_f32 v128, v100, v104\n\t"
+                    "v_fmac_f32 v132, v100, v104\n\t"
+                    "v_fmac_f32 v136, v100, v104\n\t"
+                    "v_fmac_f32 v140, v100, v104\n\t"
+                    "v_fmac_f32 v144, v100, v104\n\t"
+                    "v_fmac_f32 v148, v100, v104\n\t"
+                    "v_fmac_f32 v152, v100, v104\n\t"
+                    "v_fmac_f32 v156, v100, v104\n\t"
+                    "v_fmac_f32 v160, v100, v104\n\t"
+                    "v_fmac_f32 v164, v100, v104\n\t"
+                    "v_fmac_f32 v168, v100, v104\n\t"
+                    ::: "v100", "v104", "v108", "v112", "v116", "v120", "v124", "v128", "v132", "v136", "v140", "v144", "v148", "v152", "v156", "v160", "v164", "v168");
+            }
+        }
+    }
+    for (int it = 0; FORM < 5 && it < iters; ++it) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                if (FORM == 0) asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[i]) : "v"(x), "v"(a));
+                if (FORM == 3)
+                    asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[i]) : "v"(xs[(i + 3 * r) % 8]), "v"(as[(i / 2 + r) % 8]));
+                if (FORM == 4)
+                    asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[i]) : "v"(xs[i / 4]), "v"(as[(i % 4 + i / 4 + 4 * r) % 16]));
                 if (FORM == 1)
                     asm volatile("v_fmac_f32_dpp %0, %1, %2 row_newbcast:1 row_mask:0xf bank_mask:0xf"
                                  : "+v"(acc[i]) : "v"(x), "v"(a));
@@ -57,14 +178,16 @@ __global__ __launch_bounds__(256) void fma_kernel(float *out, long long *clk, in
 }
 
 // every lane reads 4 W bytes per instruction at consecutive addresses (conflict-free), 8 instructions per iteration
-template <int W>
+// UNIFORM: every lane of a wave reads the same address (a value broadcast to the wave)
+template <int W, bool UNIFORM = false>
 __global__ __launch_bounds__(256) void lds_kernel(float *out, long long *clk, int iters)
 {
     __shared__ __attribute__((aligned(16))) float buf[8192];
     for (int i = threadIdx.x; i < 8192; i += 256) buf[i] = i;
     __syncthreads();
     const unsigned base =
-        (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)buf + threadIdx.x * (W * 4);
+        (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)buf +
+        (UNIFORM ? (threadIdx.x >> 6) * 64 : threadIdx.x * (W * 4));
     float sum = 0.f;
     const long long c0 = clock64(), w0 = wall_clock64();
     for (int it = 0; it < iters; ++it) {
@@ -159,7 +282,7 @@ static int run_fma(Probe &p, const char *name)
     return 0;
 }
 
-template <int W>
+template <int W, bool UNIFORM = false>
 static int run_lds(Probe &p, const char *name)
 {
     const int iters = 20000;
@@ -167,7 +290,7 @@ static int run_lds(Probe &p, const char *name)
     double mhz = 0;
     for (int rep = 0; rep < 2; ++rep) {
         HW_CHECK(hipEventRecord(p.e0));
-        hipLaunchKernelGGL(lds_kernel<W>, dim3(p.wgs), dim3(256), 0, 0, p.out, p.clk, iters);
+        hipLaunchKernelGGL((lds_kernel<W, UNIFORM>), dim3(p.wgs), dim3(256), 0, 0, p.out, p.clk, iters);
         HW_CHECK(hipGetLastError());
         HW_CHECK(hipEventRecord(p.e1));
         if (finish(p, &ms, &mhz)) return 1;
@@ -246,12 +369,21 @@ int main()
     HW_CHECK(hipEventCreate(&p.e0));
     HW_CHECK(hipEventCreate(&p.e1));
     std::printf("%s, %d CUs\n", prop.name, p.cus);
-    if (run_fma<0>(p, "v_fmac_f32 v, v, v")) return 1;
     if (run_fma<1>(p, "v_fmac_f32_dpp row_newbcast")) return 1;
     if (run_fma<2>(p, "v_fmac_f32 v, s, v")) return 1;
+    if (run_fma<5>(p, "v v v: sums consecutive, a b banks 0 1")) return 1;
+    if (run_fma<6>(p, "v v v: sums banks 2 3, a b banks 0 1")) return 1;
+    if (run_fma<7>(p, "v v v: sums consecutive, a b bank 0")) return 1;
+    if (run_fma<8>(p, "v v v: sums banks 2 3, a b bank 0")) return 1;
+    if (run_fma<9>(p, "v v v: all in bank 0")) return 1;
+    if (run_fma<3>(p, "v_fmac_f32 v, v, v (8 x 8 operands)")) return 1;
+    if (run_fma<4>(p, "v_fmac_f32 v, v, v (4 x 16 operands)")) return 1;
     if (run_lds<4>(p, "ds_read_b128")) return 1;
     if (run_lds<2>(p, "ds_read_b64")) return 1;
     if (run_lds<1>(p, "ds_read_b32")) return 1;
+    if (run_lds<4, true>(p, "ds_read_b128, one address per wave")) return 1;
+    if (run_lds<2, true>(p, "ds_read_b64, one address per wave")) return 1;
+    if (run_lds<1, true>(p, "ds_read_b32, one address per wave")) return 1;
     if (run_stream<1>(31, "operands in HBM, 1 piece per lane")) return 1;
     if (run_stream<2>(31, "operands in HBM, 2 pieces per lane")) return 1;
     if (run_stream<4>(31, "operands in HBM, 4 pieces per lane")) return 1;
