@@ -427,7 +427,19 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
     if (const int rc = check_device(desc)) return rc;
 
     const int forced = g_path.load();
-    const bool tiled_possible = dd2dia_tiled_ok(desc->view, lda, ldb, batch);
+    // The tiled kernel addresses its operands with 32-bit byte offsets.  A batch whose operands are larger is
+    // walked in slabs of columns that fit: the sum over the batch is the sum of the slabs' sums, so the first slab
+    // runs with the caller's beta and every later one adds to what is there (beta = 1), one launch after the other
+    // on the caller's stream.
+    int slab = batch;
+    bool tiled_possible = dd2dia_tiled_ok(desc->view, lda, ldb, batch);
+    if (!tiled_possible && batch > DD2DIA_SLAB_MIN) {
+        const int fit = dd2dia_slab_columns(desc->view, lda, ldb);
+        if (fit >= DD2DIA_SLAB_MIN && dd2dia_tiled_ok(desc->view, lda, ldb, fit)) {
+            slab = fit;
+            tiled_possible = true;
+        }
+    }
     bool tiled;
     if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
@@ -438,9 +450,14 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
         tiled = tiled_possible;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const hipError_t e = tiled
-        ? launch_dd2dia_tiled(desc->view, C_vals, A, lda, B, ldb, batch, alpha, beta, s)
-        : launch_dd2dia_generic(desc->view, C_vals, A, lda, B, ldb, batch, alpha, beta, s);
+    hipError_t e = hipSuccess;
+    if (!tiled) {
+        e = launch_dd2dia_generic(desc->view, C_vals, A, lda, B, ldb, batch, alpha, beta, s);
+    } else {
+        for (int c0 = 0; c0 < batch && e == hipSuccess; c0 += slab)
+            e = launch_dd2dia_tiled(desc->view, C_vals, A + (long long)c0 * lda, lda, B + (long long)c0 * ldb, ldb,
+                                    std::min(slab, batch - c0), alpha, c0 == 0 ? beta : 1.f, s);
+    }
     t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "dd2dia kernel launch");
 }

@@ -2411,6 +2411,19 @@ bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch)
            b_bytes < (long long)OOB_OFFSET && c_bytes < (long long)OOB_OFFSET;
 }
 
+int dd2dia_slab_columns(const DiaView &C, long long lda, long long ldb)
+{
+    // ((n - 1) * ld + rows) * 4 < OOB_OFFSET for both operands
+    const long long floats = (long long)OOB_OFFSET / 4;
+    auto cols = [&](long long ld, long long rows) -> long long {
+        if (rows >= floats || ld <= 0) return 0;
+        return (floats - rows - 1) / ld + 1;
+    };
+    const long long n = std::min(cols(lda, C.h), cols(ldb, C.w));
+    const long long whole = n / DD2DIA_SLAB_MIN * DD2DIA_SLAB_MIN;
+    return whole >= DD2DIA_SLAB_MIN ? (int)std::min<long long>(whole, 1 << 30) : 0;
+}
+
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream)

@@ -90,6 +90,10 @@ hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, 
 // Whether the tiled dd2dia can serve these operands (row_fact 1, operand
 // extents within its 32-bit buffer addressing).
 bool dd2dia_tiled_ok(const DiaView &C, long long lda, long long ldb, int batch);
+// The largest number of batch columns (a multiple of 32) whose rows of both operands lie within the tiled
+// kernel's 32-bit byte offsets, 0 if not even DD2DIA_SLAB_MIN do.
+constexpr int DD2DIA_SLAB_MIN = 32;
+int dd2dia_slab_columns(const DiaView &C, long long lda, long long ldb);
 
 // Same contract, row_fact == 1 only: a workgroup owns 256 rows of one run
 // chunk; each lane keeps 4 rows x (longest chunk) diagonals of partial sums,

@@ -221,7 +221,9 @@ int cuvdia_learn_step_weight_decay_momentum_f32(float *W_device, float *momentum
  * dense2dia_mm (densedense_to_sparse.cu:51-120), with the documented
  * contract of src/cuv/matrix_ops/densedense_to_sparse.hpp:107-121.
  * A is h x batch (lda >= h), B is w x batch (ldb >= w).  beta == 0 never
- * reads C.  batch == 0 scales C by beta (zero-fills valid slots if beta == 0). */
+ * reads C.  batch == 0 scales C by beta (zero-fills valid slots if beta == 0).
+ * A batch whose operands are larger than 2 GiB is worked in several launches
+ * on `stream`, slab of columns after slab, each adding to C. */
 int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals_device,
                       const float *A_device, long long lda,
                       const float *B_device, long long ldb, int batch,
