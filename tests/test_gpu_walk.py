@@ -178,3 +178,32 @@ def test_walk_under_graph_capture_and_replay(oracle, gu):
     finally:
         L.cuvdia_set_path(_lib.PATH_AUTO)
     gu.assert_close_mag(D.to_host_colmajor(eager), oracle.prod(A, B), oracle.prod_mag(A, B), "walk eager")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_walk_on_random_window_shapes(oracle, gu, seed):
+    """Seeded draws of the map (width a multiple of 64, any height), window (3, 5, 7), channels, a matrix that is
+    square or a few rows wider or narrower, batch and factors; both transposes, the walking kernel forced."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(9000 + seed)
+    px = int(rng.choice([64, 128, 192, 256, 320]))
+    fs = int(rng.choice([3, 5, 7]))
+    ch = int(rng.choice([1, 1, 2, 3]))
+    py = int(rng.integers(fs + 1, 40))
+    n = px * py
+    r = fs // 2
+    offs = [c * n + dy * px + dx for c in range(ch) for dy in range(-r, r + 1) for dx in range(-r, r + 1)]
+    h = n * ch
+    w = h + int(rng.choice([0, 0, px, -px, 64])) if ch == 1 else h
+    batch = int(rng.choice([1, 24, 40, 64, 65, 128, 200, 300]))
+    alpha, beta = float(rng.uniform(-2, 2)), float(rng.choice([0.0, 1.0, rng.uniform(-1, 1)]))
+    A = oracle.Dia(h, w, offs, None, 1)
+    A.vals[:] = np.nan
+    m = oracle.valid_mask(A)
+    A.vals[m] = rng.uniform(-1, 1, int(m.sum())).astype(np.float32)
+    for trans in ("n", "t"):
+        B, dst = _operands(rng, A, batch, trans)
+        what = "seed %d: map %dx%d, window %d, %d channels, %dx%d, batch %d, '%s'" % (seed, px, py, fs, ch, h, w, batch, trans)
+        print(what, flush=True)
+        _, ran = gu.check_prod(oracle, A, B, None if beta == 0.0 else dst, trans, alpha, beta, _lib.PATH_WALK, what)
+        assert ran == _lib.PATH_WALK
