@@ -213,6 +213,16 @@ def bench_scale(args, torch, D, W, dev):
             torch.cuda.synchronize()
             reps = max(2, min(20, int(2e4 / max(1.0, nbytes / 2e6))))
             s = torch.cuda.current_stream()
+            # about 30 ms of untimed replays first: an operation timed right after its operands were drawn reads a
+            # few per cent slow
+            w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            w0.record(s)
+            graph.replay()
+            w1.record(s)
+            torch.cuda.synchronize()
+            for _ in range(max(1, min(200, int(30.0 / max(1e-3, w0.elapsed_time(w1)))))):
+                graph.replay()
+            torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(s)
             for _ in range(reps):
