@@ -436,7 +436,10 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
     if (!tiled_possible && batch > DD2DIA_SLAB_MIN) {
         const int fit = dd2dia_slab_columns(desc->view, lda, ldb);
         if (fit >= DD2DIA_SLAB_MIN && dd2dia_tiled_ok(desc->view, lda, ldb, fit)) {
-            slab = fit;
+            // slabs of about equal width rather than full ones and a sliver
+            const int count = (batch + fit - 1) / fit;
+            const int even = ((batch + count - 1) / count + DD2DIA_SLAB_MIN - 1) / DD2DIA_SLAB_MIN * DD2DIA_SLAB_MIN;
+            slab = std::min(fit, even);
             tiled_possible = true;
         }
     }

@@ -1659,8 +1659,9 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
 // ------------------------------------------------------------ tiled dd2dia --
 //
 // Workgroup = 256 rows of ONE unit: a run chunk, or two chunks whose first
-// shifts differ by delta (a multiple of 4, at most 128) -- e.g. two rows of a
-// 2-d window.  Lane l owns rows row0 + 4l .. 4l+3 and 4 x LC partial sums per
+// shifts differ by delta (a multiple of 4) -- e.g. two rows of a 2-d window
+// (what follows describes pairs up to 128 rows apart; DdShape lists the other
+// forms).  Lane l owns rows row0 + 4l .. 4l+3 and 4 x LC partial sums per
 // chunk (LC = the longest chunk of the table; positions past a chunk's own
 // length are computed and dropped).  A table with runs of more than 8 shifts
 // (window rows wider than 8) is walked in the products' chunks of up to 13
@@ -1694,41 +1695,50 @@ constexpr int DD_BG = 4;           // batch columns per step
 // keeps as many running sums as a pair but is worked by 4 waves: three such
 // workgroups share a CU (registers allow 3 waves per SIMD, and the block the
 // sums are added in is kept just under a third of the CU's LDS).
-// WIDE: a pair whose chunks start more than PAIR_NARROW_DELTA rows apart (window rows of a map wider than 128):
-// its band takes a third 16-byte piece per lane and column.
-template <int NCH, int LC, bool WIDE = false>
+// WIDE says how a pair is served.  The two chunks of a pair start delta rows apart; for row i the first pairs it
+// with rows i + s0 + j of B, the second with rows i + s0 + delta + j.
+//   DD_NARROW, DD_WIDE -- both chunks work on the SAME rows of A: one copy of A's rows and one band of B that
+//     holds both windows, delta rows apart (two 16-byte pieces per lane and column up to PAIR_NARROW_DELTA, a
+//     third up to PAIR_BAND_DELTA: window rows of a map wider than 128); 8 waves, alone on their CU;
+//   DD_SHIFTED -- the second chunk works on the rows delta ABOVE the first's, so that both read the SAME rows of B:
+//     one band of one piece (the tile is cut short, dd_short_rows), one window per column for both chunks, and two
+//     copies of A's rows.  Any distance that is a multiple of 4; 4 waves, three such workgroups to a CU.
+constexpr int DD_NARROW = 0, DD_WIDE = 1, DD_SHIFTED = 2;
+template <int NCH, int LC, int WIDE = DD_NARROW>
 struct DdShape {
     static_assert(NCH == 1 || LC <= CHUNK_MAX, "pairs are made of short chunks");
-    static_assert(NCH == 2 || !WIDE, "only pairs are wide");
+    static_assert(NCH == 2 || WIDE == DD_NARROW, "only pairs come in forms");
     static constexpr bool LONG = LC > CHUNK_MAX;
     static constexpr int SPAN = LONG ? SP_CHUNK_MAX : CHUNK_MAX;    // shifts a chunk can have
-    static constexpr int NQ = NCH == 1 ? 4 : WIDE ? 8 : 6;      // 64-row blocks of the band
-    static constexpr int NB = WIDE ? 3 : 2;                     // 16-byte pieces a lane holds per column
+    static constexpr int NQ = (NCH == 1 || WIDE == DD_SHIFTED) ? 4 : WIDE == DD_WIDE ? 8 : 6;   // 64-row blocks of the band
+    static constexpr int NB = WIDE == DD_WIDE ? 3 : WIDE == DD_SHIFTED ? 1 : 2;   // 16-byte pieces a lane holds per column
     static constexpr int PITCH = 64 * NQ + (LONG ? 16 : 8);     // staged rows per column: 264, 272, 392 or 520
-    static constexpr int WAVES = NCH == 2 ? 8 : 4;
+    static constexpr int WAVES = (NCH == 2 && WIDE != DD_SHIFTED) ? 8 : 4;
     static constexpr int RED_PAD = LONG ? 4 : 8;              // a long chunk's sums then fit a third of a CU's LDS
     static constexpr int WAVE_FLOATS = 2 * DD_BG * PITCH + 4;   // two buffers + a slot idle lanes write to
     static constexpr int STAGE_FLOATS = WAVES * WAVE_FLOATS;
 };
 static_assert(DdShape<2, CHUNK_MAX>::PITCH >= DD_ROWS + PAIR_NARROW_DELTA + CHUNK_MAX, "a pair's band must fit its buffer");
-static_assert(DdShape<2, CHUNK_MAX, true>::PITCH >= DD_ROWS + PAIR_MAX_DELTA + CHUNK_MAX, "a wide pair's band must fit its buffer");
-static_assert(DdShape<2, CHUNK_MAX>::NB == 2 && DdShape<2, CHUNK_MAX, true>::NB == 3 && DdShape<1, CHUNK_MAX>::NB == 2, "pieces per lane");
+static_assert(DdShape<2, CHUNK_MAX, DD_WIDE>::PITCH >= DD_ROWS + PAIR_BAND_DELTA + CHUNK_MAX, "a wide pair's band must fit its buffer");
+static_assert(DdShape<2, CHUNK_MAX>::NB == 2 && DdShape<2, CHUNK_MAX, DD_WIDE>::NB == 3 && DdShape<1, CHUNK_MAX>::NB == 2, "pieces per lane");
 static_assert(DdShape<1, SP_CHUNK_MAX>::PITCH >= DD_ROWS + 4 * ((4 + SP_CHUNK_MAX - 1 + 3) / 4) - 4,
               "a long chunk's last window must fit its buffer");
 
 // What a wave has in flight of A for one group of 4 batch columns (two of
 // these alternate; B's pieces need one set of registers only, see the loop).
+template <int NA>
 struct DdStage {
-    float a[DD_BG][4];    // this lane's 4 rows of each column
+    float a[NA][DD_BG][4];    // this lane's 4 rows of each column (a shifted pair: and the 4 rows delta above)
 };
 
 template <int LC, int NCH>
 constexpr int dd_red_floats() { return 4 * 4 * (NCH * LC * 64 + DdShape<NCH, LC>::RED_PAD); }
-template <int LC, int NCH, bool WIDE = false>
+template <int LC, int NCH, int WIDE = DD_NARROW>
 constexpr int dd_lds_floats()
 {
-    return DdShape<NCH, LC, WIDE>::STAGE_FLOATS > dd_red_floats<LC, NCH>() ? DdShape<NCH, LC, WIDE>::STAGE_FLOATS
-                                                                           : dd_red_floats<LC, NCH>();
+    // (a shifted pair adds its chunks' sums one chunk after the other, in the block of a single chunk)
+    constexpr int red = WIDE == DD_SHIFTED ? dd_red_floats<LC, 1>() : dd_red_floats<LC, NCH>();
+    return DdShape<NCH, LC, WIDE>::STAGE_FLOATS > red ? DdShape<NCH, LC, WIDE>::STAGE_FLOATS : red;
 }
 
 // Rows of a tile.  A launch of single chunks only (no pairs) cuts its tiles 8 (long chunks: 16) rows short of
@@ -1737,7 +1747,7 @@ constexpr int dd_lds_floats()
 template <int LC>
 constexpr int dd_short_rows() { return DD_ROWS - (LC > CHUNK_MAX ? 16 : 8); }
 
-template <int LC, int NCH, bool AVEC, bool WIDE = false, bool SHORT = false>
+template <int LC, int NCH, bool AVEC, int WIDE = DD_NARROW, bool SHORT = false>
 __device__ __forceinline__ void dd2dia_unit(
     float *lds, int row0, const Chunk *ck1, const Chunk *ck2, float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
@@ -1745,13 +1755,18 @@ __device__ __forceinline__ void dd2dia_unit(
     unsigned c_bytes)
 {
     typedef DdShape<NCH, LC, WIDE> S;
-    static_assert(!SHORT || NCH == 1, "only launches of single chunks use short tiles");
-    constexpr int TR = SHORT ? dd_short_rows<LC>() : DD_ROWS;             // rows of the tile
+    constexpr bool SHIFTED = WIDE == DD_SHIFTED;
+    static_assert(!SHORT || NCH == 1, "short tiles: launches of single chunks, and of shifted pairs (which say so)");
+    static_assert(!SHIFTED || AVEC, "pairs are formed with 16-byte loads of A only");
+    constexpr int TR = (SHORT || SHIFTED) ? dd_short_rows<LC>() : DD_ROWS;    // rows of the tile
     constexpr int PITCH = S::PITCH, WAVES = S::WAVES, NB = SHORT ? 1 : S::NB;
+    constexpr int NA = SHIFTED ? 2 : 1;                      // copies of A's rows a lane holds per column
+    constexpr int NWIN = SHIFTED ? 1 : NCH;                  // windows of B a lane reads per column
+    constexpr int NRED = SHIFTED ? 1 : NCH;                  // chunks whose sums meet in LDS at a time
     static_assert(!SHORT || TR + S::SPAN <= 256 || (S::LONG && TR + 16 <= 256), "a short tile's band is one piece per lane");
     constexpr int WIN = 4 + LC - 1;
     constexpr int WQ = (WIN + 3) / 4;
-    constexpr int RED_T = NCH * LC * 64 + S::RED_PAD;        // floats between the 4 rows a lane owns: keeps the
+    constexpr int RED_T = NRED * LC * 64 + S::RED_PAD;       // floats between the 4 rows a lane owns: keeps the
                                                     // row-major read below free of bank conflicts
     constexpr int RED_WAVE = 4 * RED_T;
 
@@ -1774,12 +1789,15 @@ __device__ __forceinline__ void dd2dia_unit(
         }
     }
     const int delta = NCH == 2 ? s0[NCH - 1] - s0[0] : 0;      // rows between the two windows
-    const int need = TR + delta + S::SPAN;                      // staged rows that are ever read
+    const int wdelta = SHIFTED ? 0 : delta;                     // .. inside the staged band
+    const int need = TR + wdelta + S::SPAN;                     // staged rows that are ever read
     const int base = row0 + s0[0];                              // first staged row of B
     // Every slot of the unit pairs row i with row i + s0 + j of B: with the
     // whole band outside B the unit stores no matrix element, and there is
     // nothing to compute or to write (the whole workgroup leaves together).
     if (base + need <= 0 || base >= w) return;
+    // .. and with every row of the tile (a shifted pair: and every row delta above) past A's last
+    if (row0 - (SHIFTED ? delta : 0) >= h) return;
     const int myrow = row0 + 4 * lane;
 
     // C values this lane will combine at the end: row row0 + 64*wave + lane of
@@ -1788,9 +1806,9 @@ __device__ __forceinline__ void dd2dia_unit(
     // where no matrix element sits.
     auto c_offset = [&](int n, int j) -> unsigned {
         const int sl = slots[n][j];
-        const int o = row0 + 64 * wave + lane;
+        const int o = row0 + 64 * wave + lane - ((SHIFTED && n) ? delta : 0);
         const int in = o + s0[n] + j;
-        const bool ok = (wave < 4) & (sl >= 0) & (o < h) & (in >= 0) & (in < w) & (64 * wave + lane < TR);
+        const bool ok = (wave < 4) & (sl >= 0) & (o >= 0) & (o < h) & (in >= 0) & (in < w) & (64 * wave + lane < TR);
         return ok ? ((unsigned)sl * (unsigned)stride + (unsigned)o) * 4u : OOB_OFFSET;
     };
     float cpre[NCH][LC];
@@ -1838,6 +1856,8 @@ __device__ __forceinline__ void dd2dia_unit(
         rare_hi = max(rare_hi, rare_lo);
     }
     unsigned a_off[4];
+    unsigned a_off2 = OOB_OFFSET;                     // a shifted pair: the rows delta above (delta is a multiple of 4)
+    if (SHIFTED) a_off2 = ((myrow - delta >= 0) & (myrow - delta + 3 < h) & (4 * lane + 3 < TR)) ? (unsigned)(myrow - delta) * 4u : OOB_OFFSET;
     if (AVEC) {
         a_off[0] = ((myrow + 3 < h) & (4 * lane + 3 < TR)) ? (unsigned)myrow * 4u : OOB_OFFSET;
     } else {
@@ -1870,7 +1890,7 @@ __device__ __forceinline__ void dd2dia_unit(
     float4 bq[DD_BG][NB];
     // requests column i of group g: B rows into bq, A rows into st.a
     const unsigned rare_span = (unsigned)(rare_hi - rare_lo);
-    auto issue_col = [&](int g, int i, DdStage &st) {
+    auto issue_col = [&](int g, int i, DdStage<NA> &st) {
         const int b0 = __builtin_amdgcn_readfirstlane(g * DD_BG);   // wave-uniform: keeps column offsets scalar
         const int col = b0 + i;
         const bool live = (unsigned)(col - rare_lo) < rare_span;      // rare_lo <= col < rare_hi in one compare
@@ -1886,14 +1906,18 @@ __device__ __forceinline__ void dd2dia_unit(
         const unsigned cola = (unsigned)col * lda4;
         if (AVEC) {
             const float4 v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[0], cola, 0));
-            st.a[i][0] = v.x; st.a[i][1] = v.y; st.a[i][2] = v.z; st.a[i][3] = v.w;
+            st.a[0][i][0] = v.x; st.a[0][i][1] = v.y; st.a[0][i][2] = v.z; st.a[0][i][3] = v.w;
+            if constexpr (SHIFTED) {
+                const float4 u = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off2, cola, 0));
+                st.a[1][i][0] = u.x; st.a[1][i][1] = u.y; st.a[1][i][2] = u.z; st.a[1][i][3] = u.w;
+            }
         } else {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                st.a[i][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, a_off[t], cola, 0));
+                st.a[0][i][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, a_off[t], cola, 0));
         }
     };
-    auto issue = [&](int g, DdStage &st) {
+    auto issue = [&](int g, DdStage<NA> &st) {
 #pragma unroll
         for (int i = 0; i < DD_BG; ++i) issue_col(g, i, st);
     };
@@ -1907,10 +1931,10 @@ __device__ __forceinline__ void dd2dia_unit(
             *reinterpret_cast<float4 *>(tail2 ? buf + i * PITCH + 512 + 4 * lane : mybuf + 2 * DD_BG * PITCH) = bq[i][2];
         wave_lds_fence();
     };
-    struct Windows { float w[NCH][WQ * 4]; };
+    struct Windows { float w[NWIN][WQ * 4]; };
     auto read_windows = [&](Windows &win, const float *buf, int i) {
 #pragma unroll
-        for (int n = 0; n < NCH; ++n) {
+        for (int n = 0; n < NWIN; ++n) {
             const float4 *p4 = reinterpret_cast<const float4 *>(buf + i * PITCH + 4 * lane + (n ? delta : 0));
 #pragma unroll
             for (int q = 0; q < WQ; ++q) {
@@ -1919,13 +1943,16 @@ __device__ __forceinline__ void dd2dia_unit(
             }
         }
     };
-    auto fmas = [&](const float (&a)[4], const Windows &win) {
+    // column i of a stage: the first chunk on the lane's rows; the second on the same rows and its own window,
+    // or (a shifted pair) on the rows delta above and the same window
+    auto fmas = [&](const DdStage<NA> &st, int i, const Windows &win) {
 #pragma unroll
         for (int n = 0; n < NCH; ++n)
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int j = 0; j < LC; ++j) acc[n][t][j] = __builtin_fmaf(a[t], win.w[n][t + j], acc[n][t][j]);
+                for (int j = 0; j < LC; ++j)
+                    acc[n][t][j] = __builtin_fmaf(st.a[SHIFTED ? n : 0][i][t], win.w[SHIFTED ? 0 : n][t + j], acc[n][t][j]);
     };
     // Step k works on group wave + WAVES*k out of stage set k & 1 and LDS
     // buffer k & 1, one column at a time: column i's rows of B go to LDS and
@@ -1933,7 +1960,7 @@ __device__ __forceinline__ void dd2dia_unit(
     // of the next group is requested right after, so every load has one whole
     // step to arrive and the requests are spread between the FMA blocks.  Past
     // the last group the requests hit the empty resource.
-    auto step = [&](int k, int par, DdStage &cur, DdStage &nxt) {
+    auto step = [&](int k, int par, DdStage<NA> &cur, DdStage<NA> &nxt) {
         const float *buf = mybuf + par * (DD_BG * PITCH);
         const int gn = wave + WAVES * (k + 1);
         Windows w0, w1;
@@ -1943,27 +1970,27 @@ __device__ __forceinline__ void dd2dia_unit(
         read_windows(w1, buf, 1);
         issue_col(gn, 0, nxt);
         __builtin_amdgcn_sched_barrier(0);
-        fmas(cur.a[0], w0);
+        fmas(cur, 0, w0);
         __builtin_amdgcn_sched_barrier(0);
         commit_col(par, 2);
         read_windows(w0, buf, 2);
         issue_col(gn, 1, nxt);
         __builtin_amdgcn_sched_barrier(0);
-        fmas(cur.a[1], w1);
+        fmas(cur, 1, w1);
         __builtin_amdgcn_sched_barrier(0);
         commit_col(par, 3);
         read_windows(w1, buf, 3);
         issue_col(gn, 2, nxt);
         __builtin_amdgcn_sched_barrier(0);
-        fmas(cur.a[2], w0);
+        fmas(cur, 2, w0);
         __builtin_amdgcn_sched_barrier(0);
         issue_col(gn, 3, nxt);
         __builtin_amdgcn_sched_barrier(0);
-        fmas(cur.a[3], w1);
+        fmas(cur, 3, w1);
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    DdStage st0, st1;
+    DdStage<NA> st0, st1;
     issue(wave, st0);
     // The columns left out above, while the first group's loads are on their
     // way: wave 0 fetches its 4 rows of A and, value by value, its windows of
@@ -1976,7 +2003,7 @@ __device__ __forceinline__ void dd2dia_unit(
             const unsigned colb = (unsigned)col * ldb4;
             Windows win;
 #pragma unroll
-            for (int n = 0; n < NCH; ++n)
+            for (int n = 0; n < NWIN; ++n)
 #pragma unroll
                 for (int q = 0; q < WQ * 4; ++q) {
                     const int r = base + 4 * lane + (n ? delta : 0) + q;
@@ -1985,12 +2012,16 @@ __device__ __forceinline__ void dd2dia_unit(
                 }
             const __amdgpu_buffer_rsrc_t ar = make_rsrc(A, a_bytes);
             const unsigned cola = (unsigned)col * lda4;
-            float a[4];
+            DdStage<NA> one;
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                a[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    ar, ((myrow + t < h) & (4 * lane + t < TR)) ? (unsigned)(myrow + t) * 4u + cola : OOB_OFFSET, 0, 0));
-            fmas(a, win);
+            for (int n = 0; n < NA; ++n)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int r = myrow - (n ? delta : 0) + t;
+                    one.a[n][0][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        ar, ((r >= 0) & (r < h) & (4 * lane + t < TR)) ? (unsigned)r * 4u + cola : OOB_OFFSET, 0, 0));
+                }
+            fmas(one, 0, win);
         }
     }
     int k = 0;
@@ -2026,28 +2057,31 @@ __device__ __forceinline__ void dd2dia_unit(
                     acc[n][t][j] += red[wave * RED_WAVE + t * RED_T + (n * LC + j) * 64 + lane];
         // no barrier needed here: below, wave q overwrites only the block it has just read
     }
+    // (a shifted pair: one chunk after the other through the block of a single chunk)
 #pragma unroll
-    for (int n = 0; n < NCH; ++n)
+    for (int n0 = 0; n0 < NCH; n0 += NRED) {
+        if (n0 > 0) __syncthreads();                // the block is free again
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int n = 0; n < NRED; ++n)
 #pragma unroll
-            for (int j = 0; j < LC; ++j)
-                red[wave * RED_WAVE + t * RED_T + (n * LC + j) * 64 + lane] = acc[n][t][j];
-    __syncthreads();
-    {
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int j = 0; j < LC; ++j)
+                    red[wave * RED_WAVE + t * RED_T + (n * LC + j) * 64 + lane] = acc[n0 + n][t][j];
+        __syncthreads();
         const int r = 64 * wave + lane;             // row within the tile: lane r/4 owned it as its row r%4
         const float *src = red + (r & 3) * RED_T + (r >> 2);
 #pragma unroll
-        for (int n = 0; n < NCH; ++n)
+        for (int n = 0; n < NRED; ++n)
 #pragma unroll
             for (int j = 0; j < LC; ++j) {
                 float total = src[(n * LC + j) * 64];
 #pragma unroll
                 for (int p = 1; p < 4; ++p) total += src[p * RED_WAVE + (n * LC + j) * 64];
-                const unsigned off = c_offset(n, j);
+                const unsigned off = c_offset(n0 + n, j);
                 if (off != OOB_OFFSET) {
                     float *cd = reinterpret_cast<float *>(reinterpret_cast<char *>(C) + off);
-                    stream_store(cd, (beta == 0.f) ? alpha * total : beta * cpre[n][j] + alpha * total);
+                    stream_store(cd, (beta == 0.f) ? alpha * total : beta * cpre[n0 + n][j] + alpha * total);
                 }
             }
     }
@@ -2064,16 +2098,16 @@ struct DdBlock {
 // PAIRS = false: every unit is a single chunk, 4 waves per workgroup.
 // PAIRS = true: 8 waves per workgroup; a workgroup whose unit is a single
 // chunk retires its upper four waves at once.
-template <int LC, bool AVEC, bool PAIRS, bool WIDE = false>
-__global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
+template <int LC, bool AVEC, bool PAIRS, int WIDE = DD_NARROW>
+__global__ __launch_bounds__((PAIRS && WIDE != DD_SHIFTED) ? 512 : 256) void dd2dia_tiled_kernel(
     const Chunk *__restrict__ chunks, const Unit *__restrict__ units, int nunits,
     float *__restrict__ C, int stride,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
     int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes,
-    unsigned c_bytes, int blocked)
+    unsigned c_bytes, int blocked, int h_tiles)
 {
     constexpr int NCH_MAX = PAIRS ? 2 : 1;
-    static_assert(PAIRS || !WIDE, "only pairs are wide");
+    static_assert(PAIRS || WIDE == DD_NARROW, "only pairs come in forms");
     constexpr int LDS_FLOATS = dd_lds_floats<LC, NCH_MAX, WIDE>() > dd_lds_floats<LC, 1>() ? dd_lds_floats<LC, NCH_MAX, WIDE>()
                                                                                            : dd_lds_floats<LC, 1>();
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
@@ -2102,8 +2136,10 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
     rowtile = rblk * rb + pos / ub;
     unit = ublk * ub + pos % ub;
     }
-    constexpr int TR = PAIRS ? DD_ROWS : dd_short_rows<LC>();        // rows of a tile
-    if (rowtile * TR >= h || unit >= nunits) return;
+    constexpr int TR = (PAIRS && WIDE != DD_SHIFTED) ? DD_ROWS : dd_short_rows<LC>();        // rows of a tile
+    // h_tiles: row tiles of the launch -- those of A's rows, and for shifted pairs the tiles past them whose second
+    // chunk still works on rows of A
+    if (rowtile >= h_tiles || unit >= nunits) return;
     typedef const Unit __attribute__((address_space(4))) *sc_unit_ptr;
     const sc_unit_ptr u = (sc_unit_ptr)units + unit;
     const int c1 = u->c1, c2 = u->c2;
@@ -2116,7 +2152,8 @@ __global__ __launch_bounds__(PAIRS ? 512 : 256) void dd2dia_tiled_kernel(
         }
     }
     if (PAIRS && threadIdx.x >= 256) return;
-    dd2dia_unit<LC, 1, AVEC, false, !PAIRS>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
+    if (row0 >= h) return;
+    dd2dia_unit<LC, 1, AVEC, DD_NARROW, !PAIRS || WIDE == DD_SHIFTED>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
                              alpha, beta, a_bytes, b_bytes, c_bytes);
 }
 
@@ -2444,14 +2481,21 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     // than two that cannot pair): the same registers as a pair, half the
     // loads and LDS traffic per FMA.  (16-byte loads of A only, as for pairs.)
     const bool long_chunks = C.max_len_n > CHUNK_MAX && a_vec;
-    const bool pairs = use_units && !long_chunks;
-    const bool wide = pairs && C.pair_delta_max > PAIR_NARROW_DELTA;      // some pair needs the 520-row band
+    // A table with a pair further apart than one band holds runs the form that shares B's rows instead of A's
+    // (DD_SHIFTED) -- if its chunks have at least 4 shifts: pairs of shorter ones measured slower than the chunks on
+    // their own (3 x 3 windows on a 512-wide map: 409 against 310 us at batch 512), so those stay single.  Pairs that
+    // fit a band keep the forms that share A's rows: the band forms run a 7 x 7 window on a 128-wide map at batch
+    // 2048 in 81 us, the shifted form in 145.
+    const bool far = use_units && !long_chunks && C.pair_delta_max > PAIR_BAND_DELTA;
+    const bool shifted = far && C.max_len_p >= 4;
+    const bool pairs = use_units && !long_chunks && (!far || shifted);
+    const bool wide = pairs && !shifted && C.pair_delta_max > PAIR_NARROW_DELTA;      // some pair needs the 520-row band
     const Unit *units = pairs ? C.units_dev : C.single_units_dev;      // the single units count 0, 1, 2, ...
     const int nunits = long_chunks ? C.n_chunks_n : pairs ? C.n_units : C.n_chunks_p;
     const Chunk *table = long_chunks ? C.chunks_n_dev : C.chunks_p_dev;
     const int lc = long_chunks ? C.max_len_n : C.max_len_p;
-    const int tile_rows = pairs ? DD_ROWS : lc > CHUNK_MAX ? dd_short_rows<SP_CHUNK_MAX>() : dd_short_rows<CHUNK_MAX>();
-    const long long row_tiles = (C.h + tile_rows - 1) / tile_rows;
+    const int tile_rows = (pairs && !shifted) ? DD_ROWS : lc > CHUNK_MAX ? dd_short_rows<SP_CHUNK_MAX>() : dd_short_rows<CHUNK_MAX>();
+    const long long row_tiles = ((long long)C.h + (shifted ? C.pair_delta_max : 0) + tile_rows - 1) / tile_rows;
     const int ub = DdBlock::units(nunits), rb = DdBlock::rows(nunits);
     const int blocked = row_tiles * nunits > DD_BLOCKED_MIN_TILES ? 1 : 0;
     const long long blocks = blocked ? ((row_tiles + rb - 1) / rb) * ((nunits + ub - 1) / ub) * (long long)(rb * ub)
@@ -2459,11 +2503,13 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks);
 #define CUVDIA_DD_ARGS table, units, nunits, vals, C.stride, A, lda, B, ldb, C.h, C.w, batch, alpha, beta, \
-                       a_bytes, b_bytes, c_bytes, blocked
+                       a_bytes, b_bytes, c_bytes, blocked, (int)row_tiles
 #define CUVDIA_DD_LAUNCH(L)                                                                              \
     case L:                                                                                              \
-        if (wide) {                                                                                      \
-            hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, true, true>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
+        if (shifted) {                                                                                   \
+            hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, true, DD_SHIFTED>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);  \
+        } else if (wide) {                                                                               \
+            hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, true, DD_WIDE>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
         } else if (pairs) {                                                                              \
             hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, true>), grid, dim3(512), 0, stream, CUVDIA_DD_ARGS);  \
         } else {                                                                                         \

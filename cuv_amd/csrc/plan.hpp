@@ -52,11 +52,13 @@ std::vector<Chunk> plan_chunks(const int *offsets, int nd, bool transposed, int 
 
 // A unit of work of the tiled dense x dense^T projection: one chunk, or two
 // chunks of the normal table whose first shifts differ by a multiple of 4 of
-// at most PAIR_MAX_DELTA rows.  A wave serves both chunks of a pair from one
-// staged band of the second operand and one copy of the first operand's rows.
-// Up to PAIR_NARROW_DELTA rows apart the band fits two 16-byte pieces per lane
-// and column; a table with a wider pair runs the kernel that takes three.
-constexpr int PAIR_MAX_DELTA = 256;
+// at most PAIR_MAX_DELTA rows.  Up to PAIR_BAND_DELTA rows apart a wave can serve both chunks of a pair from one
+// staged band of the second operand and one copy of the first operand's rows (up to PAIR_NARROW_DELTA the band
+// fits two 16-byte pieces per lane and column; a table with a wider pair runs the kernel that takes three).  At any
+// distance it can let the second chunk work on the rows that far above the first's: both then read the same rows of
+// the second operand (window rows of a map of any width).
+constexpr int PAIR_MAX_DELTA = 4096;
+constexpr int PAIR_BAND_DELTA = 256;
 constexpr int PAIR_NARROW_DELTA = 128;
 struct Unit {
     int c1;                 // chunk index

@@ -104,8 +104,11 @@ int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
 /* Pure host function: the work units the tiled dense x dense^T projection
  * walks.  A unit is one chunk of the normal (transposed == 0) chunk table, or
  * two chunks adjacent in that table whose first shifts differ by a positive
- * multiple of 4 of at most 256 rows (two rows of a 2-d window): a wave serves
- * both from one staged band of the second operand.  c1[u] is the unit's chunk
+ * multiple of 4 of at most 4096 rows (two rows of a 2-d window): up to 256
+ * rows apart a wave serves both from one staged band of the second operand and
+ * one copy of the first operand's rows; further apart the second chunk works
+ * on the rows that far above the first's, so that both read the same rows of
+ * the second operand.  c1[u] is the unit's chunk
  * index, c2[u] its second chunk or -1.  Returns the number of units (also when
  * it exceeds cap; then nothing is written), or a negative error.  The role of
  * the block list built in src/cuv/matrix_ops/densedense_to_sparse.cu:123-171. */

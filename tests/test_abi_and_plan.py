@@ -179,10 +179,13 @@ def test_units_pair_window_rows():
 
 
 def test_units_pairing_rule():
-    # first shifts 8 apart (multiple of 4, <= 256): a pair; 7 apart or 260 apart: singles
+    # first shifts a multiple of 4 and at most 4096 apart: a pair; 7 apart, 258 apart or 4100 apart: singles
     assert _units(list(range(-8, -1)) + list(range(0, 8))) == [(0, 1)]
     assert _units(list(range(0, 13))) == [(0, -1), (1, -1)]                 # one run of 13 -> chunks 7 + 6, shifts 7 apart
-    assert _units([0, 1, 260, 261]) == [(0, -1), (1, -1)]
+    assert _units([0, 1, 258, 259]) == [(0, -1), (1, -1)]
+    assert _units([0, 1, 260, 261]) == [(0, 1)]
+    assert _units([0, 1, 4096, 4097]) == [(0, 1)]
+    assert _units([0, 1, 4100, 4101]) == [(0, -1), (1, -1)]
     assert _units([0, 1, 132, 133]) == [(0, 1)]
     assert _units([0, 1, 256, 257, 512]) == [(0, 1), (2, -1)]
     assert _units([0, 1, 128, 129, 256]) == [(0, 1), (2, -1)]

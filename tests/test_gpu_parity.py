@@ -117,6 +117,18 @@ SHAPES = [
     (1800, 1024, [dy * 256 + dx for dy in range(-2, 2) for dx in range(0, 7)], 1, 130),
     (900, 900, [dy * 192 + dx for dy in range(-2, 3) for dx in range(-3, 4)], 1, 17),
     (1111, 1300, [0, 1, 2, 64, 65, 66, 320, 321, 576, 577, 578, 1000], 1, 41),
+    # pairs further apart than a band holds (the second chunk works on the rows that far above the first's):
+    # window rows 512 and 1024 apart, square and rectangular both ways; a table that mixes a near pair, a far pair
+    # and a single; chunks 4096 apart on a matrix with fewer rows than that; rows that end inside the last tile;
+    # chunks of 3 that far apart (which stay single)
+    (4096, 4096, [dy * 512 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 1, 40),
+    (3000, 5000, [dy * 1024 + dx for dy in range(-2, 3) for dx in range(0, 5)], 1, 33),
+    (5000, 3000, [dy * 1024 + dx for dy in range(-2, 3) for dx in range(-4, 1)], 1, 64),
+    (3500, 3500, [0, 1, 2, 3, 64, 65, 66, 67, 1000, 1001, 1002, 1003, 1400, 1401, 1402, 1403, 3000], 1, 72),
+    (2000, 9000, [0, 1, 2, 3, 4096, 4097, 4098, 4099], 1, 17),
+    (1501, 1700, [dy * 600 + dx for dy in range(-1, 2) for dx in range(0, 4)], 1, 130),
+    (1500, 1700, [dy * 600 + dx for dy in range(-1, 2) for dx in range(0, 4)], 1, 130),
+    (2048, 2048, [dy * 512 + dx for dy in range(-1, 2) for dx in range(-1, 2)], 1, 24),
     # window rows a multiple of the 64-row tile apart: square, rectangular both ways, a window with
     # missing rows, ragged batch
     (2048, 2048, [dy * 64 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 1, 70),
