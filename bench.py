@@ -518,7 +518,7 @@ def main():
     # algorithmic bytes of the two products / their two durations -- which is
     # also what a profiler's per-kernel average duration corresponds to.
     kernel_names = {"up_pass": "spmm_tiled_kernel<7, 8, 1, false>", "down_pass": "spmm_tiled_kernel<7, 8, 1, false>",
-                    "weight_gradient": "dd2dia_tiled_kernel<7, true, true>"}
+                    "weight_gradient": "dd2dia_tiled_kernel<7, true, true, 0>"}
     traffic, traffic_rev = load_traffic()
     for name in per:
         per[name]["kernel"] = kernel_names[name]
