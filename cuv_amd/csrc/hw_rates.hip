@@ -50,6 +50,7 @@ __global__ __launch_bounds__(256) void fma_kernel(float *out, long long *clk, in
     //   7 -- sums in consecutive registers, both multiplicands in bank 0
     //   8 -- sums in banks 2 and 3, both multiplicands in bank 0
     //   9 -- all three operands in bank 0
+    //   10, 11 -- the DPP form with its two multiplicands in banks 0 and 1, and both in bank 0
     if (FORM >= 5) {
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
@@ -149,6 +150,46 @@ __global__ __launch_bounds__(256) void fma_kernel(float *out, long long *clk, in
                     "v_fmac_f32 v164, v100, v104\n\t"
                     "v_fmac_f32 v168, v100, v104\n\t"
                     ::: "v100", "v104", "v108", "v112", "v116", "v120", "v124", "v128", "v132", "v136", "v140", "v144", "v148", "v152", "v156", "v160", "v164", "v168");
+                if (FORM == 10)
+                asm volatile(
+                    "s_nop 1\n\t"
+                    "v_fmac_f32_dpp v108, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v109, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v110, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v111, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v112, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v113, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v114, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v115, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v116, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v117, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v118, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v119, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v120, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v121, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v122, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v123, v100, v101 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    ::: "v100", "v101", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123");
+                if (FORM == 11)
+                asm volatile(
+                    "s_nop 1\n\t"
+                    "v_fmac_f32_dpp v108, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v109, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v110, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v111, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v112, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v113, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v114, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v115, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v116, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v117, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v118, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v119, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v120, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v121, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v122, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    "v_fmac_f32_dpp v123, v100, v104 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+                    ::: "v100", "v104", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123");
             }
         }
     }
@@ -376,6 +417,8 @@ int main()
     if (run_fma<7>(p, "v v v: sums consecutive, a b bank 0")) return 1;
     if (run_fma<8>(p, "v v v: sums banks 2 3, a b bank 0")) return 1;
     if (run_fma<9>(p, "v v v: all in bank 0")) return 1;
+    if (run_fma<10>(p, "dpp: sums consecutive, a b banks 0 1")) return 1;
+    if (run_fma<11>(p, "dpp: sums consecutive, a b bank 0")) return 1;
     if (run_fma<3>(p, "v_fmac_f32 v, v, v (8 x 8 operands)")) return 1;
     if (run_fma<4>(p, "v_fmac_f32 v, v, v (4 x 16 operands)")) return 1;
     if (run_lds<4>(p, "ds_read_b128")) return 1;
