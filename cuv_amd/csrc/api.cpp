@@ -38,6 +38,9 @@ thread_local std::string t_hip_error;
 // Batches narrower than this go to the generic kernel: the tiled SpMM puts
 // one batch column on each of 64 lanes.
 constexpr int SPMM_TILED_MIN_BATCH = 24;
+// The rows-along-lanes kernel is the automatic choice from this many of its tiles (workgroups) and this batch.
+constexpr long long SPMM_ROWS_MIN_TILES = 1LL << 40;     // (not chosen automatically until measured)
+constexpr int SPMM_ROWS_MIN_BATCH = 32;
 // Largest h, w and |offset| the kernels' 32-bit row arithmetic allows.
 constexpr long long DIM_LIMIT = 1LL << 30;
 
@@ -119,7 +122,7 @@ const char *cuvdia_last_hip_error(void) { return t_hip_error.c_str(); }
 int cuvdia_set_path(int path)
 {
     if (path != CUVDIA_PATH_AUTO && path != CUVDIA_PATH_GENERIC && path != CUVDIA_PATH_TILED &&
-        path != CUVDIA_PATH_TILED_NOWALK && path != CUVDIA_PATH_WALK)
+        path != CUVDIA_PATH_TILED_NOWALK && path != CUVDIA_PATH_WALK && path != CUVDIA_PATH_ROWS)
         return CUVDIA_EINVAL;
     g_path.store(path);
     return CUVDIA_OK;
@@ -292,8 +295,12 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     };
     d->view.walk_n = walk_view(wn, wn_at);
     d->view.walk_t = walk_view(wt, wt_at);
-    auto span = [](const std::vector<Chunk> &t, int &max_len, int &s_min, int &s_max) {
+    auto span = [](const std::vector<Chunk> &t, int &max_len, int &s_min, int &s_max, int *min_len = nullptr) {
         max_len = 0;
+        if (min_len) {
+            *min_len = t.empty() ? 0 : t.front().len;
+            for (const Chunk &c : t) *min_len = std::min(*min_len, c.len);
+        }
         s_min = t.empty() ? 0 : t.front().s0;
         s_max = s_min;
         for (const Chunk &c : t) {
@@ -302,8 +309,8 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
             s_max = std::max(s_max, c.s0);
         }
     };
-    span(cn, d->view.max_len_n, d->view.s_min_n, d->view.s_max_n);
-    span(ct, d->view.max_len_t, d->view.s_min_t, d->view.s_max_t);
+    span(cn, d->view.max_len_n, d->view.s_min_n, d->view.s_max_n, &d->view.min_len_n);
+    span(ct, d->view.max_len_t, d->view.s_min_t, d->view.s_max_t, &d->view.min_len_t);
     d->view.slot_step_n = common_slot_step(cn);
     d->view.slot_step_t = common_slot_step(ct);
     int unused_min = 0, unused_max = 0;
@@ -352,6 +359,26 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const fl
     if (const int rc = check_device(desc)) return rc;
 
     const int forced = g_path.load();
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // The rows-along-lanes kernel: plain products of tables it serves (spmm_rows_ok).  Chosen when asked for,
+    // and by itself for products large enough to fill the chip with its tiles several times over.
+    {
+        const bool plain = bias == nullptr && act == CUVDIA_ACT_NONE;
+        const bool rows_possible = plain && spmm_rows_ok(desc->view, ldb, ldd, trans);
+        if (forced == CUVDIA_PATH_ROWS && !rows_possible) return CUVDIA_EUNSUPPORTED;
+        bool rows = forced == CUVDIA_PATH_ROWS;
+        if (forced == CUVDIA_PATH_AUTO && rows_possible) {
+            const int lck = trans ? desc->view.max_len_t : desc->view.max_len_n;
+            const long long tiles = ((long long)n_out + spmm_rows_tile_rows(lck) - 1) / spmm_rows_tile_rows(lck) *
+                                    (((long long)batch + 31) / 32);
+            rows = tiles >= SPMM_ROWS_MIN_TILES && batch >= SPMM_ROWS_MIN_BATCH;
+        }
+        if (rows) {
+            const hipError_t e = launch_spmm_rows(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, s);
+            t_last_path = CUVDIA_PATH_ROWS;
+            return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "spmm kernel launch");
+        }
+    }
     const bool tiled_possible = spmm_tiled_ok(desc->view, ldb, ldd, trans);
     bool tiled;
     if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
@@ -362,7 +389,6 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const fl
     } else {
         tiled = tiled_possible && batch >= SPMM_TILED_MIN_BATCH;
     }
-    hipStream_t s = static_cast<hipStream_t>(stream);
     bool walked = false;
     const int walk = forced == CUVDIA_PATH_WALK ? 1 : forced == CUVDIA_PATH_TILED_NOWALK ? -1 : 0;
     const hipError_t e = tiled
@@ -444,7 +470,8 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
         }
     }
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK ||
+        forced == CUVDIA_PATH_ROWS) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {
@@ -611,7 +638,7 @@ int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals, const int *offsets_host
 
     // the kernel family is chosen by the rule of cuvdia_spmm_layer_f32
     const int forced = g_path.load();
-    if (forced == CUVDIA_PATH_WALK) return CUVDIA_EUNSUPPORTED;
+    if (forced == CUVDIA_PATH_WALK || forced == CUVDIA_PATH_ROWS) return CUVDIA_EUNSUPPORTED;
     const bool tiled_possible = spmm_tiled_ok(view, ldb, ldd, trans);
     bool tiled;
     if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK) {
