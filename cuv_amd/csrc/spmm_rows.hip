@@ -31,6 +31,7 @@
 // acc = fma(a, x, acc); then dst = alpha*acc (beta == 0, dst not read) or fma(beta, dst, alpha*acc).
 #include <hip/hip_runtime.h>
 
+
 #include "kernels.hpp"
 
 namespace cuvdia {
@@ -42,40 +43,49 @@ constexpr int RW_WAVES = 8;
 constexpr int RW_COLS = RW_C * RW_WAVES;    // batch columns per workgroup
 constexpr int RW_LOADED = 64 * RW_T;        // rows a wave loads per column
 constexpr unsigned RW_OOB = 0x80000000u;    // a byte offset beyond every buffer resource used here
-constexpr int RW_MAX_CHUNKS = 256;
+constexpr int RW_MAX_CHUNKS = 64;         // the walk keeps table entry l in lane l
 
 constexpr int rw_valid_lanes(int lck) { return 64 - (lck - 1 + RW_T - 1) / RW_T; }
 constexpr int rw_tile_rows(int lck) { return RW_T * rw_valid_lanes(lck); }
-// LDS: two buffers of diagonal values, 2 x lck pieces of 1 KB each (piece 2 j + half: lane l's rows
+// LDS: three buffers of diagonal values (and a spare kilobyte behind them), 2 x lck pieces of 1 KB each (piece 2 j + half: lane l's rows
 // 8 l + 4 half .. + 3 of diagonal j at byte 16 l); at the end every wave passes its 4 x 512 sums through 8 KB.
 constexpr int rw_abuf_bytes(int lck) { return 2 * lck * 1024; }
-constexpr int rw_lds_bytes(int lck) { return 2 * rw_abuf_bytes(lck) > RW_WAVES * 8192 ? 2 * rw_abuf_bytes(lck) : RW_WAVES * 8192; }
+constexpr int rw_lds_bytes(int lck) { return 3 * rw_abuf_bytes(lck) + 1024 > RW_WAVES * 8192 ? 3 * rw_abuf_bytes(lck) + 1024 : RW_WAVES * 8192; }
 
 // ---- the named registers --------------------------------------------------------------------------------
+//   v32 ..  v63   own dense rows, set 2: RW_OWN2 + 8 c + k (the compiler's own values stay below v32: the
+//                 build checks the disassembly for that)
 //   v66 ..  v99   four buffers of 8 diagonal values (RW_A0, RW_A1: first register 2 mod 4; RW_A2, RW_A3: 0 mod 4)
 //   v100 .. v131  sums, RW_ACC + 8 c + t
 //   v132 .. v163  own dense rows, set 0: RW_OWN0 + 8 c + k      (window positions 0 .. 7)
-//   v164 .. v195  own dense rows, set 1 (chunks alternate between the sets: one is used while the other loads)
+//   v164 .. v195  own dense rows, set 1 (chunk i uses set i mod 3 while the sets of chunks i + 1 and i + 2 load)
 //   v196 .. v243  halo: RW_HALO + 12 c + m                      (window positions 8 + m)
+// Every statement begins with RW_DEFS (symbols and macros are per statement: the assembler keeps macros for the
+// whole translation unit, and a statement can be instantiated more than once) and ends with RW_PURGE.  The
+// statement sets RW_P (the own set of the chunk being computed), RW_Q (the set being loaded) and RW_LCK first.
 #define RW_DEFS \
     ".set RW_A0, 66\n.set RW_A1, 74\n.set RW_A2, 84\n.set RW_A3, 92\n" \
-    ".set RW_ACC, 100\n.set RW_OWN0, 132\n.set RW_OWN1, 164\n.set RW_HALO, 196\n" \
-    ".macro RW_FMAD p, j, ab\n" \
+    ".set RW_ACC, 100\n.set RW_OWN0, 132\n.set RW_OWN1, 164\n.set RW_OWN2, 32\n.set RW_HALO, 196\n" \
+    ".macro RW_SETS p, q\n" \
+    " .if \\p == 0\n .set RW_OWNP, RW_OWN0\n .endif\n .if \\p == 1\n .set RW_OWNP, RW_OWN1\n .endif\n .if \\p == 2\n .set RW_OWNP, RW_OWN2\n .endif\n" \
+    " .if \\q == 0\n .set RW_OWNQ, RW_OWN0\n .endif\n .if \\q == 1\n .set RW_OWNQ, RW_OWN1\n .endif\n .if \\q == 2\n .set RW_OWNQ, RW_OWN2\n .endif\n" \
+    ".endm\n" \
+    ".macro RW_FMAD j, ab\n" \
     " .irp c,0,1,2,3\n" \
     "  .irp t,0,1,2,3,4,5,6,7\n" \
     "   .if (\\t+\\j) < 8\n" \
-    "     v_fmac_f32 v[RW_ACC+8*\\c+\\t], v[\\ab+\\t], v[RW_OWN\\p+8*\\c+\\t+\\j]\n" \
+    "     v_fmac_f32 v[RW_ACC+8*\\c+\\t], v[\\ab+\\t], v[RW_OWNP+8*\\c+\\t+\\j]\n" \
     "   .else\n" \
     "     v_fmac_f32 v[RW_ACC+8*\\c+\\t], v[\\ab+\\t], v[RW_HALO+12*\\c+\\t+\\j-8]\n" \
     "   .endif\n" \
     "  .endr\n" \
     " .endr\n" \
     ".endm\n" \
-    ".macro RW_HALOS p, n\n" \
+    ".macro RW_HALOS n\n" \
     " .irp c,0,1,2,3\n" \
     "  .irp k,0,1,2,3,4,5,6,7\n" \
     "   .if \\k < \\n\n" \
-    "   v_mov_b32_dpp v[RW_HALO+12*\\c+\\k], v[RW_OWN\\p+8*\\c+\\k] wave_shl:1 row_mask:0xf bank_mask:0xf\n" \
+    "   v_mov_b32_dpp v[RW_HALO+12*\\c+\\k], v[RW_OWNP+8*\\c+\\k] wave_shl:1 row_mask:0xf bank_mask:0xf\n" \
     "   .endif\n" \
     "  .endr\n" \
     " .endr\n" \
@@ -87,30 +97,38 @@ constexpr int rw_lds_bytes(int lck) { return 2 * rw_abuf_bytes(lck) > RW_WAVES *
     "  .endr\n" \
     " .endr\n" \
     ".endm\n" \
-    ".macro RW_AREAD ab, j, vaddr, base\n" \
-    "  ds_read_b128 v[\\ab:\\ab+3], \\vaddr offset:\\base+\\j*2048\n" \
-    "  ds_read_b128 v[\\ab+4:\\ab+7], \\vaddr offset:\\base+\\j*2048+1024\n" \
+    ".macro RW_AREAD ab, j, vaddr\n" \
+    "  ds_read_b128 v[\\ab:\\ab+3], \\vaddr offset:\\j*2048\n" \
+    "  ds_read_b128 v[\\ab+4:\\ab+7], \\vaddr offset:\\j*2048+1024\n" \
     ".endm\n" \
-    ".macro RW_AREADJ j, vaddr, base\n" \
-    " .if ((\\j) & 3) == 0\n RW_AREAD RW_A0, (\\j), \\vaddr, \\base\n .endif\n" \
-    " .if ((\\j) & 3) == 1\n RW_AREAD RW_A1, (\\j), \\vaddr, \\base\n .endif\n" \
-    " .if ((\\j) & 3) == 2\n RW_AREAD RW_A2, (\\j), \\vaddr, \\base\n .endif\n" \
-    " .if ((\\j) & 3) == 3\n RW_AREAD RW_A3, (\\j), \\vaddr, \\base\n .endif\n" \
+    ".macro RW_AREADJ j, vaddr\n" \
+    " .if ((\\j) & 3) == 0\n RW_AREAD RW_A0, (\\j), \\vaddr\n .endif\n" \
+    " .if ((\\j) & 3) == 1\n RW_AREAD RW_A1, (\\j), \\vaddr\n .endif\n" \
+    " .if ((\\j) & 3) == 2\n RW_AREAD RW_A2, (\\j), \\vaddr\n .endif\n" \
+    " .if ((\\j) & 3) == 3\n RW_AREAD RW_A3, (\\j), \\vaddr\n .endif\n" \
     ".endm\n" \
-    ".macro RW_FMADJ p, j\n" \
-    " .if ((\\j) & 3) == 0\n RW_FMAD \\p, \\j, RW_A0\n .endif\n" \
-    " .if ((\\j) & 3) == 1\n RW_FMAD \\p, \\j, RW_A1\n .endif\n" \
-    " .if ((\\j) & 3) == 2\n RW_FMAD \\p, \\j, RW_A2\n .endif\n" \
-    " .if ((\\j) & 3) == 3\n RW_FMAD \\p, \\j, RW_A3\n .endif\n" \
+    ".macro RW_FMADJ j\n" \
+    " .if ((\\j) & 3) == 0\n RW_FMAD \\j, RW_A0\n .endif\n" \
+    " .if ((\\j) & 3) == 1\n RW_FMAD \\j, RW_A1\n .endif\n" \
+    " .if ((\\j) & 3) == 2\n RW_FMAD \\j, RW_A2\n .endif\n" \
+    " .if ((\\j) & 3) == 3\n RW_FMAD \\j, RW_A3\n .endif\n" \
+    ".endm\n" \
+    ".macro RW_XLOAD n, voff, rsrc, soff\n" \
+    " .if ((\\n) & 1) == 0\n" \
+    "  buffer_load_dwordx4 v[RW_OWNQ+4*(\\n):RW_OWNQ+4*(\\n)+3], \\voff, \\rsrc, \\soff offen\n" \
+    " .else\n" \
+    "  buffer_load_dwordx4 v[RW_OWNQ+4*(\\n):RW_OWNQ+4*(\\n)+3], \\voff, \\rsrc, \\soff offen offset:16\n" \
+    " .endif\n" \
     ".endm\n"
-#define RW_PURGE ".purgem RW_FMAD\n.purgem RW_HALOS\n.purgem RW_AREAD\n.purgem RW_AREADJ\n.purgem RW_FMADJ\n"
+#define RW_PURGE ".purgem RW_SETS\n.purgem RW_FMAD\n.purgem RW_HALOS\n.purgem RW_AREAD\n.purgem RW_AREADJ\n.purgem RW_FMADJ\n.purgem RW_XLOAD\n"
 
+#define RW_CLOB_OWN2 "v32","v33","v34","v35","v36","v37","v38","v39","v40","v41","v42","v43","v44","v45","v46","v47","v48","v49","v50","v51","v52","v53","v54","v55","v56","v57","v58","v59","v60","v61","v62","v63"
 #define RW_CLOB_A "v66","v67","v68","v69","v70","v71","v72","v73","v74","v75","v76","v77","v78","v79","v80","v81","v82","v83","v84","v85","v86","v87","v88","v89","v90","v91","v92","v93","v94","v95","v96","v97","v98","v99"
 #define RW_CLOB_ACC "v100","v101","v102","v103","v104","v105","v106","v107","v108","v109","v110","v111","v112","v113","v114","v115","v116","v117","v118","v119","v120","v121","v122","v123","v124","v125","v126","v127","v128","v129","v130","v131"
 #define RW_CLOB_OWN0 "v132","v133","v134","v135","v136","v137","v138","v139","v140","v141","v142","v143","v144","v145","v146","v147","v148","v149","v150","v151","v152","v153","v154","v155","v156","v157","v158","v159","v160","v161","v162","v163"
 #define RW_CLOB_OWN1 "v164","v165","v166","v167","v168","v169","v170","v171","v172","v173","v174","v175","v176","v177","v178","v179","v180","v181","v182","v183","v184","v185","v186","v187","v188","v189","v190","v191","v192","v193","v194","v195"
 #define RW_CLOB_HALO "v196","v197","v198","v199","v200","v201","v202","v203","v204","v205","v206","v207","v208","v209","v210","v211","v212","v213","v214","v215","v216","v217","v218","v219","v220","v221","v222","v223","v224","v225","v226","v227","v228","v229","v230","v231","v232","v233","v234","v235","v236","v237","v238","v239","v240","v241","v242","v243"
-#define RW_CLOB_ALL RW_CLOB_A, RW_CLOB_ACC, RW_CLOB_OWN0, RW_CLOB_OWN1, RW_CLOB_HALO
+#define RW_CLOB_ALL RW_CLOB_OWN2, RW_CLOB_A, RW_CLOB_ACC, RW_CLOB_OWN0, RW_CLOB_OWN1, RW_CLOB_HALO
 
 typedef int rw_int4 __attribute__((ext_vector_type(4)));
 
@@ -172,87 +190,116 @@ __device__ __forceinline__ void rw_lds_load_b32(rw_int4 rsrc, unsigned lds_byte_
                  :: "s"(lds_byte_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 
-// The arithmetic of one chunk: own set P (0 / 1), its diagonal values in LDS at byte BASE of the value block;
-// WPAR says on which diagonals this wave takes the higher priority.
-#define RW_DIAG(P, J, LAST) \
-    ".if " #J " < " #LAST "\n RW_AREADJ (" #J "+1), %0, %1\n s_waitcnt lgkmcnt(2)\n .else\n s_waitcnt lgkmcnt(0)\n .endif\n" \
-    ".if ((" #J " ^ %2) & 1)\n s_setprio 0\n .else\n s_setprio 3\n .endif\n" \
-    "RW_FMADJ " #P ", " #J "\n"
-#define RW_CHUNK7(P) \
-    RW_DEFS "RW_AREADJ 0, %0, %1\n RW_HALOS " #P ", 6\n" \
-    RW_DIAG(P, 0, 6) RW_DIAG(P, 1, 6) RW_DIAG(P, 2, 6) RW_DIAG(P, 3, 6) RW_DIAG(P, 4, 6) RW_DIAG(P, 5, 6) RW_DIAG(P, 6, 6) \
-    "s_setprio 0\n" RW_PURGE
-#define RW_CHUNK13(P) \
-    RW_DEFS "RW_AREADJ 0, %0, %1\n RW_HALOS " #P ", 12\n" \
-    RW_DIAG(P, 0, 12) RW_DIAG(P, 1, 12) RW_DIAG(P, 2, 12) RW_DIAG(P, 3, 12) RW_DIAG(P, 4, 12) RW_DIAG(P, 5, 12) RW_DIAG(P, 6, 12) \
-    RW_DIAG(P, 7, 12) RW_DIAG(P, 8, 12) RW_DIAG(P, 9, 12) RW_DIAG(P, 10, 12) RW_DIAG(P, 11, 12) RW_DIAG(P, 12, 12) \
-    "s_setprio 0\n" RW_PURGE
+// What a wave needs to request a chunk's operands: the dense rows of its 4 columns (8 loads of 16 bytes per
+// lane into own set Q) and its share of the chunk's diagonal values (NP loads that write LDS directly).
+struct RwRequest {
+    rw_int4 xr;                 // dense operand of the tile's columns (an empty resource: nothing is fetched, zeros arrive)
+    unsigned xs[RW_C];          // scalar byte offset of each column's first row
+    rw_int4 ar;                 // the diagonal values (or the empty resource)
+    unsigned as;                // scalar byte offset of the chunk's first diagonal, at the tile's first row
+    unsigned m0_base;           // LDS byte address of the wave's first piece in the value buffer
+    unsigned m0_last;           // .. of its last piece (the spare kilobyte where the wave has none)
+};
 
-template <int LCK, int P, int WPAR>
-__device__ __forceinline__ void rw_compute(unsigned a_read_addr)
-{
-    constexpr int BASE = P * rw_abuf_bytes(LCK);
-    static_assert(LCK == 7 || LCK == 13, "instantiated chunk lengths");
-    if constexpr (LCK == 7) {
-        if constexpr (P == 0) asm volatile(RW_CHUNK7(0) :: "v"(a_read_addr), "n"(BASE), "n"(WPAR) : "memory", RW_CLOB_ALL);
-        else asm volatile(RW_CHUNK7(1) :: "v"(a_read_addr), "n"(BASE), "n"(WPAR) : "memory", RW_CLOB_ALL);
-    } else {
-        if constexpr (P == 0) asm volatile(RW_CHUNK13(0) :: "v"(a_read_addr), "n"(BASE), "n"(WPAR) : "memory", RW_CLOB_ALL);
-        else asm volatile(RW_CHUNK13(1) :: "v"(a_read_addr), "n"(BASE), "n"(WPAR) : "memory", RW_CLOB_ALL);
-    }
-}
-
-// requests the wave's own dense rows of a chunk that lies wholly inside the operand: 8 loads of 16 bytes per lane
-template <int P>
-__device__ __forceinline__ void rw_load_own(unsigned voff, rw_int4 rsrc, unsigned s0, unsigned s1, unsigned s2, unsigned s3)
-{
-#define RW_OWN_LOADS(Q) \
-    RW_DEFS \
+// One diagonal of a chunk: the values of the diagonal after the next are read from LDS, this one's are waited for, the
+// two waves of a SIMD trade priority, a load or two of the chunk two steps ahead are issued, then 32 FMAs.
+// (requests per diagonal: chunks of 13 -- one per diagonal, the 8 dense loads first, then the pieces of
+// diagonal values; chunks of 7 -- two dense loads on each of the first four diagonals, a piece on the next two)
+#define RW_DIAG(J) \
+    ".if " #J " < RW_LCK\n" \
+    " .if " #J " + 2 < RW_LCK\n RW_AREADJ (" #J "+2), %[aread]\n s_waitcnt lgkmcnt(4)\n .else\n  .if " #J " + 1 < RW_LCK\n s_waitcnt lgkmcnt(2)\n  .else\n s_waitcnt lgkmcnt(0)\n  .endif\n .endif\n" \
+    " .if ((" #J " ^ RW_WPAR) & 1)\n s_setprio 0\n .else\n s_setprio 3\n .endif\n" \
+    " .if RW_LCK > 8\n" \
+    "  .if " #J " == 0\n RW_XLOAD 0, %[xvoff], %[xrs], %[xs0]\n .endif\n" \
+    "  .if " #J " == 1\n RW_XLOAD 1, %[xvoff], %[xrs], %[xs0]\n .endif\n" \
+    "  .if " #J " == 2\n RW_XLOAD 2, %[xvoff], %[xrs], %[xs1]\n .endif\n" \
+    "  .if " #J " == 3\n RW_XLOAD 3, %[xvoff], %[xrs], %[xs1]\n .endif\n" \
+    "  .if " #J " == 4\n RW_XLOAD 4, %[xvoff], %[xrs], %[xs2]\n .endif\n" \
+    "  .if " #J " == 5\n RW_XLOAD 5, %[xvoff], %[xrs], %[xs2]\n .endif\n" \
+    "  .if " #J " == 6\n RW_XLOAD 6, %[xvoff], %[xrs], %[xs3]\n .endif\n" \
+    "  .if " #J " == 7\n RW_XLOAD 7, %[xvoff], %[xrs], %[xs3]\n .endif\n" \
+    "  .if " #J " == 8\n s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n .endif\n" \
+    "  .if " #J " == 9\n s_add_u32 m0, %[m0base], 8192\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n .endif\n" \
+    "  .if " #J " == 10\n s_add_u32 m0, %[m0base], 16384\n s_nop 0\n buffer_load_dwordx4 %[av2], %[ars], %[asoff] offen lds\n .endif\n" \
+    "  .if " #J " == 11\n s_mov_b32 m0, %[m0last]\n s_nop 0\n buffer_load_dwordx4 %[av3], %[ars], %[asoff] offen lds\n .endif\n" \
+    " .else\n" \
+    "  .if " #J " == 0\n RW_XLOAD 0, %[xvoff], %[xrs], %[xs0]\n RW_XLOAD 1, %[xvoff], %[xrs], %[xs0]\n .endif\n" \
+    "  .if " #J " == 1\n RW_XLOAD 2, %[xvoff], %[xrs], %[xs1]\n RW_XLOAD 3, %[xvoff], %[xrs], %[xs1]\n .endif\n" \
+    "  .if " #J " == 2\n RW_XLOAD 4, %[xvoff], %[xrs], %[xs2]\n RW_XLOAD 5, %[xvoff], %[xrs], %[xs2]\n .endif\n" \
+    "  .if " #J " == 3\n RW_XLOAD 6, %[xvoff], %[xrs], %[xs3]\n RW_XLOAD 7, %[xvoff], %[xrs], %[xs3]\n .endif\n" \
+    "  .if " #J " == 4\n s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n .endif\n" \
+    "  .if " #J " == 5\n s_mov_b32 m0, %[m0last]\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n .endif\n" \
+    " .endif\n" \
+    " RW_FMADJ " #J "\n" \
+    ".endif\n"
+#define RW_CHUNK \
+    RW_DEFS ".set RW_LCK, %[lck]\n.set RW_WPAR, %[wpar]\n RW_SETS %[p], %[q]\n" \
     "s_nop 4\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+0:RW_OWN" #Q "+3], %0, %1, %2 offen\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+4:RW_OWN" #Q "+7], %0, %1, %2 offen offset:16\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+8:RW_OWN" #Q "+11], %0, %1, %3 offen\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+12:RW_OWN" #Q "+15], %0, %1, %3 offen offset:16\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+16:RW_OWN" #Q "+19], %0, %1, %4 offen\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+20:RW_OWN" #Q "+23], %0, %1, %4 offen offset:16\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+24:RW_OWN" #Q "+27], %0, %1, %5 offen\n" \
-    "buffer_load_dwordx4 v[RW_OWN" #Q "+28:RW_OWN" #Q "+31], %0, %1, %5 offen offset:16\n" \
-    RW_PURGE
-    if constexpr (P == 0) asm volatile(RW_OWN_LOADS(0) :: "v"(voff), "s"(rsrc), "s"(s0), "s"(s1), "s"(s2), "s"(s3) : "memory", RW_CLOB_ALL);
-    else asm volatile(RW_OWN_LOADS(1) :: "v"(voff), "s"(rsrc), "s"(s0), "s"(s1), "s"(s2), "s"(s3) : "memory", RW_CLOB_ALL);
-#undef RW_OWN_LOADS
+    "RW_AREADJ 0, %[aread]\n RW_AREADJ 1, %[aread]\n RW_HALOS (RW_LCK-1)\n" \
+    RW_DIAG(0) RW_DIAG(1) RW_DIAG(2) RW_DIAG(3) RW_DIAG(4) RW_DIAG(5) RW_DIAG(6) \
+    RW_DIAG(7) RW_DIAG(8) RW_DIAG(9) RW_DIAG(10) RW_DIAG(11) RW_DIAG(12) \
+    "s_setprio 0\n" RW_PURGE
+
+// loads a wave issues per chunk (the same for every wave, so that the waits count exactly)
+constexpr int rw_pieces_per_wave(int lck) { return (2 * lck + RW_WAVES - 1) / RW_WAVES; }
+constexpr int rw_loads_per_chunk(int lck) { return 2 * RW_C + rw_pieces_per_wave(lck); }
+
+// The arithmetic of the chunk whose operands sit in own set P and in the value buffer at a_read_addr, and the
+// requests for the chunk two steps ahead (own set (P + 2) % 3) spread between its diagonals.
+template <int LCK, int P, int WPAR>
+__device__ __forceinline__ void rw_compute(unsigned a_read_addr, unsigned x_voff, const unsigned (&a_voff)[4], const RwRequest &rq)
+{
+    static_assert(LCK == 7 || LCK == 13, "instantiated chunk lengths");
+    asm volatile(RW_CHUNK
+                 :: [aread] "v"(a_read_addr), [xvoff] "v"(x_voff), [xrs] "s"(rq.xr), [xs0] "s"(rq.xs[0]), [xs1] "s"(rq.xs[1]),
+                    [xs2] "s"(rq.xs[2]), [xs3] "s"(rq.xs[3]), [ars] "s"(rq.ar), [asoff] "s"(rq.as), [av0] "v"(a_voff[0]),
+                    [av1] "v"(a_voff[1]), [av2] "v"(a_voff[2]), [av3] "v"(a_voff[3]), [m0base] "s"(rq.m0_base),
+                    [m0last] "s"(rq.m0_last), [p] "n"(P), [q] "n"((P + 2) % 3), [wpar] "n"(WPAR), [lck] "n"(LCK)
+                 : "memory", "scc", RW_CLOB_ALL);
 }
-// the same for a chunk that crosses an end of the operand: element by element, every offset checked by its lane
-// (v[k]: byte offset of the lane's row k inside a column, or the out-of-range marker)
-template <int P, int COL>
+
+// The same requests all at once (the first two chunks of a tile, before any arithmetic).
+template <int LCK, int Q>
+__device__ __forceinline__ void rw_request_now(unsigned x_voff, const unsigned (&a_voff)[4], const RwRequest &rq)
+{
+    asm volatile(RW_DEFS "RW_SETS %[q], %[q]\n s_nop 4\n"
+                 "RW_XLOAD 0, %[xvoff], %[xrs], %[xs0]\n RW_XLOAD 1, %[xvoff], %[xrs], %[xs0]\n"
+                 "RW_XLOAD 2, %[xvoff], %[xrs], %[xs1]\n RW_XLOAD 3, %[xvoff], %[xrs], %[xs1]\n"
+                 "RW_XLOAD 4, %[xvoff], %[xrs], %[xs2]\n RW_XLOAD 5, %[xvoff], %[xrs], %[xs2]\n"
+                 "RW_XLOAD 6, %[xvoff], %[xrs], %[xs3]\n RW_XLOAD 7, %[xvoff], %[xrs], %[xs3]\n"
+                 ".if %[lck] > 8\n"
+                 " s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n"
+                 " s_add_u32 m0, %[m0base], 8192\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n"
+                 " s_add_u32 m0, %[m0base], 16384\n s_nop 0\n buffer_load_dwordx4 %[av2], %[ars], %[asoff] offen lds\n"
+                 " s_mov_b32 m0, %[m0last]\n s_nop 0\n buffer_load_dwordx4 %[av3], %[ars], %[asoff] offen lds\n"
+                 ".else\n"
+                 " s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n"
+                 " s_mov_b32 m0, %[m0last]\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n"
+                 ".endif\n" RW_PURGE
+                 :: [xvoff] "v"(x_voff), [xrs] "s"(rq.xr), [xs0] "s"(rq.xs[0]), [xs1] "s"(rq.xs[1]),
+                    [xs2] "s"(rq.xs[2]), [xs3] "s"(rq.xs[3]), [ars] "s"(rq.ar), [asoff] "s"(rq.as), [av0] "v"(a_voff[0]),
+                    [av1] "v"(a_voff[1]), [av2] "v"(a_voff[2]), [av3] "v"(a_voff[3]), [m0base] "s"(rq.m0_base),
+                    [m0last] "s"(rq.m0_last), [q] "n"(Q), [lck] "n"(LCK)
+                 : "memory", "scc", RW_CLOB_ALL);
+}
+
+// the dense rows of one column of a chunk that crosses an end of the operand: element by element, every offset
+// checked by its lane (v[k]: byte offset of the lane's row k inside the column, or the out-of-range marker)
+template <int Q, int COL>
 __device__ __forceinline__ void rw_load_own_checked(const unsigned (&v)[8], rw_int4 rsrc)
 {
-#define RW_OWN_LOADS1(Q, CC) \
-    RW_DEFS \
-    "s_nop 4\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+0], %0, %8, 0 offen\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+1], %1, %8, 0 offen\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+2], %2, %8, 0 offen\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+3], %3, %8, 0 offen\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+4], %4, %8, 0 offen\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+5], %5, %8, 0 offen\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+6], %6, %8, 0 offen\n" \
-    "buffer_load_dword v[RW_OWN" #Q "+8*" #CC "+7], %7, %8, 0 offen\n" \
-    RW_PURGE
-#define RW_OWN_ARGS "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]), "s"(rsrc)
-    if constexpr (P == 0) {
-        if constexpr (COL == 0) asm volatile(RW_OWN_LOADS1(0, 0) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-        if constexpr (COL == 1) asm volatile(RW_OWN_LOADS1(0, 1) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-        if constexpr (COL == 2) asm volatile(RW_OWN_LOADS1(0, 2) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-        if constexpr (COL == 3) asm volatile(RW_OWN_LOADS1(0, 3) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-    } else {
-        if constexpr (COL == 0) asm volatile(RW_OWN_LOADS1(1, 0) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-        if constexpr (COL == 1) asm volatile(RW_OWN_LOADS1(1, 1) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-        if constexpr (COL == 2) asm volatile(RW_OWN_LOADS1(1, 2) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-        if constexpr (COL == 3) asm volatile(RW_OWN_LOADS1(1, 3) :: RW_OWN_ARGS : "memory", RW_CLOB_ALL);
-    }
-#undef RW_OWN_ARGS
-#undef RW_OWN_LOADS1
+    asm volatile(RW_DEFS "RW_SETS %[q], %[q]\n s_nop 4\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+0], %[v0], %[rs], 0 offen\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+1], %[v1], %[rs], 0 offen\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+2], %[v2], %[rs], 0 offen\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+3], %[v3], %[rs], 0 offen\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+4], %[v4], %[rs], 0 offen\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+5], %[v5], %[rs], 0 offen\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+6], %[v6], %[rs], 0 offen\n"
+                 "buffer_load_dword v[RW_OWNQ+8*%[c]+7], %[v7], %[rs], 0 offen\n" RW_PURGE
+                 :: [v0] "v"(v[0]), [v1] "v"(v[1]), [v2] "v"(v[2]), [v3] "v"(v[3]), [v4] "v"(v[4]), [v5] "v"(v[5]),
+                    [v6] "v"(v[6]), [v7] "v"(v[7]), [rs] "s"(rsrc), [q] "n"(Q), [c] "n"(COL)
+                 : "memory", RW_CLOB_ALL);
 }
 
 template <int LCK>
@@ -262,8 +309,11 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
     int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes)
 {
     constexpr int TR = rw_tile_rows(LCK), ABUF = rw_abuf_bytes(LCK), PIECES = 2 * LCK;
-    constexpr int PIECE_IT = (PIECES + RW_WAVES - 1) / RW_WAVES;          // pieces of diagonal values a wave fetches per chunk
-    __shared__ __attribute__((aligned(16))) unsigned char lds[rw_lds_bytes(LCK)];
+    constexpr int NP = rw_pieces_per_wave(LCK);                           // pieces of diagonal values a wave fetches per chunk
+    constexpr int NLOADS = rw_loads_per_chunk(LCK);
+    constexpr unsigned DUMP = 3u * ABUF;                                  // a spare kilobyte behind the three value buffers
+    static_assert(NP == (LCK > 8 ? 4 : 2), "the statements above issue this many pieces");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tile = rw_xcd_tile(blockIdx.x, gridDim.x);
@@ -273,22 +323,25 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
 
     // The chunks that have rows inside the operand: the table is sorted by shift, so they are a contiguous
     // range.  A chunk's valid rows read the dense rows [a0, a0 + TR + LCK - 1), a0 = row0 + its shift.
+    // Lane l also keeps what the walk needs of table entry l -- shift and first table position -- so that the
+    // loop reads an entry with v_readlane, not from memory.
+    const Chunk *mine = chunks + min(lane, nchunks - 1);
+    const int tab_s0 = mine->s0, tab_slot0 = mine->slot[0];
     int c_lo = nchunks, c_hi = 0;
-    for (int k = 0; k < RW_MAX_CHUNKS; k += 64) {
-        if (k >= nchunks) break;
-        const int idx = k + lane;
-        const int a0 = row0 + chunks[min(idx, nchunks - 1)].s0;
+    {
+        const int a0 = row0 + tab_s0;
         const bool outside = (a0 + TR + LCK - 1 <= 0) | (a0 >= n_in);
-        const unsigned long long m = __builtin_amdgcn_ballot_w64(!outside & (idx < nchunks));
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(!outside & (lane < nchunks));
         if (m) {
-            c_lo = min(c_lo, k + (int)__builtin_ctzll(m));
-            c_hi = max(c_hi, k + 64 - (int)__builtin_clzll(m));
+            c_lo = (int)__builtin_ctzll(m);
+            c_hi = 64 - (int)__builtin_clzll(m);
         }
     }
     const int nk = __builtin_amdgcn_readfirstlane(max(c_hi - c_lo, 0));
+    c_lo = __builtin_amdgcn_readfirstlane(c_lo);
 
-    const rw_int4 xr_all = rw_rsrc(X + (long long)col0 * ldx, (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4));
     const float *xcol0 = X + (long long)col0 * ldx;
+    const rw_int4 xr_all = rw_rsrc(xcol0, (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4));
     const rw_int4 ar = rw_rsrc(vals, a_bytes);
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned char *)&lds[0];
     const unsigned a_read_addr = lds0 + 16u * (unsigned)lane;
@@ -302,94 +355,143 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
     // transposed product of a table listed in ascending order), and for the transposed product a value is
     // indexed by its INPUT row, one further per diagonal.  A lane reaches diagonal j of a chunk through a
     // non-negative byte offset from the chunk's first diagonal in memory: diagonal 0 when slot_step > 0, the
-    // last one otherwise.
+    // last one otherwise.  Piece 2 j + half (the rows 8 l + 4 half .. of diagonal j) is fetched by wave
+    // (2 j + half) % 8; a wave without a last piece asks for nothing (out-of-range marker) into the spare kilobyte.
     const bool ascending = slot_step > 0;
     const unsigned dj = ascending ? ((unsigned)slot_step * (unsigned)stride + (unsigned)ashift) * 4u
                                   : ((unsigned)(-slot_step) * (unsigned)stride - (unsigned)ashift) * 4u;
-    unsigned a_voff[PIECE_IT];
+    unsigned a_voff[4];
 #pragma unroll
-    for (int it = 0; it < PIECE_IT; ++it) {
+    for (int it = 0; it < 4; ++it) {
         const int pw = wave + RW_WAVES * it;                              // piece 2 j + half
         const int j = pw >> 1;
-        a_voff[it] = (unsigned)(ascending ? j : LCK - 1 - j) * dj + (unsigned)(8 * lane + 4 * (pw & 1)) * 4u;
+        a_voff[it] = (it < NP && pw < PIECES) ? (unsigned)(ascending ? j : LCK - 1 - j) * dj + (unsigned)(8 * lane + 4 * (pw & 1)) * 4u
+                                              : RW_OOB;
     }
+    const bool has_last = wave + RW_WAVES * (NP - 1) < PIECES;
 
-    typedef const int __attribute__((address_space(4))) *sc_int_ptr;
-    // requests chunk number i of the walk into value buffer / own set `par`
-    auto issue = [&](int i, auto par_c) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(par_c)::value;
-        const sc_int_ptr e = (sc_int_ptr)(chunks + c_lo + i);
-        const int s0 = e[0], slot0 = e[2];
-        const int a0 = row0 + s0;
-        const unsigned abuf = lds0 + (unsigned)(PAR * ABUF);
-        const bool fast = (a0 >= 0) & (a0 + RW_LOADED + LCK - 1 <= n_in) & (row0 + RW_LOADED <= n_out);
-        if (fast) {
-            const int slot_first = ascending ? slot0 : slot0 + (LCK - 1) * slot_step;      // the first in memory
-            const int in_first = ashift ? s0 + (ascending ? 0 : LCK - 1) : 0;
-            const unsigned soff = ((unsigned)slot_first * (unsigned)stride + (unsigned)(row0 + in_first)) * 4u;
+    struct Entry { int s0, slot0; };
+    auto entry = [&](int i) __attribute__((always_inline)) {
+        const int at = c_lo + min(i, max(nk - 1, 0));
+        return Entry{__builtin_amdgcn_readlane(tab_s0, at), __builtin_amdgcn_readlane(tab_slot0, at)};
+    };
+    // can chunk e be requested with whole 16-byte pieces: its 512 rows of every column and of every diagonal exist
+    auto whole = [&](const Entry &e) __attribute__((always_inline)) {
+        const int a0 = row0 + e.s0;
+        return (a0 >= 0) & (a0 + RW_LOADED + LCK - 1 <= n_in) & (row0 + RW_LOADED <= n_out);
+    };
+    // the requests of chunk e into own set / value buffer q; real == false: the empty resources
+    auto request = [&](const Entry &e, int q, bool real) __attribute__((always_inline)) {
+        RwRequest rq;
+        // (the empty resource: the same with a size of 0, every lane out of range)
+        rq.xr = rw_int4{xr_all.x, xr_all.y, real ? xr_all.z : 0, xr_all.w};
+        rq.ar = rw_int4{ar.x, ar.y, real ? ar.z : 0, ar.w};
+        const unsigned a0b = (unsigned)(row0 + e.s0) * 4u;
 #pragma unroll
-            for (int it = 0; it < PIECE_IT; ++it) {
-                const int pw = wave + RW_WAVES * it;
-                if (pw < PIECES) rw_lds_load_b128(ar, abuf + 1024u * (unsigned)pw, a_voff[it], soff);
-            }
-            const unsigned a0b = (unsigned)a0 * 4u;
-            rw_load_own<PAR>(x_voff, xr_all, colb[0] + a0b, colb[1] + a0b, colb[2] + a0b, colb[3] + a0b);
-        } else {
-            // element by element: a value whose input row does not exist is padding and becomes 0, as does a
-            // dense row outside the operand
+        for (int c = 0; c < RW_C; ++c) rq.xs[c] = real ? colb[c] + a0b : 0u;
+        const int slot_first = ascending ? e.slot0 : e.slot0 + (LCK - 1) * slot_step;      // the first in memory
+        const int in_first = ashift ? e.s0 + (ascending ? 0 : LCK - 1) : 0;
+        rq.as = real ? ((unsigned)slot_first * (unsigned)stride + (unsigned)(row0 + in_first)) * 4u : 0u;
+        rq.m0_base = lds0 + (unsigned)(q * ABUF) + 1024u * (unsigned)wave;
+        rq.m0_last = has_last ? rq.m0_base + 8192u * (unsigned)(NP - 1) : lds0 + DUMP;
+        return rq;
+    };
+    // a chunk that crosses an end of the operand, element by element: a value whose input row does not exist
+    // is padding and becomes 0, as does a dense row outside the operand
+    auto request_checked = [&](const Entry &e, auto q_c) __attribute__((always_inline)) {
+        constexpr int Q = decltype(q_c)::value;
+        const unsigned abuf = lds0 + (unsigned)(Q * ABUF);
+        const int a0 = row0 + e.s0;
 #pragma unroll
-            for (int it = 0; it < PIECE_IT; ++it) {
-                const int pw = wave + RW_WAVES * it;
-                if (pw < PIECES) {
-                    const int j = pw >> 1, half = pw & 1;
-                    const unsigned dbase = ((unsigned)(slot0 + j * slot_step) * (unsigned)stride) * 4u;
+        for (int it = 0; it < NP; ++it) {
+            const int pw = wave + RW_WAVES * it;
+            if (pw < PIECES) {
+                const int j = pw >> 1, half = pw & 1;
+                const unsigned dbase = ((unsigned)(e.slot0 + j * slot_step) * (unsigned)stride) * 4u;
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int o = row0 + 8 * (16 * q + (lane >> 2)) + 4 * half + (lane & 3);
-                        const int in = o + s0 + j;
-                        const bool ok = ((unsigned)in < (unsigned)n_in) & (o < n_out);
-                        rw_lds_load_b32(ar, abuf + 1024u * (unsigned)pw + 256u * (unsigned)q,
-                                        ok ? dbase + (unsigned)(ashift ? in : o) * 4u : RW_OOB);
-                    }
+                for (int q = 0; q < 4; ++q) {
+                    const int o = row0 + 8 * (16 * q + (lane >> 2)) + 4 * half + (lane & 3);
+                    const int in = o + e.s0 + j;
+                    const bool ok = ((unsigned)in < (unsigned)n_in) & (o < n_out);
+                    rw_lds_load_b32(ar, abuf + 1024u * (unsigned)pw + 256u * (unsigned)q,
+                                    ok ? dbase + (unsigned)(ashift ? in : o) * 4u : RW_OOB);
                 }
             }
-            unsigned v[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int r = a0 + 8 * lane + k;
-                v[k] = (unsigned)r < (unsigned)n_in ? (unsigned)r * 4u : RW_OOB;
-            }
-            // (the range check of a buffer load counts the scalar offset in: every column gets a resource of its
-            // own that ends with the column's last row)
-            rw_load_own_checked<PAR, 0>(v, rw_rsrc(xcol0 + colb[0] / 4u, (unsigned)n_in * 4u));
-            rw_load_own_checked<PAR, 1>(v, rw_rsrc(xcol0 + colb[1] / 4u, (unsigned)n_in * 4u));
-            rw_load_own_checked<PAR, 2>(v, rw_rsrc(xcol0 + colb[2] / 4u, (unsigned)n_in * 4u));
-            rw_load_own_checked<PAR, 3>(v, rw_rsrc(xcol0 + colb[3] / 4u, (unsigned)n_in * 4u));
         }
-    };
-    auto top = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory", RW_CLOB_ALL); };
-    auto compute = [&](auto par_c) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(par_c)::value;
-        if (wave < 4) rw_compute<LCK, PAR, 0>(a_read_addr);
-        else rw_compute<LCK, PAR, 1>(a_read_addr);
+        unsigned v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int r = a0 + 8 * lane + k;
+            v[k] = (unsigned)r < (unsigned)n_in ? (unsigned)r * 4u : RW_OOB;
+        }
+        // (the range check of a buffer load counts the scalar offset in: every column gets a resource of its
+        // own that ends with the column's last row)
+        rw_load_own_checked<Q, 0>(v, rw_rsrc(xcol0 + colb[0] / 4u, (unsigned)n_in * 4u));
+        rw_load_own_checked<Q, 1>(v, rw_rsrc(xcol0 + colb[1] / 4u, (unsigned)n_in * 4u));
+        rw_load_own_checked<Q, 2>(v, rw_rsrc(xcol0 + colb[2] / 4u, (unsigned)n_in * 4u));
+        rw_load_own_checked<Q, 3>(v, rw_rsrc(xcol0 + colb[3] / 4u, (unsigned)n_in * 4u));
     };
 
     asm volatile(RW_DEFS ".irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31\n"
                          " v_mov_b32 v[RW_ACC+\\i], 0\n.endr\n" RW_PURGE ::: RW_CLOB_ALL);
-    if (nk > 0) issue(0, std::integral_constant<int, 0>{});
-    for (int i = 0; i < nk; i += 2) {
-        top();
-        if (i + 1 < nk) issue(i + 1, std::integral_constant<int, 1>{});
-        compute(std::integral_constant<int, 0>{});
-        if (i + 1 >= nk) break;
-        top();
-        if (i + 2 < nk) issue(i + 2, std::integral_constant<int, 0>{});
-        compute(std::integral_constant<int, 1>{});
+
+    // Chunk i of the walk lives in own set and value buffer i % 3.  Its operands are requested while chunk
+    // i - 2 is computed (the first two before anything else), so they have the whole of chunk i - 1 to arrive;
+    // a chunk that crosses an end of the operand is requested element by element after chunk i - 2 instead (the
+    // statement's own requests then go through the empty resources, so that every wave issues the same number
+    // of loads per chunk whatever happens and the waits count exactly).
+    bool exact = false;         // the loads in flight behind those of the chunk about to be computed are the NLOADS of one statement
+    if (nk > 0) {
+        const Entry e0 = entry(0);
+        if (whole(e0)) rw_request_now<LCK, 0>(x_voff, a_voff, request(e0, 0, true));
+        else request_checked(e0, std::integral_constant<int, 0>{});
+        if (nk > 1) {
+            const Entry e1 = entry(1);
+            if (whole(e1)) {
+                rw_request_now<LCK, 1>(x_voff, a_voff, request(e1, 1, true));
+                exact = true;
+            } else {
+                request_checked(e1, std::integral_constant<int, 1>{});
+            }
+        }
+    }
+    // what the statement of a step requests (chunk i + 2), prepared one step ahead -- behind the arithmetic of
+    // the step before, where the waves wait for each other anyway
+    struct Next { RwRequest rq; Entry e; bool checked; };
+    auto prepare = [&](int ii, int q) __attribute__((always_inline)) {
+        const Entry e = entry(ii);
+        const bool there = ii < nk, w = whole(e);
+        return Next{request(e, q, there && w), e, there && !w};
+    };
+    Next nx = prepare(2, 2);
+    auto step = [&](int i, auto p_c) __attribute__((always_inline)) {
+        constexpr int P = decltype(p_c)::value, Q = (P + 2) % 3;
+        // chunk i must be in: everything but the loads issued behind it
+        if (exact) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(NLOADS) : "memory", RW_CLOB_ALL);
+        else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory", RW_CLOB_ALL);
+        const unsigned aread = a_read_addr + (unsigned)(P * ABUF);
+        if (wave < 4) rw_compute<LCK, P, 0>(aread, x_voff, a_voff, nx.rq);
+        else rw_compute<LCK, P, 1>(aread, x_voff, a_voff, nx.rq);
+        exact = true;
+        if (nx.checked) {
+            request_checked(nx.e, std::integral_constant<int, Q>{});
+            exact = false;
+        }
+        nx = prepare(i + 3, P);
+    };
+    for (int i = 0; i < nk;) {
+        step(i, std::integral_constant<int, 0>{});
+        if (++i >= nk) break;
+        step(i, std::integral_constant<int, 1>{});
+        if (++i >= nk) break;
+        step(i, std::integral_constant<int, 2>{});
+        ++i;
     }
 
     // The sums leave through LDS so that a column's rows go to memory in 16-byte pieces, lane after lane: every
     // wave writes its 4 x 512 sums to its own 8 KB (column c at 2 KB c, the lane's 8 rows at 32 bytes x lane)
     // and reads back rows 4 l .. 4 l + 3 and 256 + 4 l .. of each column.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the last statements' requests (empty, but they write LDS)
     __syncthreads();                                // every wave is through with the value buffers
     const unsigned out_addr = lds0 + 8192u * (unsigned)wave + 32u * (unsigned)lane;
     asm volatile(RW_DEFS
@@ -449,7 +551,7 @@ bool spmm_rows_ok(const DiaView &A, long long ldb, long long ldd, bool trans)
     const int step = trans ? A.slot_step_t : A.slot_step_n;
     const long long x_bytes = ((RW_COLS - 1) * ldb + n_in) * 4;
     const long long a_bytes = (long long)A.nd * A.stride * 4;
-    if (A.rf != 1 || (lck != 7 && lck != 13) || lck_min != lck || step == 0 || nchunks > RW_MAX_CHUNKS) return false;
+    if (A.rf != 1 || (lck != 7 && lck != 13) || lck_min != lck || step == 0 || nchunks > RW_MAX_CHUNKS) return false;   // (a lane per table entry)
     // values are indexed by a row of the matrix (the output row, or the input row of the transposed product):
     // with every diagonal as long as the matrix has rows, a tile's 512 rows of a diagonal stay inside the array
     if (A.stride < A.h) return false;
@@ -474,9 +576,17 @@ hipError_t launch_spmm_rows(const DiaView &A, const float *vals, const float *B,
 #define RW_ARGS trans ? A.chunks_t_dev : A.chunks_n_dev, trans ? A.n_chunks_t : A.n_chunks_n, vals, A.stride, trans ? 1 : 0, \
                 trans ? A.slot_step_t : A.slot_step_n, B, ldb, dst, ldd, n_out, n_in, batch, alpha, beta, (int)col_tiles, \
                 (unsigned)((long long)A.nd * A.stride * 4)
-    if (lck == 7) hipLaunchKernelGGL((spmm_rows_kernel<7>), grid, dim3(64 * RW_WAVES), 0, stream, RW_ARGS);
-    else if (lck == 13) hipLaunchKernelGGL((spmm_rows_kernel<13>), grid, dim3(64 * RW_WAVES), 0, stream, RW_ARGS);
-    else return hipErrorNotSupported;
+    if (lck == 7) {
+        hipLaunchKernelGGL((spmm_rows_kernel<7>), grid, dim3(64 * RW_WAVES), rw_lds_bytes(7), stream, RW_ARGS);
+    } else if (lck == 13) {
+        // more LDS than a kernel may use without saying so
+        static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_rows_kernel<13>),
+                                                              hipFuncAttributeMaxDynamicSharedMemorySize, rw_lds_bytes(13));
+        if (allowed != hipSuccess) return allowed;
+        hipLaunchKernelGGL((spmm_rows_kernel<13>), grid, dim3(64 * RW_WAVES), rw_lds_bytes(13), stream, RW_ARGS);
+    } else {
+        return hipErrorNotSupported;
+    }
 #undef RW_ARGS
     return hipGetLastError();
 }
