@@ -18,7 +18,15 @@ count every operand once and only the valid diagonal slots
 (cuv_amd.workloads.spmm_bytes / dd2dia_bytes).  `roofline` describes the
 slowest of the three kernels, timed on its own with HIP events on the launch
 stream.  `cpu_baseline` is the single-threaded CPU oracle (a restatement of the
-reference's host loops) on the same step, on this machine's host cores.
+reference's host loops) on the same step, on this machine's host cores;
+`cpu_baseline_all_cores` runs the same oracle on every core this process may
+use (threads over batch columns for the products, over diagonals for the
+gradient) -- the reference itself has no threaded host path.
+
+Every timed leg is preceded by `settle_ms` of untimed replays of the very
+launches it times (clocks and caches in their steady state), so that a run of
+a few steps reads what a long one reads.  `clocks` holds the shader and memory
+clocks read (rocm-smi) while the step's graph is running.
 
 Prints one JSON line on stdout.
 """
@@ -79,7 +87,9 @@ def parse():
     ap.add_argument("--legs", default="all", choices=["all", "rotating"],
                     help="'rotating': only the legs that stream from HBM (no cache-warm legs, no large-layer record), "
                          "so that a profiler's per-kernel averages describe the same launches as the headline figures")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--settle-ms", type=float, default=200.0,
+                    help="untimed replays of a leg's own launches before it is timed, in ms of GPU time")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
     return ap.parse_args()
 
@@ -135,10 +145,12 @@ def measure_cfg4(steps, torch, D, W, dev, with_aux=True):
         ops["forward"][0]()
     torch.cuda.synchronize()
     res = {}
+    from cuv_amd import _lib
     for name, (fn, nbytes) in ops.items():
         ms = timed(fn)
         tf = flops / (ms * 1e-3) / 1e12
-        res[name] = dict(ms=ms, bytes=nbytes, flops=flops, gbs=nbytes / (ms * 1e-3) / 1e9,
+        res[name] = dict(ms=ms, kernel=_lib.lib().cuvdia_last_kernel().decode(), bytes=nbytes, flops=flops,
+                         gbs=nbytes / (ms * 1e-3) / 1e9,
                          frac_hbm=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, tflops=tf,
                          frac_fp32_valu=tf / FP32_VALU_PEAK_TFLOPS, frac_fp32_valu_broadcast=tf / FP32_VALU_BROADCAST_TFLOPS)
     aux = {}
@@ -173,9 +185,24 @@ def bench_scale(args, torch, D, W, dev):
     costs (launch, first loads, final stores) no longer weigh.  Inputs are drawn on the device; from the second case
     on the operands of a call exceed the 256 MB Infinity Cache, so every launch streams from HBM."""
     cases = [(128, 128), (128, 512), (128, 2048), (128, 4096), (256, 1024), (512, 128), (512, 512), (1024, 128)]
+    out = measure_scale(cases, torch, D, W, dev)
+    best = max(r[k]["gbs"] for r in out for k in ("up_pass", "down_pass", "weight_gradient"))
+    print(json.dumps(dict(
+        metric="achieved HBM GB/s, DIA SpMM (both transposes) + densedense_to_dia, size sweep", unit="GB/s",
+        value=best, n_gpus=1, steps=None, warmup=3, higher_is_better=True, scaling="weak", vs_baseline=None,
+        dtype="f32", data="synthetic",
+        config=dict(workload="7x7 window on a px x px map (49 diagonals), batch b, for several (px, b); "
+                             "each product timed alone; value = the best single figure of the sweep"),
+        cases=out)))
+
+
+def measure_scale(cases, torch, D, W, dev):
+    """One row per (map width, batch): each product timed alone from a HIP graph of ten launches, with the name of
+    the kernel that served it."""
+    from cuv_amd import _lib
+    L = _lib.lib()
     g = torch.Generator(device=dev)
     g.manual_seed(0xC0FFEE + 5)
-    stream = torch.cuda.current_stream()
     out = []
     for px, batch in cases:
         n = px * px
@@ -205,6 +232,7 @@ def bench_scale(args, torch, D, W, dev):
             # ten launches per graph replay: Python cannot issue launches every few microseconds
             for _ in range(3):
                 fn()
+            kernel = L.cuvdia_last_kernel().decode()
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
@@ -232,19 +260,12 @@ def bench_scale(args, torch, D, W, dev):
             torch.cuda.synchronize()
             us = e0.elapsed_time(e1) / (10 * reps) * 1e3
             row[name] = dict(us=us, bytes=nbytes, gbs=nbytes / us / 1e3, frac_hbm=nbytes / us / 1e3 / HBM_PEAK_GBS,
-                             tflops=flops / us / 1e6)
+                             tflops=flops / us / 1e6, kernel=kernel)
             del graph
         out.append(row)
         del A, G, X, H, Y, bd
         torch.cuda.empty_cache()
-    best = max(r[k]["gbs"] for r in out for k in ("up_pass", "down_pass", "weight_gradient"))
-    print(json.dumps(dict(
-        metric="achieved HBM GB/s, DIA SpMM (both transposes) + densedense_to_dia, size sweep", unit="GB/s",
-        value=best, n_gpus=1, steps=None, warmup=3, higher_is_better=True, scaling="weak", vs_baseline=None,
-        dtype="f32", data="synthetic",
-        config=dict(workload="7x7 window on a px x px map (49 diagonals), batch b, for several (px, b); "
-                             "each product timed alone; value = the best single figure of the sweep"),
-        cases=out)))
+    return out
 
 
 def bench_layer(args, torch, D, W, dev):
@@ -313,6 +334,94 @@ def bench_layer(args, torch, D, W, dev):
         us=us, learn_step=dict(bytes=step_bytes, gbs=step_bytes / (lw * 1e-6) / 1e9,
                                frac_hbm=step_bytes / (lw * 1e-6) / 1e9 / HBM_PEAK_GBS,
                                note="warm: the 6.4 MB working set stays in cache between launches"))))
+
+
+def read_clocks(torch, enqueue, eager):
+    """Shader and memory clock while the step runs: about a second of the step's launches is enqueued, rocm-smi is
+    asked (a child process) while the GPU works through them, then the queue is drained.  None where rocm-smi is
+    not there or does not answer."""
+    import re
+    import shutil
+    import subprocess
+    exe = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    if not os.path.exists(exe):
+        return None
+    try:
+        if eager:
+            enqueue()
+            graph = None
+        else:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                enqueue()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            for _ in range(max(1, min(20000, int(1500.0 / max(1e-3, e0.elapsed_time(e1)))))):
+                graph.replay()
+        txt = subprocess.run([exe, "--showclocks", "-d", "0"], capture_output=True, text=True, timeout=20).stdout
+        busy = not torch.cuda.current_stream().query()
+        torch.cuda.synchronize()
+        found = {}
+        for line in txt.splitlines():
+            m = re.search(r"\b(sclk|mclk|fclk|socclk) clock level:?\s*\S*\s*\((\d+)\s*Mhz\)", line, re.I)
+            if m:
+                found[m.group(1).lower() + "_mhz"] = int(m.group(2))
+        if not found:
+            return None
+        found["source"] = "rocm-smi --showclocks, read after the timed legs while a graph of the step's launches was replaying"
+        found["gpu_busy_when_read"] = bool(busy)
+        return found
+    except Exception as e:           # the clocks are a note beside the figures, never a reason to fail the run
+        return dict(error=str(e)[:200])
+
+
+def cpu_all_cores(O, np, p, w1, w2, w3, step_bytes, step_flops, one_core_s):
+    """The oracle's step on every core this process may use (at most 16, the share of one GPU's host): the two
+    products split over the batch columns, the gradient over the diagonals (its sum runs over the batch, so
+    a split over columns would need a reduction the reference does not have), one thread per share -- the
+    library calls release the interpreter lock.  The reference's host path is single-threaded
+    (spmv.cu:145-220, densedense_to_sparse.cu:204-252): this leg says what the same loops give when all cores
+    run them, not what the reference does."""
+    from concurrent.futures import ThreadPoolExecutor
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    cores = max(1, min(16, cores))
+    od = O.Dia(p.h, p.w, p.offsets, p.stride, 1, w1.vals)
+    batch = w1.X.shape[1]
+    col_cuts = [batch * k // cores for k in range(cores + 1)]
+    col_shares = [(a, b) for a, b in zip(col_cuts[:-1], col_cuts[1:]) if b > a]
+    dia_cuts = [p.nd * k // cores for k in range(cores + 1)]
+    dia_shares = [(a, b) for a, b in zip(dia_cuts[:-1], dia_cuts[1:]) if b > a]
+    subs = []
+    for a, b in dia_shares:
+        subs.append(O.Dia(p.h, p.w, p.offsets[a:b], p.stride, 1, w3.vals[a * p.stride:b * p.stride].copy()))
+    Xs = [np.asfortranarray(w1.X[:, a:b]) for a, b in col_shares]
+    Hs = [np.asfortranarray(w2.X[:, a:b]) for a, b in col_shares]
+    Ds = [np.asfortranarray(w2.dst[:, a:b]) for a, b in col_shares]
+
+    def run(pool):
+        list(pool.map(lambda x: O.prod(od, x), Xs))
+        list(pool.map(lambda hd: O.prod(od, hd[0], hd[1], "t", 1.0, 0.5), zip(Hs, Ds)))
+        list(pool.map(lambda d: O.dd2dia(d, w3.A, w3.B, w3.alpha, w3.beta), subs))
+    reps = []
+    with ThreadPoolExecutor(max_workers=cores) as pool:
+        run(pool)
+        for _ in range(5):
+            t = time.perf_counter()
+            run(pool)
+            reps.append(time.perf_counter() - t)
+    med = statistics.median(reps)
+    return dict(value=step_bytes / med / 1e9, unit="GB/s", cores=cores, kind="port",
+                sample="the full step (cfg1+cfg2+cfg3), median of 5 repetitions; products split over batch columns, "
+                       "gradient over diagonals, one thread per core",
+                ms_per_step=med * 1e3, gflops=step_flops / med / 1e9, speedup_over_one_core=one_core_s / med,
+                note="an extrapolation of the reference's host path, which is single-threaded: what its loops reach "
+                     "when every core runs a share")
 
 
 def main():
@@ -445,6 +554,42 @@ def main():
                 fn(i)
         return g
 
+    settled = []
+
+    def settle(fn, plan, n):
+        """Untimed: the launches about to be timed, replayed for args.settle_ms of GPU time (measured on one
+        replay first), so that the timed region starts with clocks, caches and the graph itself in the state
+        a long run reaches."""
+        if args.settle_ms <= 0:
+            return
+        w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+        def once():
+            if plan is None:
+                for i in range(min(n, nsets)):
+                    fn(i)
+            else:
+                (plan[0] or plan[2]).replay()
+        torch.cuda.synchronize()
+        w0.record(stream)
+        once()
+        w1.record(stream)
+        torch.cuda.synchronize()
+        one_ms = max(1e-3, w0.elapsed_time(w1))
+        last_replay_ms[0] = one_ms
+        reps = max(1, min(100000, int(args.settle_ms / one_ms)))
+        w0.record(stream)
+        for _ in range(reps):
+            once()
+        w1.record(stream)
+        torch.cuda.synchronize()
+        settled.append(w0.elapsed_time(w1))
+
+    last_replay_ms = [1.0]
+
+    def gate_reps(plan):
+        return max(2, min(2000, int(10.0 / max(1e-3, last_replay_ms[0])) + 1))
+
     def timed(fn, n):
         """Exactly n calls fn(0..n-1) (fn must depend on i only through i % nsets)
         between two HIP events on the launch stream; returns ms per call."""
@@ -458,8 +603,17 @@ def main():
                 if g is not None:
                     g.replay()
             plan = (gfull, full, grest)
+        settle(fn, plan, n)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
+        if plan is not None:
+            # About 10 ms of the same replays go first, untimed, and are still running while the host enqueues the
+            # first event, the timed replays and the second event: the GPU then takes the timed region from its
+            # queue in the state a long run is in, and the time the host needs to submit a graph (hundreds of
+            # microseconds right after a burst of replays) is not read as kernel time -- which matters when the
+            # whole region is one replay of 20 steps.
+            for _ in range(gate_reps(plan)):
+                (plan[0] or plan[2]).replay()
         e0.record(stream)
         if plan is None:
             for i in range(n):
@@ -477,6 +631,16 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
+    # which kernel serves each operation: asked of the library, call by call
+    kernel_names, kernel_paths = {}, {}
+    for name, fn in (("up_pass", up), ("down_pass", down), ("weight_gradient", grad)):
+        fn(sets[0])
+        kernel_names[name] = L.cuvdia_last_kernel().decode()
+        kernel_paths[name] = L.cuvdia_last_path()
+    torch.cuda.synchronize()
+    if not kernel_names["up_pass"].startswith("spmm_") or not kernel_names["weight_gradient"].startswith("dd2dia_"):
+        print("unexpected kernels: %r" % kernel_names, file=sys.stderr)
+        sys.exit(1)
     t0 = time.perf_counter()
     ms_step = timed(step, args.steps)
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
@@ -500,9 +664,9 @@ def main():
                          gbs=wl.bytes / (ms * 1e-3) / 1e9, gflops=wl.flops / (ms * 1e-3) / 1e9,
                          frac_hbm=wl.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
     # The dominant kernel's two launches of a step as they follow each other in the step (up-pass, then down-pass,
-    # set after set): its average launch duration for the roofline entry.  Timed alone, each product reads
-    # about 0.4 us longer per launch than here (a run of identical launches all read, then all write, at the
-    # same moments); a profiler's per-kernel average over the run lies between the two.
+    # set after set), reported beside the roofline entry (which is computed from the legs above).  Timed alone,
+    # each product reads about 0.4 us longer per launch than here (a run of identical launches all read, then
+    # all write, at the same moments); a profiler's per-kernel average over the run lies between the two.
     def up_down(i):
         s_ = sets[i % nsets]
         up(s_); down(s_)
@@ -517,8 +681,13 @@ def main():
     # down-pass).  Its roofline entry is per launch, averaged over the two --
     # algorithmic bytes of the two products / their two durations -- which is
     # also what a profiler's per-kernel average duration corresponds to.
-    kernel_names = {"up_pass": "spmm_tiled_kernel<7, 8, 1, false>", "down_pass": "spmm_tiled_kernel<7, 8, 1, false>",
-                    "weight_gradient": "dd2dia_tiled_kernel<7, true, true, 0>"}
+    # (the same launches once more, after every timed leg: the choice of kernel must not have changed)
+    for name, fn in (("up_pass", up), ("down_pass", down), ("weight_gradient", grad)):
+        fn(sets[0])
+        if L.cuvdia_last_kernel().decode() != kernel_names[name] or L.cuvdia_last_path() != kernel_paths[name]:
+            print("kernel choice changed during the run: %s" % name, file=sys.stderr)
+            sys.exit(1)
+    torch.cuda.synchronize()
     traffic, traffic_rev = load_traffic()
     for name in per:
         per[name]["kernel"] = kernel_names[name]
@@ -527,9 +696,12 @@ def main():
         # broadcast-operand FMAs (the products' form; the projection's plain FMAs could run at twice that)
         per[name]["hbm_floor_us"] = per[name]["bytes"] / (HBM_PEAK_GBS * 1e9) * 1e6
         per[name]["valu_floor_us"] = per[name]["flops"] / (FP32_VALU_BROADCAST_TFLOPS * 1e12) * 1e6
-    sp_us = pair_us / 2
+    sp_us = (per["up_pass"]["us"] + per["down_pass"]["us"]) / 2          # the same legs as ops[]
     sp_bytes = (per["up_pass"]["bytes"] + per["down_pass"]["bytes"]) / 2
     sp_flops = (per["up_pass"]["flops"] + per["down_pass"]["flops"]) / 2
+    if kernel_names["up_pass"] != kernel_names["down_pass"]:
+        print("the two products ran different kernels (%r): the roofline entry assumes one" % kernel_names, file=sys.stderr)
+        sys.exit(1)
     if 2 * sp_us >= per["weight_gradient"]["us"]:
         gbs = sp_bytes / (sp_us * 1e-6) / 1e9
         sp_traffic = None
@@ -538,8 +710,9 @@ def main():
         roofline = dict(bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS,
                         traffic=sp_traffic, traffic_rev=traffic_rev,
                         kernel=kernel_names["up_pass"],
-                        op="up_pass+down_pass (mean per launch, the two launched one after the other as in the step)",
-                        launches_per_step=2, us_per_launch=sp_us, algorithmic_bytes=sp_bytes,
+                        op="up_pass+down_pass (mean per launch of ops.up_pass.us and ops.down_pass.us, each timed alone)",
+                        launches_per_step=2, us_per_launch=sp_us, us_per_launch_in_step_order=pair_us / 2,
+                        algorithmic_bytes=sp_bytes,
                         hbm_floor_us=sp_bytes / (HBM_PEAK_GBS * 1e9) * 1e6,
                         valu_floor_us=sp_flops / (FP32_VALU_BROADCAST_TFLOPS * 1e12) * 1e6,
                         note="by intensity (7-10 FLOP/B) the kernel sits on the ridge of the rate its broadcast-operand "
@@ -566,18 +739,29 @@ def main():
         frac_of_hbm_peak=step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         gflops=step_flops / (ms_step * 1e-3) / 1e9,
         wall_ms_per_step_incl_capture=wall_ms, launch="eager" if args.no_graph else "hip_graph",
-        ops=per, warm_us=warm, parity=checked, roofline=roofline)
+        settle_ms=dict(requested_per_leg=args.settle_ms, spent_per_leg=[round(x, 1) for x in settled],
+                       note="untimed replays of each leg's own launches before it is timed"),
+        clocks=None, ops=per, warm_us=warm, parity=checked, roofline=roofline)
 
     if args.legs == "all":
         # the large layer (cfg4) beside the headline figures: an auxiliary record, no part of `value`
-        del sets
+        keep = sets[0]
+        del sets, s
         torch.cuda.empty_cache()
         cfg4_config, cfg4_res, _ = measure_cfg4(20, torch, D, W, dev, with_aux=False)
         out["aux"] = dict(cfg4=dict(config=cfg4_config, ops=cfg4_res,
                                     note="bound by the fp32 vector rate (57 FLOP per algorithmic byte): "
                                          "frac_fp32_valu is against the published 157.3 TFLOP/s, "
                                          "frac_fp32_valu_broadcast against the 78.6 TFLOP/s of FMAs with a "
-                                         "DPP-broadcast or scalar operand, the form these kernels use"))
+                                         "DPP-broadcast or scalar operand, the form these kernels use"),
+                          scale=dict(config="the headline layer's pattern (7x7 window, 49 diagonals) on a px x px map at "
+                                            "batch b: each product timed alone (full sweep: --workload scale)",
+                                     cases=measure_scale([(128, 2048), (512, 128), (512, 512)], torch, D, W, dev)))
+
+    else:
+        keep = sets[0]
+    # last of the GPU work (a query of the management interface is followed by slower launches for a while)
+    out["clocks"] = read_clocks(torch, lambda: [(up(keep), down(keep), grad(keep)) for _ in range(30)], args.no_graph)
 
     if not args.no_cpu:
         from oracle import oracle as O
@@ -593,6 +777,7 @@ def main():
         out["cpu_baseline"] = dict(value=step_bytes / med / 1e9, unit="GB/s", cores=1, kind="port",
                                    sample="the full step (cfg1+cfg2+cfg3), median of 5 repetitions",
                                    ms_per_step=med * 1e3, gflops=step_flops / med / 1e9)
+        out["cpu_baseline_all_cores"] = cpu_all_cores(O, np, p, w1, w2, w3, step_bytes, step_flops, med)
     print(json.dumps(out))
 
 

@@ -48,6 +48,10 @@ def lib():
     L.cuvdia_plan_chunks_max.argtypes = [ip, c_int, c_int, c_int, ip, ip, ip, c_int]
     L.cuvdia_plan_units.argtypes = [ip, c_int, ip, ip, c_int]
     L.cuvdia_plan_walk.argtypes = [ip, c_int, c_int, c_int, ip, ip, ip, ip]
+    L.cuvdia_plan_walk_launch.argtypes = [ip, c_int, c_int, c_int, c_int, c_int, c_int]
+    L.cuvdia_plan_walk_launch.restype = c_ll
+    L.cuvdia_last_kernel.argtypes = []
+    L.cuvdia_last_kernel.restype = ctypes.c_char_p
     L.cuvdia_desc_create.argtypes = [ctypes.POINTER(c_vp), ip, c_int, c_int, c_int, c_int, c_int]
     L.cuvdia_desc_destroy.argtypes = [c_vp]
     L.cuvdia_desc_info.argtypes = [c_vp, ip, ip, ctypes.POINTER(c_ll)]

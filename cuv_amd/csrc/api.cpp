@@ -7,6 +7,8 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdint>
+#include <cstdarg>
+#include <cstdio>
 #include <cstring>
 #include <list>
 #include <mutex>
@@ -33,6 +35,7 @@ namespace {
 
 std::atomic_int g_path{CUVDIA_PATH_AUTO};
 thread_local int t_last_path = 0;
+thread_local char t_last_kernel[96] = "";
 thread_local std::string t_hip_error;
 
 // Batches narrower than this go to the generic kernel: the tiled SpMM puts
@@ -98,6 +101,16 @@ int validate_shape(const int *offsets, int nd, int h, int w, int stride, int rf)
 
 }  // namespace
 
+namespace cuvdia {
+void note_kernel(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_last_kernel, sizeof t_last_kernel, fmt, ap);
+    va_end(ap);
+}
+}  // namespace cuvdia
+
 extern "C" {
 
 int cuvdia_abi_version(void) { return 1; }
@@ -129,6 +142,7 @@ int cuvdia_set_path(int path)
 }
 
 int cuvdia_last_path(void) { return t_last_path; }
+const char *cuvdia_last_kernel(void) { return t_last_kernel; }
 
 int cuvdia_plan_chunks_max(const int *offsets_host, int nd, int transposed, int max_len,
                            int *s0, int *len, int *slot, int cap)
@@ -174,6 +188,31 @@ int cuvdia_plan_walk(const int *offsets_host, int nd, int stride, int transposed
     if (lck) *lck = wp.lck;
     const int rows = spmm_walk_tile_rows(wp.lck, wp.k, wp.s0);
     return rows > 0 && wp.period % rows == 0 ? 2 : 1;
+}
+
+long long cuvdia_plan_walk_launch(const int *offsets_host, int nd, int stride, int h, int w, int transposed,
+                                  int batch)
+{
+    if (!offsets_host || nd < 1 || batch < 0) return CUVDIA_EINVAL;
+    if (const int rc = validate_shape(offsets_host, nd, h, w, stride, 1)) return rc;
+    const bool trans = transposed != 0;
+    WalkPlan wp;
+    DiaView view{};
+    try {
+        const std::vector<Chunk> chunks = plan_chunks(offsets_host, nd, trans, SP_CHUNK_MAX);
+        plan_walk(chunks, stride, trans, wp);
+        view.n_chunks_n = view.n_chunks_t = (int)chunks.size();
+    } catch (const std::bad_alloc &) {
+        return CUVDIA_ENOMEM;
+    }
+    if (!wp.ok) return 0;
+    // the conditions of the automatic choice in cuvdia_spmm_layer_f32, for packed operands
+    view.h = h; view.w = w; view.nd = nd; view.stride = stride; view.rf = 1;
+    const long long n_out = trans ? w : h, n_in = trans ? h : w;
+    if (batch < SPMM_TILED_MIN_BATCH || !spmm_tiled_ok(view, n_in, n_out, trans)) return 0;
+    long long workgroups = 0;
+    (void)spmm_walk_plan(wp.lck, wp.k, wp.s0, wp.period, n_out, n_in, ((long long)batch + 63) / 64, false, &workgroups);
+    return workgroups;
 }
 
 int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap)
@@ -620,19 +659,20 @@ int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals, const int *offsets_host
     view.h = h; view.w = w; view.nd = nd; view.stride = stride; view.rf = row_fact;
     view.offsets_dev = reinterpret_cast<const int *>(tables);
     const Chunk *chunks_dev = reinterpret_cast<const Chunk *>(tables + NOALLOC_CHUNKS_AT);
-    int max_len = 0, s_min = chunks.front().s0, s_max = s_min;
+    int max_len = 0, min_len = chunks.front().len, s_min = chunks.front().s0, s_max = s_min;
     for (const Chunk &c : chunks) {
         max_len = std::max(max_len, c.len);
+        min_len = std::min(min_len, c.len);
         s_min = std::min(s_min, c.s0);
         s_max = std::max(s_max, c.s0);
     }
     if (trans) {
         view.chunks_t_dev = chunks_dev; view.n_chunks_t = (int)chunks.size();
-        view.max_len_t = max_len; view.s_min_t = s_min; view.s_max_t = s_max;
+        view.max_len_t = max_len; view.min_len_t = min_len; view.s_min_t = s_min; view.s_max_t = s_max;
         view.slot_step_t = common_slot_step(chunks);
     } else {
         view.chunks_n_dev = chunks_dev; view.n_chunks_n = (int)chunks.size();
-        view.max_len_n = max_len; view.s_min_n = s_min; view.s_max_n = s_max;
+        view.max_len_n = max_len; view.min_len_n = min_len; view.s_min_n = s_min; view.s_max_n = s_max;
         view.slot_step_n = common_slot_step(chunks);
     }
 

@@ -352,8 +352,10 @@ __global__ __launch_bounds__(AXPBY_THREADS) void momentum_kernel(
 //      no guards and never sees padding;
 //   2. each lane reads its column's window of T + LCK - 1 values with 16-byte
 //      LDS reads (the column pitch / 4 is odd, so the 64 lanes spread over
-//      all banks).  Every chunk is processed as LCK diagonals, LCK = the
-//      longest chunk of the table; shorter chunks carry zeros;
+//      all banks).  The kernel is instantiated for LCK = the longest chunk
+//      of the table; a chunk of LCK diagonals runs one straight-line block
+//      of FMAs, a shorter one only the diagonals it has (a wave-uniform test
+//      per diagonal), so no dense value meets a diagonal that is not stored;
 //   3. for each diagonal j the wave reads A_j[its T rows] into one VGPR (lane
 //      & (T-1) selects the row) and issues T FMAs whose first operand is that
 //      VGPR broadcast within each 16-lane row by DPP (row_newbcast:t):
@@ -578,6 +580,38 @@ __device__ __forceinline__ void spmm_rows_range(float (&acc)[T], const SpWindow<
     }
 }
 
+// The same for a chunk of `len` < LCK diagonals (wave-uniform): the diagonals it does not have are skipped, not
+// multiplied as zeros -- a product 0 * Inf or 0 * NaN with a dense row that the chunk's own diagonals do not
+// reach would put a NaN where the reference's loop over stored elements leaves a finite sum.
+template <int LCK, int T, int J, int J1>
+__device__ __forceinline__ void spmm_rows_range_upto(float (&acc)[T], const SpWindow<LCK, T> &win, int len)
+{
+    if constexpr (J < J1) {
+        if (J < len) {
+            if constexpr (T == 8) {
+                fma_diagonals8<J, 1, 0>(acc, win.a, win.w);
+            } else {
+                fma_block8<J, 0>(acc, win.a[J], win.w);
+                fma_block8<J, 8>(acc, win.a[J], win.w);
+            }
+        }
+        spmm_rows_range_upto<LCK, T, J + 1, J1>(acc, win, len);
+    }
+}
+// diagonals J .. J1 - 1 of a chunk of `len` diagonals: the straight-line block for a full chunk, the guarded
+// one otherwise.  MIXED = false: the kernel for tables all of whose chunks have LCK diagonals (every window table),
+// which carries neither the test nor the second block.
+template <int LCK, int T, int J, int J1, bool MIXED>
+__device__ __forceinline__ void spmm_rows_chunk(float (&acc)[T], const SpWindow<LCK, T> &win, int len)
+{
+    if constexpr (LCK == 1 || !MIXED) {
+        spmm_rows_range<LCK, T, J, J1>(acc, win);
+    } else {
+        if (len == LCK) spmm_rows_range<LCK, T, J, J1>(acc, win);
+        else spmm_rows_range_upto<LCK, T, J, J1>(acc, win, len);
+    }
+}
+
 template <int LCK, int T>
 __device__ __forceinline__ void spmm_read_window(SpWindow<LCK, T> &win, const float *win_lds,
                                                  const float *a_lds)
@@ -619,7 +653,7 @@ constexpr unsigned OOB_OFFSET = 0x80000000u;     // >= every resource size used 
 // and shifted into place on the way.  While the FMAs of chunk c run, chunk
 // c+1 is being written to the other LDS buffer (its window is read right after
 // the barrier), chunk c+2 is in flight and chunk c+3 has just been requested.
-template <int LCK, int T, int NTAB, bool EP>
+template <int LCK, int T, int NTAB, bool EP, bool MIXED>
 __device__ __forceinline__ void spmm_tile_edge(
     float (&lds)[2][SP_STAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
@@ -708,6 +742,17 @@ __device__ __forceinline__ void spmm_tile_edge(
         }
     };
 
+    auto chunk_len = [&](int c) {
+        const int cc = min(c, nchunks - 1);
+        int len = __builtin_amdgcn_readlane(tab_len[0], cc & 63);
+#pragma unroll
+        for (int k = 1; k < NTAB; ++k) {
+            const int l = __builtin_amdgcn_readlane(tab_len[k], cc & 63);
+            len = (cc >> 6) == k ? l : len;
+        }
+        return len;
+    };
+
     // Dense rows come as 16-byte pieces.  A piece that straddles the operand's
     // first or last row is fetched from the nearest in-range position instead
     // (rows rc..rc+3) and shifted into place when it is written to LDS, so the
@@ -777,7 +822,7 @@ __device__ __forceinline__ void spmm_tile_edge(
         commit(next, lds[(c + 1) & 1]);
         fetch_info(c + 4, info_next);
         issue(info, next, c + 3);
-        spmm_rows<LCK, T, 0>(acc, win_cur);
+        spmm_rows_chunk<LCK, T, 0, LCK, MIXED>(acc, win_cur, MIXED ? chunk_len(c) : LCK);
         __syncthreads();
         read_window(win_next, lds[(c + 1) & 1]);
     };
@@ -911,7 +956,7 @@ static_assert(SP_COLS * SP_DQUADS % 64 == 0 && SP_ROWS + SP_CHUNK_MAX - 1 <= SP_
 // `first` is the table position (relative to `chunks`) of the chunk to walk first, the others following in table
 // order: a tile with one crossing chunk takes that one first and runs the INNER loop.  All chunks inside:
 // <INNER, !FIRST_ANY>; one crossing chunk: <INNER, FIRST_ANY>; anything else: <!INNER, FIRST_ANY>, first = 0.
-template <int LCK, int NTAB, bool EP, bool INNER, bool FIRST_ANY>
+template <int LCK, int NTAB, bool EP, bool MIXED, bool INNER, bool FIRST_ANY>
 __device__ __forceinline__ void spmm_tile_lean(
     float (&lds)[3][SP_DSTAGE_FLOATS], int row0, int col0,
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
@@ -1124,6 +1169,7 @@ __device__ __forceinline__ void spmm_tile_lean(
 
     SpWindow<LCK, T> w0, w1;
     int s_cur, s_n1, s_n2;                  // shifts of the chunk whose window is read next, and of the two after it
+    int l_cur, l_n1, l_n2;                  // lengths of the chunk whose FMAs run next, and of the two after it
     {
         const Entry h0 = fetch(0), h1 = fetch(1), h2 = fetch(2);
         issue(0, lds0, h0, std::false_type{}, std::integral_constant<bool, !FIRST_ANY>{});
@@ -1132,6 +1178,9 @@ __device__ __forceinline__ void spmm_tile_lean(
         s_cur = h0.s0;
         s_n1 = h1.s0;
         s_n2 = h2.s0;
+        l_cur = h0.len;
+        l_n1 = h1.len;
+        l_n2 = h2.len;
     }
     Entry e0 = fetch(3), e1 = e0;
     // The first window can be read as soon as chunk 0 (and the destination values) is in: the loads of
@@ -1150,7 +1199,7 @@ __device__ __forceinline__ void spmm_tile_lean(
     auto run_loop = [&](auto three_c) __attribute__((always_inline)) {
     constexpr bool THREE = decltype(three_c)::value;
     auto iteration = [&](int c, int b, int b1, SpWindow<LCK, T> &cur, SpWindow<LCK, T> &nxt, const Entry &use, Entry &next) __attribute__((always_inline)) {
-        spmm_rows_range<LCK, T, 0, JH>(acc, cur);
+        spmm_rows_chunk<LCK, T, 0, JH, MIXED>(acc, cur, l_cur);
         // chunk c+1 must be in; the loads of chunk c+2 (requested whenever c+2 < 3 or it exists) may stay out
         const bool younger = (c + 2 < 3) | (c + 2 < nchunks);
         if (!younger) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -1163,7 +1212,10 @@ __device__ __forceinline__ void spmm_tile_lean(
         s_n1 = s_n2;
         s_n2 = use.s0;
         next = fetch(c + 4);
-        spmm_rows_range<LCK, T, JH, LCK>(acc, cur);
+        spmm_rows_chunk<LCK, T, JH, LCK, MIXED>(acc, cur, l_cur);
+        l_cur = l_n1;
+        l_n1 = l_n2;
+        l_n2 = use.len;
     };
     int c = 0, b = 0, b1 = 1, b2 = 2;
     if (nchunks & 1) {
@@ -1236,7 +1288,8 @@ __device__ __forceinline__ void spmm_tile_lean(
 }
 
 // EP = false: the plain product (no bias, no activation); EP = true applies `ep`.
-template <int LCK, int T, int NTAB, bool EP>
+// MIXED = true: the table has chunks shorter than LCK (their missing diagonals are skipped, see spmm_rows_chunk).
+template <int LCK, int T, int NTAB, bool EP, bool MIXED>
 __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     const Chunk *__restrict__ chunks, int nchunks, const float *__restrict__ vals, int stride,
     int ashift, const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
@@ -1320,17 +1373,17 @@ __global__ __launch_bounds__(64 * SpShape<T>::WAVES, 4) void spmm_tiled_kernel(
     // only the chunks inside the operand are walked; the others would add zeros
     // A tile with one crossing chunk walks that chunk first: everything the loop then touches lies inside.
     if (lean && inner)
-        spmm_tile_lean<LCK, NTAB, EP, true, false>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
+        spmm_tile_lean<LCK, NTAB, EP, MIXED, true, false>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
                                                    ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, slot_step, ep);
     else if (lean && crossing == 1 && c_hi > c_lo)
-        spmm_tile_lean<LCK, NTAB, EP, true, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
+        spmm_tile_lean<LCK, NTAB, EP, MIXED, true, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
                                                   ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes,
                                                   cross_at - c_lo, slot_step, ep);
     else if (lean)
-        spmm_tile_lean<LCK, NTAB, EP, false, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
+        spmm_tile_lean<LCK, NTAB, EP, MIXED, false, true>(lds3, row0, col0, chunks + c_lo, c_hi - c_lo, vals, stride, ashift, X,
                                                    ldx, Y, ldy, n_out, n_in, batch, alpha, beta, a_bytes, 0, slot_step, ep);
     else
-        spmm_tile_edge<LCK, T, NTAB, EP>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
+        spmm_tile_edge<LCK, T, NTAB, EP, MIXED>(lds, row0, col0, chunks, nchunks, vals, stride, ashift, X, ldx, Y, ldy,
                                          n_out, n_in, batch, alpha, beta, a_bytes, ep);
 }
 
@@ -2174,6 +2227,7 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
     while (done < batch) {
         const int slab = batch - done < 65535 * CB ? batch - done : 65535 * CB;
         const dim3 grid(gx, (unsigned)((slab + CB - 1) / CB));
+        note_kernel("spmm_generic_kernel<%d>", CB);
         hipLaunchKernelGGL(spmm_generic_kernel<CB>, grid, dim3(256), 0, stream,
                            A.offsets_dev, A.nd, vals, A.stride, A.h, A.w, A.rf,
                            B + (long long)done * ldb, ldb, dst + (long long)done * ldd, ldd,
@@ -2219,6 +2273,7 @@ struct SpLaunch {
     dim3 grid;
     hipStream_t stream;
     int lck;
+    bool mixed;                 // some chunk of the table is shorter than lck
 };
 // The walking kernel's launch (its unit instantiates the kernel); returns hipErrorNotSupported when no
 // instantiation fits the table.
@@ -2235,8 +2290,7 @@ struct WalkLaunch {
     unsigned a_bytes;
     hipStream_t stream;
 };
-hipError_t spmm_walk_launch(const WalkLaunch &L, bool dry_run);
-int spmm_walk_tile_rows(int lck, int k, int s0);     // output rows per tile of the instantiation that serves the window; 0: none
+hipError_t spmm_walk_launch(const WalkLaunch &L);
 hipError_t spmm_tiled_launch_1_5(const SpLaunch &L);
 hipError_t spmm_tiled_launch_6_9(const SpLaunch &L);
 hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
@@ -2245,16 +2299,24 @@ hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
 // at the sizes this path is measured on.
 #define CUVDIA_SPMM_ARGS L.chunks, L.nchunks, L.vals, L.stride, L.ashift, L.B, L.ldb, L.dst, L.ldd, L.n_out, L.n_in, \
                          L.batch, L.alpha, L.beta, L.col_tiles, L.col_group, L.a_bytes, L.s_min, L.s_max, L.period_tiles, L.slot_step, L.ep
+#define CUVDIA_SPMM_LAUNCH_ONE(K, NTAB, EP, MIXED)                                                                    \
+    hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, NTAB, EP, MIXED>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS)
+#define CUVDIA_SPMM_LAUNCH_TAB(K, NTAB)                                                                               \
+    do {                                                                                                              \
+        if (K > 1 && L.mixed) {                                                                                       \
+            if (fused) CUVDIA_SPMM_LAUNCH_ONE(K, NTAB, true, (K > 1));                                                \
+            else CUVDIA_SPMM_LAUNCH_ONE(K, NTAB, false, (K > 1));                                                     \
+        } else {                                                                                                      \
+            if (fused) CUVDIA_SPMM_LAUNCH_ONE(K, NTAB, true, false);                                                  \
+            else CUVDIA_SPMM_LAUNCH_ONE(K, NTAB, false, false);                                                       \
+        }                                                                                                             \
+    } while (0)
 #define CUVDIA_SPMM_LAUNCH(K)                                                                                         \
     case K:                                                                                                           \
-        if (L.nchunks <= 64 && !fused)                                                                                \
-            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 1, false>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS); \
-        else if (L.nchunks <= 64)                                                                                     \
-            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 1, true>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS);  \
-        else if (!fused)                                                                                              \
-            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 4, false>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS); \
-        else                                                                                                          \
-            hipLaunchKernelGGL((spmm_tiled_kernel<K, 8, 4, true>), L.grid, dim3(512), 0, L.stream, CUVDIA_SPMM_ARGS);  \
+        note_kernel("spmm_tiled_kernel<%d, 8, %d, %s, %s>", K, L.nchunks <= 64 ? 1 : 4, fused ? "true" : "false",     \
+                    (K > 1 && L.mixed) ? "true" : "false");                                                           \
+        if (L.nchunks <= 64) CUVDIA_SPMM_LAUNCH_TAB(K, 1);                                                            \
+        else CUVDIA_SPMM_LAUNCH_TAB(K, 4);                                                                            \
         break;
 #if CUVDIA_IN_PART(5)
 // rows per wave of the instantiation that serves a window of k rows of lck diagonals whose first shift is
@@ -2269,18 +2331,39 @@ static int walk_rows_per_wave(int lck, int k, int s0)
     return 0;
 }
 int spmm_walk_tile_rows(int lck, int k, int s0) { return 8 * walk_rows_per_wave(lck, k, s0); }
-hipError_t spmm_walk_launch(const WalkLaunch &L, bool dry_run)
+// Tiles per segment of a walking launch, 0 when the walking kernel does not run: no instantiation for the
+// window, row counts that its tiles do not divide, or -- unless `forced` -- a launch that would not fill the chip.
+// Segments are as long as they can be while the launch still has SP_WALK_WGS workgroups, but no shorter than
+// the window has rows: a segment of S tiles stages S + k - 1 blocks.
+int spmm_walk_plan(int lck, int k, int s0, int period, long long n_out, long long n_in, long long col_tiles,
+                   bool forced, long long *workgroups)
+{
+    if (workgroups) *workgroups = 0;
+    const int rows = spmm_walk_tile_rows(lck, k, s0);
+    if (rows == 0 || n_out % rows != 0 || n_in % 4 != 0 || period % rows != 0) return 0;
+    const long long tp = period / rows;
+    const long long walk_len = (n_out / rows + tp - 1) / tp;
+    const long long walks = tp * col_tiles;
+    long long nseg = (SP_WALK_WGS + walks - 1) / walks;
+    if (nseg > walk_len / k) nseg = walk_len / k;
+    if (forced && nseg < 1) nseg = 1;
+    if (nseg < 1 || !(forced || nseg * walks >= SP_WALK_MIN_WGS)) return 0;
+    const long long seg_tiles = (walk_len + nseg - 1) / nseg;
+    if (workgroups) *workgroups = ((walk_len + seg_tiles - 1) / seg_tiles) * walks;
+    return (int)seg_tiles;
+}
+hipError_t spmm_walk_launch(const WalkLaunch &L)
 {
     const int rows = spmm_walk_tile_rows(L.lck, L.k, L.s0);
     if (rows == 0) return hipErrorNotSupported;
-    if (L.n_out % rows != 0 || L.n_in % 4 != 0 || L.period % rows != 0) return hipErrorNotSupported;
-    if (dry_run) return hipSuccess;
+    if (L.n_out % rows != 0 || L.n_in % 4 != 0 || L.period % rows != 0 || L.seg_tiles < 1) return hipErrorNotSupported;
     const int tp = L.period / rows;
     const int walk_len = (L.n_out / rows + tp - 1) / tp;
     const int nseg = (walk_len + L.seg_tiles - 1) / L.seg_tiles;
     const dim3 grid((unsigned)((long long)nseg * tp * L.col_tiles));
 #define CUVDIA_WALK_ARGS L.tab, L.ngroups, L.period, L.s0, L.astep4, L.seg_tiles, L.vals, L.B, L.ldb, L.dst, L.ldd, \
                          L.n_out, L.n_in, L.batch, L.alpha, L.beta, L.col_tiles, L.a_bytes
+    note_kernel("spmm_walk_kernel<%d, %d, 8, %d>", L.lck, L.lck, L.lck == 7 ? 1 : L.lck == 5 ? 2 : 3);
     if (L.lck == 7) hipLaunchKernelGGL((spmm_walk_kernel<7, 7, 8, 1>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
     else if (L.lck == 5) hipLaunchKernelGGL((spmm_walk_kernel<5, 5, 8, 2>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
     else hipLaunchKernelGGL((spmm_walk_kernel<3, 3, 8, 3>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
@@ -2322,6 +2405,8 @@ hipError_t spmm_tiled_launch_10_13(const SpLaunch &L)
 }
 #endif
 #undef CUVDIA_SPMM_LAUNCH
+#undef CUVDIA_SPMM_LAUNCH_TAB
+#undef CUVDIA_SPMM_LAUNCH_ONE
 #undef CUVDIA_SPMM_ARGS
 
 #if CUVDIA_IN_PART(4)
@@ -2345,21 +2430,11 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     if (walk >= 0 && wk.tab_dev != nullptr && ep.bias == nullptr && ep.act == 0) {
         WalkLaunch W{wk.tab_dev, wk.ngroups, wk.period, wk.s0, wk.astep4, wk.lck, wk.k, 0, vals, B, ldb, dst, ldd,
                      n_out, n_in, batch, alpha, beta, (int)col_tiles, (unsigned)((long long)A.nd * A.stride * 4), stream};
-        if (spmm_walk_launch(W, true) == hipSuccess) {
-            // Segments: as long as they can be while the launch still fills the chip (SP_WALK_WGS workgroups),
-            // but no shorter than the window has rows -- a segment of S tiles stages S + k - 1 blocks.
-            const int rows = spmm_walk_tile_rows(wk.lck, wk.k, wk.s0);
-            const long long tp = wk.period / rows;
-            const long long walk_len = (n_out / rows + tp - 1) / tp;
-            const long long walks = tp * col_tiles;
-            long long nseg = (SP_WALK_WGS + walks - 1) / walks;
-            if (nseg > walk_len / wk.k) nseg = walk_len / wk.k;
-            if (walk > 0 && nseg < 1) nseg = 1;
-            if (nseg >= 1 && (walk > 0 || nseg * walks >= SP_WALK_MIN_WGS)) {
-                W.seg_tiles = (int)((walk_len + nseg - 1) / nseg);
-                if (walked) *walked = true;
-                return spmm_walk_launch(W, false);
-            }
+        const int seg_tiles = spmm_walk_plan(wk.lck, wk.k, wk.s0, wk.period, n_out, n_in, col_tiles, walk > 0, nullptr);
+        if (seg_tiles > 0) {
+            W.seg_tiles = seg_tiles;
+            if (walked) *walked = true;
+            return spmm_walk_launch(W);
         }
     }
     if (walk > 0) return hipErrorNotSupported;
@@ -2371,7 +2446,8 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
                      (wk.tab_dev != nullptr && wk.period % SP_ROWS == 0 && row_tiles * col_tiles > SP_RENUMBER_MIN_TILES)
                          ? wk.period / SP_ROWS : 0,
                      trans ? A.slot_step_t : A.slot_step_n, ep,
-                     dim3((unsigned)(row_tiles * col_tiles)), stream, lck};
+                     dim3((unsigned)(row_tiles * col_tiles)), stream, lck,
+                     (trans ? A.min_len_t : A.min_len_n) != lck};
     if (lck <= 5) return spmm_tiled_launch_1_5(L);
     if (lck <= 9) return spmm_tiled_launch_6_9(L);
     return spmm_tiled_launch_10_13(L);
@@ -2385,6 +2461,7 @@ hipError_t launch_dd2dia_generic(const DiaView &C, float *vals, const float *A, 
     int done = 0;
     while (done < C.nd) {
         const int slab = C.nd - done < 65535 ? C.nd - done : 65535;
+        note_kernel("dd2dia_generic_kernel");
         hipLaunchKernelGGL(dd2dia_generic_kernel, dim3(gx, (unsigned)slab), dim3(256), 0, stream,
                            C.offsets_dev + done, vals + (long long)done * C.stride, C.stride,
                            C.h, C.w, C.rf, A, lda, B, ldb, batch, alpha, beta);
@@ -2521,6 +2598,9 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     case L:                                                                                              \
         hipLaunchKernelGGL((dd2dia_tiled_kernel<L, true, false>), grid, dim3(256), 0, stream, CUVDIA_DD_ARGS);      \
         break;
+    if (lc > CHUNK_MAX) note_kernel("dd2dia_tiled_kernel<%d, true, false, 0>", lc);
+    else note_kernel("dd2dia_tiled_kernel<%d, %s, %s, %d>", lc, (shifted || wide || pairs || a_vec) ? "true" : "false",
+                     (shifted || wide || pairs) ? "true" : "false", shifted ? DD_SHIFTED : wide ? DD_WIDE : DD_NARROW);
     switch (lc) {
         CUVDIA_DD_LAUNCH(1) CUVDIA_DD_LAUNCH(2) CUVDIA_DD_LAUNCH(3) CUVDIA_DD_LAUNCH(4)
         CUVDIA_DD_LAUNCH(5) CUVDIA_DD_LAUNCH(6) CUVDIA_DD_LAUNCH(7) CUVDIA_DD_LAUNCH(8)

@@ -65,7 +65,15 @@ hipError_t launch_spmm_generic(const DiaView &A, const float *vals, const float 
 // -1 -- never the walking kernel.  *walked (if not null) tells which ran.
 // Output rows per tile of the walking kernel's instantiation for a window of k rows of lck diagonals whose first
 // shift is s0; 0 when there is none.
+// Records the name of the kernel a launcher is about to launch, written the way a profiler prints it
+// ("spmm_tiled_kernel<7, 8, 1, false>"), for cuvdia_last_kernel(); per host thread.
+void note_kernel(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 int spmm_walk_tile_rows(int lck, int k, int s0);
+// Tiles per segment of the walking launch for such a window on n_out x n_in rows and col_tiles tiles of 64 batch
+// columns, and the launch's workgroups; 0 when the walking kernel does not run there (no instantiation, row
+// counts its tiles do not divide, or -- unless forced -- too few workgroups to fill the chip).
+int spmm_walk_plan(int lck, int k, int s0, int period, long long n_out, long long n_in, long long col_tiles,
+                   bool forced, long long *workgroups);
 hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B, long long ldb,
                              float *dst, long long ldd, int batch, bool trans,
                              float alpha, float beta, SpEpilogue ep, hipStream_t stream,

@@ -576,6 +576,7 @@ hipError_t launch_spmm_rows(const DiaView &A, const float *vals, const float *B,
 #define RW_ARGS trans ? A.chunks_t_dev : A.chunks_n_dev, trans ? A.n_chunks_t : A.n_chunks_n, vals, A.stride, trans ? 1 : 0, \
                 trans ? A.slot_step_t : A.slot_step_n, B, ldb, dst, ldd, n_out, n_in, batch, alpha, beta, (int)col_tiles, \
                 (unsigned)((long long)A.nd * A.stride * 4)
+    note_kernel("spmm_rows_kernel<%d>", lck);
     if (lck == 7) {
         hipLaunchKernelGGL((spmm_rows_kernel<7>), grid, dim3(64 * RW_WAVES), rw_lds_bytes(7), stream, RW_ARGS);
     } else if (lck == 13) {

@@ -7,7 +7,7 @@
 // The descriptor classes keep their names and constructors; on the device the
 // descriptor is the matrix's O(num_dia) run table instead of the reference's
 // list of 16x16 blocks (densedense_to_sparse.cu:123-171).  The
-// host_memory_space twin of densedense_to_dia lives with the test oracle.
+// host_memory_space twin of densedense_to_dia is in cuv/matrix_ops/host_ops.hpp.
 #ifndef __DENSEDENSE_TO_SPARSE_HPP__
 #define __DENSEDENSE_TO_SPARSE_HPP__
 

@@ -5,7 +5,7 @@
 // the preconditions of the host version (diagonals.cu:28-29), result visible
 // on return.  The mean runs over the valid slots of a diagonal, as in the
 // reference's host version; padding is never read.  The host_memory_space
-// twin lives with the test oracle.
+// twin is in cuv/matrix_ops/host_ops.hpp.
 #ifndef __CUV_DIAGONALS_HPP__
 #define __CUV_DIAGONALS_HPP__
 

@@ -6,7 +6,7 @@
 // preconditions (each throws std::runtime_error with the stringified
 // condition), results visible on return.  The work is done by
 // cuvdia_spmm_f32 (hand-written HIP for gfx950); there is no CPU fallback in
-// this header -- the host_memory_space twins live with the test oracle.
+// this header -- the host_memory_space twins are in cuv/matrix_ops/host_ops.hpp.
 #ifndef __CUV_MATRIX_OPS_HPP__
 #define __CUV_MATRIX_OPS_HPP__
 

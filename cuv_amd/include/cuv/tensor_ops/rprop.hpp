@@ -3,8 +3,8 @@
 // Mirrors src/cuv/tensor_ops/rprop.hpp:127-128,150-154 of the reference
 // (bodies in src/cuv/tensor_ops/rprop.cu:148-156,324-346) for
 // dev_memory_space: same signature and preconditions, result visible on
-// return.  For a DIA weight matrix call it on W.vec() and dW.vec().  The
-// host_memory_space twin lives with the test oracle.
+// return.  For a DIA weight matrix call it on W.vec() and dW.vec().  This
+// tree has no host_memory_space twin of it (the reference's is rprop.cu:148-156 on host tensors).
 #ifndef __CUV_RPROP_HPP__
 #define __CUV_RPROP_HPP__
 

@@ -124,11 +124,25 @@ int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap
  * is not 0.  Returns 0: no window table; 1: a window table that the products
  * walk tile by tile (with their row tiles numbered period-major on launches of
  * many rounds); 2: a window table with a walking kernel (centred 3x3, 5x5 or
- * 7x7 window, period a multiple of 64: the kernel the automatic choice takes
- * on products of many tiles whose row counts are multiples of 64); negative:
- * an error.  No counterpart in the reference. */
+ * 7x7 window, period a multiple of 64); negative: an error.  The answer is
+ * about the TABLE only.  Whether a given product runs the walking kernel also
+ * depends on its shape -- cuvdia_plan_walk_launch answers that.  No
+ * counterpart in the reference. */
 int cuvdia_plan_walk(const int *offsets_host, int nd, int stride, int transposed,
                      int *period, int *k, int *ngroups, int *lck);
+
+/* Pure host function: does the automatic choice of cuvdia_spmm_f32 run the
+ * walking kernel for the plain product (no bias, no activation) of an h x w
+ * matrix with this table (row_fact 1) and `batch` packed dense columns?
+ * Returns the number of workgroups of that launch, or 0 when another kernel
+ * serves: the table is no window table with a walking kernel (see
+ * cuvdia_plan_walk), the output row count is no multiple of 64 or the input
+ * row count no multiple of 4, batch < 24, or the launch would have fewer than
+ * 384 workgroups (a product of few tiles is served tile by tile).  Negative:
+ * an error.  cuvdia_set_path(CUVDIA_PATH_WALK) waives the last condition
+ * only.  No counterpart in the reference. */
+long long cuvdia_plan_walk_launch(const int *offsets_host, int nd, int stride, int h, int w,
+                                  int transposed, int batch);
 
 /* dst = beta*dst + alpha*op(A)*B for a batch of dense columns.
  * Replaces prod<float,dev_memory_space,column_major>(dst, dia A, B, transA,
@@ -274,8 +288,13 @@ int cuvdia_dd2dia_offsets_f32(float *C_vals_device, const int *offsets_host,
  * device copy of the offset table and of the chunk table the kernels walk -- which a
  * descriptor keeps in memory it allocates -- lives in a static device array
  * of 20480 bytes inside the library (one copy per GPU, held until the process
- * ends), so the call performs no hipMalloc, no hipFree and no allocating
- * library call, and touches neither the descriptor cache nor its lock.  Every
+ * ends), so the call allocates and frees no DEVICE memory -- no hipMalloc, no
+ * hipFree, no allocating library call -- and touches neither the descriptor
+ * cache nor its lock.  (It does plan the chunk table on the host, in a small
+ * std::vector on the host heap.)  The first call on a GPU also resolves the
+ * array's address there (hipGetSymbolAddress, which may load the library's
+ * code object): make that first call outside stream capture; every later
+ * call on that GPU may be captured.  Every
  * call rewrites the part of the array it uses with one small fill kernel per
  * 3584 bytes of table, enqueued on `stream` ahead of the product (the bytes
  * travel as kernel arguments, so the host table may be reused on return).
@@ -307,6 +326,13 @@ int cuvdia_set_path(int path);
  * (CUVDIA_PATH_GENERIC, CUVDIA_PATH_TILED or -- a product served by the
  * walking kernel -- CUVDIA_PATH_WALK; 0 before any call). */
 int cuvdia_last_path(void);
+
+/* Name of the kernel the most recent compute call on this thread launched
+ * (the last one, where a call launches several), written as a profiler
+ * prints it, e.g. "spmm_tiled_kernel<7, 8, 1, false>"; "" before any call.
+ * The string belongs to the library and is overwritten by the next call.
+ * No counterpart in the reference. */
+const char *cuvdia_last_kernel(void);
 
 /* Static string for an error code. */
 const char *cuvdia_strerror(int code);

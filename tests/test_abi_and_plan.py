@@ -265,3 +265,41 @@ def test_tables_that_are_no_window_tables():
     assert _walk([dx for dx in range(3)] + [64 + dx for dx in range(3)] + [5000 + dx for dx in range(3)], 8192)[0] == 0
     from cuv_amd import _lib
     assert _lib.lib().cuvdia_plan_walk(None, 3, 16, 0, None, None, None, None) == _lib.EINVAL
+
+
+def _walk_launch(offs, stride, h, w, batch, transposed=0):
+    from cuv_amd import _lib
+    offs = np.ascontiguousarray(offs, np.int32)
+    ip = ctypes.POINTER(ctypes.c_int)
+    return _lib.lib().cuvdia_plan_walk_launch(offs.ctypes.data_as(ip), offs.size, stride, h, w, transposed, batch)
+
+
+def test_walk_launch_depends_on_the_shape_too():
+    """cuvdia_plan_walk judges the table; whether a product walks also needs row counts the 64-row tiles divide,
+    batch >= 24 and a launch of at least 384 workgroups."""
+    from cuv_amd import _lib, workloads as W
+    n = 512 * 512
+    offs = W.window_offsets(512, 7)
+    assert _walk(offs, n)[0] == 2
+    # 512 x 512 map, batch 128: tp = 8 tiles per period, 2 column tiles -> 16 walks of 512 tiles, 32 segments each
+    assert _walk_launch(offs, n, n, n, 128) == 512
+    assert _walk_launch(offs, n, n, n, 128, 1) == 512
+    # a narrow batch goes to the generic kernels
+    assert _walk_launch(offs, n, n, n, 16) == 0
+    # output rows no multiple of 64 (the table is the same, the matrix ends 40 rows early), both directions
+    assert _walk(offs, n)[0] == 2
+    assert _walk_launch(offs, n, n - 40, n, 128) == 0
+    assert _walk_launch(offs, n, n, n - 40, 128, 1) == 0
+    # ... but only the OUTPUT side needs multiples of 64; the input side multiples of 4
+    assert _walk_launch(offs, n, n, n - 40, 128) > 0
+    assert _walk_launch(offs, n, n, n - 42, 128) == 0
+    # the headline layer's shape: 128 x 128 map, batch 128 -- too few workgroups, served tile by tile
+    small = W.window_offsets(128, 7)
+    assert _walk(small, 128 * 128)[0] == 2
+    assert _walk_launch(small, 128 * 128, 128 * 128, 128 * 128, 128) == 0
+    # no window table / no walking kernel for the window
+    assert _walk_launch(list(range(-3, 4)), 4096, 4096, 4096, 128) == 0
+    assert _walk_launch(W.window_offsets(256, 13, 4), 4 * 256 * 256, 4 * 256 * 256, 4 * 256 * 256, 512) == 0
+    # argument errors
+    assert _walk_launch(offs, n, n, n, -1) == _lib.EINVAL
+    assert _walk_launch(offs, n - 8, n, n, 128) < 0          # stride shorter than the diagonals

@@ -245,9 +245,8 @@ def test_dd2dia_nan_in_the_gaps_around_the_operands(oracle, gu, offs):
 def test_inf_in_the_dense_operand_reaches_only_the_rows_that_use_it(oracle, gu):
     """One Inf in B: with a table whose chunks all have the table's longest length -- every 2-d window pattern --
     the tiled kernels multiply exactly the elements the matrix stores, so the Inf shows up in the result rows
-    that reference its row and nowhere else, as in the generic kernels and the reference's host loop.  (A
-    table that mixes chunk lengths pads the shorter chunks with zero-valued diagonals in the tiled kernels;
-    0 * Inf then yields NaN in neighbouring rows: documented in include/cuvdia.h.)"""
+    that reference its row and nowhere else, as in the generic kernels and the reference's host loop.  (Tables
+    that mix chunk lengths: the next test.)"""
     from cuv_amd import _lib
     rng = np.random.default_rng(5)
     h = w = 1024
@@ -267,6 +266,42 @@ def test_inf_in_the_dense_operand_reaches_only_the_rows_that_use_it(oracle, gu):
         assert (~fin).sum() == len(offs)                 # the rows that use B[500, 3], in column 3 only
         a, b = outs[_lib.PATH_GENERIC], outs[_lib.PATH_TILED]
         np.testing.assert_allclose(a[fin], b[fin], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("offs", [list(range(-3, 4)) + [100, 101],
+                                  list(range(-8, -1)) + list(range(0, 8)) + [100, 101]],
+                         ids=["7+2", "7+8+2"])
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_non_finite_values_with_chunks_of_mixed_length(oracle, gu, offs, trans):
+    """Inf and NaN in B under a table whose chunks differ in length (the kernel is built for the longest): a
+    shorter chunk must run only the diagonals it has, or 0 * Inf from the dense rows next to its own would put
+    NaN into result rows that do not reference them.  The masks of Inf, NaN and finite results equal the
+    oracle's on every kernel family -- in the interior, in the tiles at both ends of the operand (which take
+    the other body of the tiled kernel) and with beta != 0."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(len(offs))
+    h = w = 1024
+    A = _rand_dia(oracle, rng, h, w, offs)
+    B = np.asfortranarray(rng.uniform(-1, 1, (w, 70)).astype(np.float32))
+    dst = np.asfortranarray(rng.uniform(-1, 1, (h, 70)).astype(np.float32))
+    B[600, 3] = np.inf
+    B[211, 40] = np.nan
+    B[2, 5] = -np.inf           # first tile
+    B[1021, 6] = np.nan         # last tile
+    B[130, 69] = np.inf         # the second column tile (6 valid columns)
+    for alpha, beta, d in ((1.0, 0.0, None), (0.75, -1.5, dst)):
+        with np.errstate(invalid="ignore"):
+            ref = oracle.prod(A, B, d, trans, alpha, beta)
+        assert 0 < (~np.isfinite(ref)).sum() < 5 * len(offs) + 1
+        for path in _paths(1):
+            got, ran = gu.gpu_prod(A, B, d, trans, alpha, beta, path)
+            assert ran == path
+            what = "path %d, %s, beta %g" % (path, trans, beta)
+            assert np.array_equal(np.isnan(got), np.isnan(ref)), what
+            assert np.array_equal(np.isposinf(got), np.isposinf(ref)), what
+            assert np.array_equal(np.isneginf(got), np.isneginf(ref)), what
+            fin = np.isfinite(ref)
+            np.testing.assert_allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-5, err_msg=what)
 
 
 def test_batch_zero_and_errors(oracle, gu):

@@ -142,6 +142,81 @@ def test_single_main_diagonal_is_elementwise(oracle):
     assert np.array_equal(oracle.spmv(d, x, np.zeros(20, np.float32)), d.vals[:20] * x)
 
 
+def _identity_dia(o, n):
+    d = o.Dia(n, n, [0], None, 1)
+    d.vals[:] = 0
+    d.vals[:n] = 1
+    return d
+
+
+def test_bias_act_on_identity_is_the_logistic_function(oracle):
+    """With A the identity the layer update is sigmoid(x + bias) element by element: checked against
+    1 / (1 + exp(-t)) evaluated in fp64 by math.exp on the fp32 sum t, to fp32 rounding of the steps
+    (expf, the add, the divide: below 1e-7 absolute on values in (0, 1))."""
+    import math
+    n, batch = 37, 5
+    rng = np.random.default_rng(31)
+    d = _identity_dia(oracle, n)
+    X = np.asfortranarray(rng.uniform(-6, 6, (n, batch)).astype(np.float32))
+    bias = rng.uniform(-2, 2, n).astype(np.float32)
+    got = oracle.prod_bias_act(d, X, None, "n", 1.0, 0.0, bias=bias, sigmoid=True)
+    assert got.dtype == np.float32 and got.shape == (n, batch)
+    worst = 0.0
+    for i in range(n):
+        for j in range(batch):
+            t = float(np.float32(X[i, j] + bias[i]))
+            worst = max(worst, abs(float(got[i, j]) - 1.0 / (1.0 + math.exp(-t))))
+    assert worst <= 1e-7, worst
+    # the transposed product of the identity is the same update
+    assert np.array_equal(got, oracle.prod_bias_act(d, X, None, "t", 1.0, 0.0, bias=bias, sigmoid=True))
+    # without the activation: the sum itself, rounded once
+    lin = oracle.prod_bias_act(d, X, None, "n", 1.0, 0.0, bias=bias, sigmoid=False)
+    assert np.array_equal(lin, (X + bias[:, None]).astype(np.float32))
+
+
+def test_bias_act_bias_is_added_per_row_and_exactly(oracle):
+    """The bias belongs to the output ROW (matrix_plus_col) and enters after the product: with power-of-two
+    biases and small-integer operands every step is exact, so the difference of two runs is the bias itself --
+    a bias added per column, before alpha, or scaled by beta fails."""
+    rng = np.random.default_rng(32)
+    h, w, batch = 24, 30, 6
+    d = _rand_dia(oracle, rng, h, w, [-3, 0, 2, 9])
+    d.vals[:] = np.where(np.isnan(d.vals), d.vals, np.round(d.vals * 4))
+    B = np.asfortranarray(rng.integers(-3, 4, (w, batch)).astype(np.float32))
+    dst = np.asfortranarray(rng.integers(-3, 4, (h, batch)).astype(np.float32))
+    bias = (2.0 ** rng.integers(-2, 4, h)).astype(np.float32)
+    base = oracle.prod_bias_act(d, B, dst, "n", 2.0, -0.5, bias=None, sigmoid=False)
+    withb = oracle.prod_bias_act(d, B, dst, "n", 2.0, -0.5, bias=bias, sigmoid=False)
+    assert np.array_equal(base, oracle.prod(d, B, dst, "n", 2.0, -0.5))
+    assert np.array_equal(withb - base, np.broadcast_to(bias[:, None], (h, batch)))
+    # transposed: the bias has one entry per column of A
+    bias_t = (2.0 ** rng.integers(-2, 4, w)).astype(np.float32)
+    Bt = np.asfortranarray(rng.integers(-3, 4, (h, batch)).astype(np.float32))
+    base_t = oracle.prod_bias_act(d, Bt, None, "t", 1.0, 0.0)
+    with_t = oracle.prod_bias_act(d, Bt, None, "t", 1.0, 0.0, bias=bias_t)
+    assert np.array_equal(with_t - base_t, np.broadcast_to(bias_t[:, None], (w, batch)))
+
+
+def test_bias_act_special_values(oracle):
+    """sigmoid(0) == 0.5 exactly; large arguments saturate to 0 and 1 without NaN; sigmoid(-t) == 1 - sigmoid(t)
+    to one rounding."""
+    n = 8
+    d = _identity_dia(oracle, n)
+    X = np.zeros((n, 3), np.float32, order="F")
+    assert np.array_equal(oracle.prod_bias_act(d, X, sigmoid=True), np.full((n, 3), 0.5, np.float32))
+    # a bias cancelling the input lands on 0.5 too
+    X[:] = 1.25
+    got = oracle.prod_bias_act(d, X, bias=np.full(n, -1.25, np.float32), sigmoid=True)
+    assert np.array_equal(got, np.full((n, 3), 0.5, np.float32))
+    with np.errstate(over="ignore"):
+        X[:, 0], X[:, 1], X[:, 2] = 200.0, -200.0, 3.0
+        sat = oracle.prod_bias_act(d, X, sigmoid=True)
+        assert np.all(sat[:, 0] == 1.0) and np.all(sat[:, 1] == 0.0) and not np.isnan(sat).any()
+        X[:, 1] = -3.0
+        sym = oracle.prod_bias_act(d, X, sigmoid=True)
+    assert np.all(np.abs(sym[:, 1] - (np.float32(1) - sym[:, 2])) <= 6e-8)
+
+
 def test_trans_equals_explicit_transpose(oracle):
     rng = np.random.default_rng(4)
     h, w, offs = 30, 22, [-4, 0, 1, 7]

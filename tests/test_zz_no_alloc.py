@@ -100,3 +100,84 @@ def test_noalloc_rejects_tables_beyond_its_capacity():
     assert rc == 0
     torch.cuda.synchronize()
     assert bool((out == 0.0).all())
+
+
+def test_noalloc_leaves_free_device_memory_unchanged(oracle):
+    """Free device memory as the driver reports it is the same before and after a series of calls with
+    tables of different sizes (the operands are allocated beforehand; the first call on the device, which
+    resolves the static array, is made before the first reading)."""
+    import torch
+    from cuv_amd import _lib
+    L = _lib.lib()
+    n, batch = 2048, 64
+    vals = torch.rand(64 * n, device="cuda:0")
+    B = torch.rand(batch * n, device="cuda:0")
+    out = torch.zeros(batch * n, device="cuda:0")
+
+    def call(offs):
+        offs = np.asarray(offs, np.int32)
+        rc = L.cuvdia_spmm_offsets_noalloc_f32(vals.data_ptr(), offs.ctypes.data_as(IP), len(offs), n, n, n, 1,
+                                               B.data_ptr(), n, out.data_ptr(), n, batch, b"n", 1.0, 0.0, None)
+        assert rc == 0, L.cuvdia_strerror(rc)
+
+    call([0, 1])
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for offs in (_window(32, 5), [-5, 0, 9], list(range(-30, 30)), [7 * i - 200 for i in range(64)]):
+        call(offs)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, "free device memory changed by %d bytes" % (free0 - free1)
+
+
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_noalloc_under_graph_capture(oracle, trans):
+    """A call recorded into a graph (after one eager call on the device) replays correctly: three replays with
+    the dense operand rewritten and eager work between them, each against the allocating entry point run
+    eagerly on the same operands."""
+    import torch
+    from cuv_amd import _lib, dia as D
+    L = _lib.lib()
+    rng = np.random.default_rng(977)
+    h, w, batch = 1024, 1024, 64
+    A = _rand_dia(oracle, rng, h, w, _window(32, 5))
+    n_in, n_out = (h, w) if trans == "t" else (w, h)
+    vals = torch.from_numpy(A.vals).cuda()
+    Bd = torch.empty(batch, n_in, device="cuda:0")
+    dst0 = torch.from_numpy(rng.uniform(-1, 1, (batch, n_out)).astype(np.float32)).cuda()
+    out = torch.empty(batch, n_out, device="cuda:0")
+    ref = torch.empty(batch, n_out, device="cuda:0")
+    offs = A.offsets
+
+    def run(fn, dst, stream):
+        rc = fn(vals.data_ptr(), offs.ctypes.data_as(IP), A.nd, A.stride, h, w, 1, Bd.data_ptr(), n_in,
+                dst.data_ptr(), n_out, batch, trans.encode(), 0.75, 0.5, stream)
+        assert rc == 0, L.cuvdia_strerror(rc)
+
+    Bd.copy_(torch.from_numpy(rng.uniform(-1, 1, (batch, n_in)).astype(np.float32)))
+    out.copy_(dst0)
+    run(L.cuvdia_spmm_offsets_noalloc_f32, out, None)          # the first call on the device: outside capture
+    torch.cuda.synchronize()
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        run(L.cuvdia_spmm_offsets_noalloc_f32, out, ctypes.c_void_p(side.cuda_stream))
+        graph.capture_end()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    for replay in range(3):
+        Bd.copy_(torch.from_numpy(rng.uniform(-1, 1, (batch, n_in)).astype(np.float32)))
+        out.copy_(dst0)
+        ref.copy_(dst0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        run(L.cuvdia_spmm_offsets_f32, ref, None)
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), "replay %d differs from the eager result" % replay
+        assert float(out.abs().sum()) > 0
+    assert L.cuvdia_cache_clear() == 0
