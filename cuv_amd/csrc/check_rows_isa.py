@@ -1,13 +1,13 @@
 #!/usr/bin/env python3
 """Build-time check of the machine code of spmm_rows.hip (run by the Makefile on the device pass's output).
 
-The rows-along-lanes kernel names its vector registers outright inside inline assembly (v32 and up: three sets of
+The rows-along-lanes kernel names its vector registers outright inside inline assembly (v44 and up: three sets of
 dense rows, the diagonal-value buffers, the sums, the halo) and loads into them asynchronously, across statement
 boundaries.  The compiler knows of them only through clobber lists, so two things are outside its guarantees and
 are verified here on the disassembly instead, before the code can reach a GPU:
 
-  1. Register ownership.  No compiler-generated instruction may touch v32 or above, except lane spills of scalar
-     registers into v64/v65 (which the kernel leaves free).  A compiler temporary in a register that has a load in
+  1. Register ownership.  No compiler-generated instruction may touch v44 or above, except lane spills of scalar
+     registers into v76/v77 (which the kernel leaves free).  A compiler temporary in a register that has a load in
      flight is overwritten when the load lands -- with a buffer descriptor under construction in it, the next
      load goes to a wild address.
   2. Wait states the compiler does not pad around inline assembly on gfx950:
@@ -25,12 +25,12 @@ import subprocess
 import sys
 import tempfile
 
-FIRST_OWNED = 32                 # RW_OWN2 in spmm_rows.hip: the lowest register the assembly names
-SPILL_LANES = (64, 65)           # left free between the own sets and the value buffers
+FIRST_OWNED = 44                 # RW_OWN2 in spmm_rows.hip: the lowest register the assembly names
+SPILL_LANES = (76, 77)           # left free between the own sets and the value buffers
 # what the assembly itself issues on the owned registers
 ASM_OPS = {'v_fmac_f32_e32', 'v_mov_b32_dpp', 'ds_read_b128', 'buffer_load_dwordx4', 'buffer_load_dword',
            'ds_write_b128'}
-ACC_FIRST = 100                  # RW_ACC: zeroed with v_mov_b32 v, 0 by the assembly
+ACC_FIRST = 112                  # RW_ACC: zeroed with v_mov_b32 v, 0 by the assembly
 
 
 def disassemble(path, llvm_bin):

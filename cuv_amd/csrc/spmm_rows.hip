@@ -16,7 +16,7 @@
 //     window of column c sits in consecutive registers from a multiple of 4, the 8 values of diagonal j in
 //     consecutive registers from 2 (mod 4) for j = 0, 1 (mod 4) and from 0 (mod 4) for j = 2, 3 (mod 4).  The
 //     compiler cannot place registers, so the chunk's arithmetic is one assembly statement on named registers
-//     (v64 and up; the compiler's own values stay below, which the build checks);
+//     (v44 and up; the compiler's own values stay below, which the build checks);
 //   * the last one or two lanes of a wave have no neighbour to take their halo from: they compute nothing that
 //     is stored, and a tile is 8 x 62 = 496 rows (LCK > 7) or 8 x 63 = 504 rows (LCK <= 7).
 //
@@ -53,19 +53,19 @@ constexpr int rw_abuf_bytes(int lck) { return 2 * lck * 1024; }
 constexpr int rw_lds_bytes(int lck) { return 3 * rw_abuf_bytes(lck) + 1024 > RW_WAVES * 8192 ? 3 * rw_abuf_bytes(lck) + 1024 : RW_WAVES * 8192; }
 
 // ---- the named registers --------------------------------------------------------------------------------
-//   v32 ..  v63   own dense rows, set 2: RW_OWN2 + 8 c + k (the compiler's own values stay below v32: the
+//   v44 ..  v75   own dense rows, set 2: RW_OWN2 + 8 c + k (the compiler's own values stay below v44: the
 //                 build checks the disassembly for that)
-//   v66 ..  v99   four buffers of 8 diagonal values (RW_A0, RW_A1: first register 2 mod 4; RW_A2, RW_A3: 0 mod 4)
-//   v100 .. v131  sums, RW_ACC + 8 c + t
-//   v132 .. v163  own dense rows, set 0: RW_OWN0 + 8 c + k      (window positions 0 .. 7)
-//   v164 .. v195  own dense rows, set 1 (chunk i uses set i mod 3 while the sets of chunks i + 1 and i + 2 load)
-//   v196 .. v243  halo: RW_HALO + 12 c + m                      (window positions 8 + m)
+//   v78 ..  v111  four buffers of 8 diagonal values (RW_A0, RW_A1: first register 2 mod 4; RW_A2, RW_A3: 0 mod 4)
+//   v112 .. v143  sums, RW_ACC + 8 c + t
+//   v144 .. v175  own dense rows, set 0: RW_OWN0 + 8 c + k      (window positions 0 .. 7)
+//   v176 .. v207  own dense rows, set 1 (chunk i uses set i mod 3 while the sets of chunks i + 1 and i + 2 load)
+//   v208 .. v255  halo: RW_HALO + 12 c + m                      (window positions 8 + m)
 // Every statement begins with RW_DEFS (symbols and macros are per statement: the assembler keeps macros for the
 // whole translation unit, and a statement can be instantiated more than once) and ends with RW_PURGE.  The
 // statement sets RW_P (the own set of the chunk being computed), RW_Q (the set being loaded) and RW_LCK first.
 #define RW_DEFS \
-    ".set RW_A0, 66\n.set RW_A1, 74\n.set RW_A2, 84\n.set RW_A3, 92\n" \
-    ".set RW_ACC, 100\n.set RW_OWN0, 132\n.set RW_OWN1, 164\n.set RW_OWN2, 32\n.set RW_HALO, 196\n" \
+    ".set RW_A0, 78\n.set RW_A1, 86\n.set RW_A2, 96\n.set RW_A3, 104\n" \
+    ".set RW_ACC, 112\n.set RW_OWN0, 144\n.set RW_OWN1, 176\n.set RW_OWN2, 44\n.set RW_HALO, 208\n" \
     ".macro RW_SETS p, q\n" \
     " .if \\p == 0\n .set RW_OWNP, RW_OWN0\n .endif\n .if \\p == 1\n .set RW_OWNP, RW_OWN1\n .endif\n .if \\p == 2\n .set RW_OWNP, RW_OWN2\n .endif\n" \
     " .if \\q == 0\n .set RW_OWNQ, RW_OWN0\n .endif\n .if \\q == 1\n .set RW_OWNQ, RW_OWN1\n .endif\n .if \\q == 2\n .set RW_OWNQ, RW_OWN2\n .endif\n" \
@@ -122,12 +122,12 @@ constexpr int rw_lds_bytes(int lck) { return 3 * rw_abuf_bytes(lck) + 1024 > RW_
     ".endm\n"
 #define RW_PURGE ".purgem RW_SETS\n.purgem RW_FMAD\n.purgem RW_HALOS\n.purgem RW_AREAD\n.purgem RW_AREADJ\n.purgem RW_FMADJ\n.purgem RW_XLOAD\n"
 
-#define RW_CLOB_OWN2 "v32","v33","v34","v35","v36","v37","v38","v39","v40","v41","v42","v43","v44","v45","v46","v47","v48","v49","v50","v51","v52","v53","v54","v55","v56","v57","v58","v59","v60","v61","v62","v63"
-#define RW_CLOB_A "v66","v67","v68","v69","v70","v71","v72","v73","v74","v75","v76","v77","v78","v79","v80","v81","v82","v83","v84","v85","v86","v87","v88","v89","v90","v91","v92","v93","v94","v95","v96","v97","v98","v99"
-#define RW_CLOB_ACC "v100","v101","v102","v103","v104","v105","v106","v107","v108","v109","v110","v111","v112","v113","v114","v115","v116","v117","v118","v119","v120","v121","v122","v123","v124","v125","v126","v127","v128","v129","v130","v131"
-#define RW_CLOB_OWN0 "v132","v133","v134","v135","v136","v137","v138","v139","v140","v141","v142","v143","v144","v145","v146","v147","v148","v149","v150","v151","v152","v153","v154","v155","v156","v157","v158","v159","v160","v161","v162","v163"
-#define RW_CLOB_OWN1 "v164","v165","v166","v167","v168","v169","v170","v171","v172","v173","v174","v175","v176","v177","v178","v179","v180","v181","v182","v183","v184","v185","v186","v187","v188","v189","v190","v191","v192","v193","v194","v195"
-#define RW_CLOB_HALO "v196","v197","v198","v199","v200","v201","v202","v203","v204","v205","v206","v207","v208","v209","v210","v211","v212","v213","v214","v215","v216","v217","v218","v219","v220","v221","v222","v223","v224","v225","v226","v227","v228","v229","v230","v231","v232","v233","v234","v235","v236","v237","v238","v239","v240","v241","v242","v243"
+#define RW_CLOB_OWN2 "v44","v45","v46","v47","v48","v49","v50","v51","v52","v53","v54","v55","v56","v57","v58","v59","v60","v61","v62","v63","v64","v65","v66","v67","v68","v69","v70","v71","v72","v73","v74","v75"
+#define RW_CLOB_A "v78","v79","v80","v81","v82","v83","v84","v85","v86","v87","v88","v89","v90","v91","v92","v93","v94","v95","v96","v97","v98","v99","v100","v101","v102","v103","v104","v105","v106","v107","v108","v109","v110","v111"
+#define RW_CLOB_ACC "v112","v113","v114","v115","v116","v117","v118","v119","v120","v121","v122","v123","v124","v125","v126","v127","v128","v129","v130","v131","v132","v133","v134","v135","v136","v137","v138","v139","v140","v141","v142","v143"
+#define RW_CLOB_OWN0 "v144","v145","v146","v147","v148","v149","v150","v151","v152","v153","v154","v155","v156","v157","v158","v159","v160","v161","v162","v163","v164","v165","v166","v167","v168","v169","v170","v171","v172","v173","v174","v175"
+#define RW_CLOB_OWN1 "v176","v177","v178","v179","v180","v181","v182","v183","v184","v185","v186","v187","v188","v189","v190","v191","v192","v193","v194","v195","v196","v197","v198","v199","v200","v201","v202","v203","v204","v205","v206","v207"
+#define RW_CLOB_HALO "v208","v209","v210","v211","v212","v213","v214","v215","v216","v217","v218","v219","v220","v221","v222","v223","v224","v225","v226","v227","v228","v229","v230","v231","v232","v233","v234","v235","v236","v237","v238","v239","v240","v241","v242","v243","v244","v245","v246","v247","v248","v249","v250","v251","v252","v253","v254","v255"
 #define RW_CLOB_ALL RW_CLOB_OWN2, RW_CLOB_A, RW_CLOB_ACC, RW_CLOB_OWN0, RW_CLOB_OWN1, RW_CLOB_HALO
 
 typedef int rw_int4 __attribute__((ext_vector_type(4)));
@@ -191,10 +191,11 @@ __device__ __forceinline__ void rw_lds_load_b32(rw_int4 rsrc, unsigned lds_byte_
 }
 
 // What a wave needs to request a chunk's operands: the dense rows of its 4 columns (8 loads of 16 bytes per
-// lane into own set Q) and its share of the chunk's diagonal values (NP loads that write LDS directly).
+// lane into own set Q, the column in the lane's byte offset) and its share of the chunk's diagonal values (NP
+// loads that write LDS directly).
 struct RwRequest {
     rw_int4 xr;                 // dense operand of the tile's columns (an empty resource: nothing is fetched, zeros arrive)
-    unsigned xs[RW_C];          // scalar byte offset of each column's first row
+    unsigned xs;                // scalar byte offset of the chunk's first dense row
     rw_int4 ar;                 // the diagonal values (or the empty resource)
     unsigned as;                // scalar byte offset of the chunk's first diagonal, at the tile's first row
     unsigned m0_base;           // LDS byte address of the wave's first piece in the value buffer
@@ -210,23 +211,23 @@ struct RwRequest {
     " .if " #J " + 2 < RW_LCK\n RW_AREADJ (" #J "+2), %[aread]\n s_waitcnt lgkmcnt(4)\n .else\n  .if " #J " + 1 < RW_LCK\n s_waitcnt lgkmcnt(2)\n  .else\n s_waitcnt lgkmcnt(0)\n  .endif\n .endif\n" \
     " .if ((" #J " ^ RW_WPAR) & 1)\n s_setprio 0\n .else\n s_setprio 3\n .endif\n" \
     " .if RW_LCK > 8\n" \
-    "  .if " #J " == 0\n RW_XLOAD 0, %[xvoff], %[xrs], %[xs0]\n .endif\n" \
-    "  .if " #J " == 1\n RW_XLOAD 1, %[xvoff], %[xrs], %[xs0]\n .endif\n" \
-    "  .if " #J " == 2\n RW_XLOAD 2, %[xvoff], %[xrs], %[xs1]\n .endif\n" \
-    "  .if " #J " == 3\n RW_XLOAD 3, %[xvoff], %[xrs], %[xs1]\n .endif\n" \
-    "  .if " #J " == 4\n RW_XLOAD 4, %[xvoff], %[xrs], %[xs2]\n .endif\n" \
-    "  .if " #J " == 5\n RW_XLOAD 5, %[xvoff], %[xrs], %[xs2]\n .endif\n" \
-    "  .if " #J " == 6\n RW_XLOAD 6, %[xvoff], %[xrs], %[xs3]\n .endif\n" \
-    "  .if " #J " == 7\n RW_XLOAD 7, %[xvoff], %[xrs], %[xs3]\n .endif\n" \
+    "  .if " #J " == 0\n RW_XLOAD 0, %[xv0], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 1\n RW_XLOAD 1, %[xv0], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 2\n RW_XLOAD 2, %[xv1], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 3\n RW_XLOAD 3, %[xv1], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 4\n RW_XLOAD 4, %[xv2], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 5\n RW_XLOAD 5, %[xv2], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 6\n RW_XLOAD 6, %[xv3], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 7\n RW_XLOAD 7, %[xv3], %[xrs], %[xs]\n .endif\n" \
     "  .if " #J " == 8\n s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n .endif\n" \
     "  .if " #J " == 9\n s_add_u32 m0, %[m0base], 8192\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n .endif\n" \
     "  .if " #J " == 10\n s_add_u32 m0, %[m0base], 16384\n s_nop 0\n buffer_load_dwordx4 %[av2], %[ars], %[asoff] offen lds\n .endif\n" \
     "  .if " #J " == 11\n s_mov_b32 m0, %[m0last]\n s_nop 0\n buffer_load_dwordx4 %[av3], %[ars], %[asoff] offen lds\n .endif\n" \
     " .else\n" \
-    "  .if " #J " == 0\n RW_XLOAD 0, %[xvoff], %[xrs], %[xs0]\n RW_XLOAD 1, %[xvoff], %[xrs], %[xs0]\n .endif\n" \
-    "  .if " #J " == 1\n RW_XLOAD 2, %[xvoff], %[xrs], %[xs1]\n RW_XLOAD 3, %[xvoff], %[xrs], %[xs1]\n .endif\n" \
-    "  .if " #J " == 2\n RW_XLOAD 4, %[xvoff], %[xrs], %[xs2]\n RW_XLOAD 5, %[xvoff], %[xrs], %[xs2]\n .endif\n" \
-    "  .if " #J " == 3\n RW_XLOAD 6, %[xvoff], %[xrs], %[xs3]\n RW_XLOAD 7, %[xvoff], %[xrs], %[xs3]\n .endif\n" \
+    "  .if " #J " == 0\n RW_XLOAD 0, %[xv0], %[xrs], %[xs]\n RW_XLOAD 1, %[xv0], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 1\n RW_XLOAD 2, %[xv1], %[xrs], %[xs]\n RW_XLOAD 3, %[xv1], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 2\n RW_XLOAD 4, %[xv2], %[xrs], %[xs]\n RW_XLOAD 5, %[xv2], %[xrs], %[xs]\n .endif\n" \
+    "  .if " #J " == 3\n RW_XLOAD 6, %[xv3], %[xrs], %[xs]\n RW_XLOAD 7, %[xv3], %[xrs], %[xs]\n .endif\n" \
     "  .if " #J " == 4\n s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n .endif\n" \
     "  .if " #J " == 5\n s_mov_b32 m0, %[m0last]\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n .endif\n" \
     " .endif\n" \
@@ -247,12 +248,12 @@ constexpr int rw_loads_per_chunk(int lck) { return 2 * RW_C + rw_pieces_per_wave
 // The arithmetic of the chunk whose operands sit in own set P and in the value buffer at a_read_addr, and the
 // requests for the chunk two steps ahead (own set (P + 2) % 3) spread between its diagonals.
 template <int LCK, int P, int WPAR>
-__device__ __forceinline__ void rw_compute(unsigned a_read_addr, unsigned x_voff, const unsigned (&a_voff)[4], const RwRequest &rq)
+__device__ __forceinline__ void rw_compute(unsigned a_read_addr, const unsigned (&x_voff)[RW_C], const unsigned (&a_voff)[4], const RwRequest &rq)
 {
     static_assert(LCK == 7 || LCK == 13, "instantiated chunk lengths");
     asm volatile(RW_CHUNK
-                 :: [aread] "v"(a_read_addr), [xvoff] "v"(x_voff), [xrs] "s"(rq.xr), [xs0] "s"(rq.xs[0]), [xs1] "s"(rq.xs[1]),
-                    [xs2] "s"(rq.xs[2]), [xs3] "s"(rq.xs[3]), [ars] "s"(rq.ar), [asoff] "s"(rq.as), [av0] "v"(a_voff[0]),
+                 :: [aread] "v"(a_read_addr), [xv0] "v"(x_voff[0]), [xv1] "v"(x_voff[1]), [xv2] "v"(x_voff[2]), [xv3] "v"(x_voff[3]),
+                    [xrs] "s"(rq.xr), [xs] "s"(rq.xs), [ars] "s"(rq.ar), [asoff] "s"(rq.as), [av0] "v"(a_voff[0]),
                     [av1] "v"(a_voff[1]), [av2] "v"(a_voff[2]), [av3] "v"(a_voff[3]), [m0base] "s"(rq.m0_base),
                     [m0last] "s"(rq.m0_last), [p] "n"(P), [q] "n"((P + 2) % 3), [wpar] "n"(WPAR), [lck] "n"(LCK)
                  : "memory", "scc", RW_CLOB_ALL);
@@ -260,13 +261,13 @@ __device__ __forceinline__ void rw_compute(unsigned a_read_addr, unsigned x_voff
 
 // The same requests all at once (the first two chunks of a tile, before any arithmetic).
 template <int LCK, int Q>
-__device__ __forceinline__ void rw_request_now(unsigned x_voff, const unsigned (&a_voff)[4], const RwRequest &rq)
+__device__ __forceinline__ void rw_request_now(const unsigned (&x_voff)[RW_C], const unsigned (&a_voff)[4], const RwRequest &rq)
 {
     asm volatile(RW_DEFS "RW_SETS %[q], %[q]\n s_nop 4\n"
-                 "RW_XLOAD 0, %[xvoff], %[xrs], %[xs0]\n RW_XLOAD 1, %[xvoff], %[xrs], %[xs0]\n"
-                 "RW_XLOAD 2, %[xvoff], %[xrs], %[xs1]\n RW_XLOAD 3, %[xvoff], %[xrs], %[xs1]\n"
-                 "RW_XLOAD 4, %[xvoff], %[xrs], %[xs2]\n RW_XLOAD 5, %[xvoff], %[xrs], %[xs2]\n"
-                 "RW_XLOAD 6, %[xvoff], %[xrs], %[xs3]\n RW_XLOAD 7, %[xvoff], %[xrs], %[xs3]\n"
+                 "RW_XLOAD 0, %[xv0], %[xrs], %[xs]\n RW_XLOAD 1, %[xv0], %[xrs], %[xs]\n"
+                 "RW_XLOAD 2, %[xv1], %[xrs], %[xs]\n RW_XLOAD 3, %[xv1], %[xrs], %[xs]\n"
+                 "RW_XLOAD 4, %[xv2], %[xrs], %[xs]\n RW_XLOAD 5, %[xv2], %[xrs], %[xs]\n"
+                 "RW_XLOAD 6, %[xv3], %[xrs], %[xs]\n RW_XLOAD 7, %[xv3], %[xrs], %[xs]\n"
                  ".if %[lck] > 8\n"
                  " s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n"
                  " s_add_u32 m0, %[m0base], 8192\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n"
@@ -276,8 +277,8 @@ __device__ __forceinline__ void rw_request_now(unsigned x_voff, const unsigned (
                  " s_mov_b32 m0, %[m0base]\n s_nop 0\n buffer_load_dwordx4 %[av0], %[ars], %[asoff] offen lds\n"
                  " s_mov_b32 m0, %[m0last]\n s_nop 0\n buffer_load_dwordx4 %[av1], %[ars], %[asoff] offen lds\n"
                  ".endif\n" RW_PURGE
-                 :: [xvoff] "v"(x_voff), [xrs] "s"(rq.xr), [xs0] "s"(rq.xs[0]), [xs1] "s"(rq.xs[1]),
-                    [xs2] "s"(rq.xs[2]), [xs3] "s"(rq.xs[3]), [ars] "s"(rq.ar), [asoff] "s"(rq.as), [av0] "v"(a_voff[0]),
+                 :: [xv0] "v"(x_voff[0]), [xv1] "v"(x_voff[1]), [xv2] "v"(x_voff[2]), [xv3] "v"(x_voff[3]),
+                    [xrs] "s"(rq.xr), [xs] "s"(rq.xs), [ars] "s"(rq.ar), [asoff] "s"(rq.as), [av0] "v"(a_voff[0]),
                     [av1] "v"(a_voff[1]), [av2] "v"(a_voff[2]), [av3] "v"(a_voff[3]), [m0base] "s"(rq.m0_base),
                     [m0last] "s"(rq.m0_last), [q] "n"(Q), [lck] "n"(LCK)
                  : "memory", "scc", RW_CLOB_ALL);
@@ -323,8 +324,9 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
 
     // The chunks that have rows inside the operand: the table is sorted by shift, so they are a contiguous
     // range.  A chunk's valid rows read the dense rows [a0, a0 + TR + LCK - 1), a0 = row0 + its shift.
-    // Lane l also keeps what the walk needs of table entry l -- shift and first table position -- so that the
-    // loop reads an entry with v_readlane, not from memory.
+    // Lane l keeps what the walk needs of table entry l, ready-made, so that a step reads the entry of the
+    // chunk it requests with three v_readlane and the two waves of a SIMD spend next to nothing between two
+    // chunks' arithmetic (whatever one of them does there, the other runs alone, at half the rate).
     const Chunk *mine = chunks + min(lane, nchunks - 1);
     const int tab_s0 = mine->s0, tab_slot0 = mine->slot[0];
     int c_lo = nchunks, c_hi = 0;
@@ -342,15 +344,17 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
 
     const float *xcol0 = X + (long long)col0 * ldx;
     const rw_int4 xr_all = rw_rsrc(xcol0, (unsigned)(((long long)(cols_here - 1) * ldx + n_in) * 4));
-    const rw_int4 ar = rw_rsrc(vals, a_bytes);
+    const rw_int4 ar_all = rw_rsrc(vals, a_bytes);
     const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) unsigned char *)&lds[0];
     const unsigned a_read_addr = lds0 + 16u * (unsigned)lane;
-    const unsigned x_voff = 32u * (unsigned)lane;
-    // the wave's columns (one past the batch is replaced by the last valid one: its sums are never stored)
-    unsigned colb[RW_C];
+    // the wave's columns (one past the batch is replaced by the last valid one: its sums are never stored); a
+    // lane's byte offset inside the tile's dense operand is its column's first row + its own 8 rows
+    auto column_bytes = [&](int c) __attribute__((always_inline)) {
+        return (unsigned)min(RW_C * wave + c, cols_here - 1) * ((unsigned)ldx * 4u);
+    };
+    unsigned x_voff[RW_C];
 #pragma unroll
-    for (int c = 0; c < RW_C; ++c)
-        colb[c] = __builtin_amdgcn_readfirstlane((unsigned)min(RW_C * wave + c, cols_here - 1) * ((unsigned)ldx * 4u));
+    for (int c = 0; c < RW_C; ++c) x_voff[c] = column_bytes(c) + 32u * (unsigned)lane;
     // Diagonal values: a chunk's diagonals sit at evenly spaced table positions, slot_step apart (negative for the
     // transposed product of a table listed in ascending order), and for the transposed product a value is
     // indexed by its INPUT row, one further per diagonal.  A lane reaches diagonal j of a chunk through a
@@ -369,51 +373,59 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
                                               : RW_OOB;
     }
     const bool has_last = wave + RW_WAVES * (NP - 1) < PIECES;
+    const unsigned m0_wave = lds0 + 1024u * (unsigned)wave;
 
-    struct Entry { int s0, slot0; };
-    auto entry = [&](int i) __attribute__((always_inline)) {
-        const int at = c_lo + min(i, max(nk - 1, 0));
-        return Entry{__builtin_amdgcn_readlane(tab_s0, at), __builtin_amdgcn_readlane(tab_slot0, at)};
-    };
-    // can chunk e be requested with whole 16-byte pieces: its 512 rows of every column and of every diagonal exist
-    auto whole = [&](const Entry &e) __attribute__((always_inline)) {
-        const int a0 = row0 + e.s0;
-        return (a0 >= 0) & (a0 + RW_LOADED + LCK - 1 <= n_in) & (row0 + RW_LOADED <= n_out);
-    };
-    // the requests of chunk e into own set / value buffer q; real == false: the empty resources
-    auto request = [&](const Entry &e, int q, bool real) __attribute__((always_inline)) {
-        RwRequest rq;
-        // (the empty resource: the same with a size of 0, every lane out of range)
-        rq.xr = rw_int4{xr_all.x, xr_all.y, real ? xr_all.z : 0, xr_all.w};
-        rq.ar = rw_int4{ar.x, ar.y, real ? ar.z : 0, ar.w};
-        const unsigned a0b = (unsigned)(row0 + e.s0) * 4u;
-#pragma unroll
-        for (int c = 0; c < RW_C; ++c) rq.xs[c] = real ? colb[c] + a0b : 0u;
-        const int slot_first = ascending ? e.slot0 : e.slot0 + (LCK - 1) * slot_step;      // the first in memory
-        const int in_first = ashift ? e.s0 + (ascending ? 0 : LCK - 1) : 0;
-        rq.as = real ? ((unsigned)slot_first * (unsigned)stride + (unsigned)(row0 + in_first)) * 4u : 0u;
-        rq.m0_base = lds0 + (unsigned)(q * ABUF) + 1024u * (unsigned)wave;
-        rq.m0_last = has_last ? rq.m0_base + 8192u * (unsigned)(NP - 1) : lds0 + DUMP;
-        return rq;
+    // Table entry l as lane l holds it: can the chunk be requested with whole 16-byte pieces (its 512 rows of
+    // every column and of every diagonal exist), and if so the scalar byte offsets of its first dense row and of
+    // its first diagonal in memory at the tile's first row.
+    int tab_whole;
+    unsigned tab_xs, tab_as;
+    {
+        const int a0 = row0 + tab_s0;
+        const bool w = (a0 >= 0) & (a0 + RW_LOADED + LCK - 1 <= n_in) & (row0 + RW_LOADED <= n_out);
+        const int slot_first = ascending ? tab_slot0 : tab_slot0 + (LCK - 1) * slot_step;
+        const int in_first = ashift ? tab_s0 + (ascending ? 0 : LCK - 1) : 0;
+        tab_whole = w ? 1 : 0;
+        tab_xs = w ? (unsigned)a0 * 4u : 0u;
+        tab_as = w ? ((unsigned)slot_first * (unsigned)stride + (unsigned)(row0 + in_first)) * 4u : 0u;
+    }
+    // The requests of chunk ii of the walk into own set / value buffer q, or -- past the end of the walk, and
+    // for a chunk that cannot be requested whole -- the empty resources (the same with a size of 0: every lane
+    // is out of range, nothing is fetched, zeros arrive) with scalar offsets of 0.
+    struct Next { RwRequest rq; int at; bool checked; };
+    RwRequest rq_cur{xr_all, 0u, ar_all, 0u, 0u, 0u};
+    auto prepare = [&](int ii, int q) __attribute__((always_inline)) {
+        const int at = c_lo + min(ii, max(nk - 1, 0));
+        const bool there = ii < nk;
+        const bool w = __builtin_amdgcn_readlane(tab_whole, at) != 0;
+        const bool real = there && w;
+        rq_cur.xr.z = real ? xr_all.z : 0;
+        rq_cur.ar.z = real ? ar_all.z : 0;
+        rq_cur.xs = real ? (unsigned)__builtin_amdgcn_readlane((int)tab_xs, at) : 0u;
+        rq_cur.as = real ? (unsigned)__builtin_amdgcn_readlane((int)tab_as, at) : 0u;
+        rq_cur.m0_base = m0_wave + (unsigned)(q * ABUF);
+        rq_cur.m0_last = has_last ? rq_cur.m0_base + 8192u * (unsigned)(NP - 1) : lds0 + DUMP;
+        return Next{rq_cur, at, there && !w};
     };
     // a chunk that crosses an end of the operand, element by element: a value whose input row does not exist
     // is padding and becomes 0, as does a dense row outside the operand
-    auto request_checked = [&](const Entry &e, auto q_c) __attribute__((always_inline)) {
+    auto request_checked = [&](int at, auto q_c) __attribute__((always_inline)) {
         constexpr int Q = decltype(q_c)::value;
+        const int s0 = __builtin_amdgcn_readlane(tab_s0, at), slot0 = __builtin_amdgcn_readlane(tab_slot0, at);
         const unsigned abuf = lds0 + (unsigned)(Q * ABUF);
-        const int a0 = row0 + e.s0;
+        const int a0 = row0 + s0;
 #pragma unroll
         for (int it = 0; it < NP; ++it) {
             const int pw = wave + RW_WAVES * it;
             if (pw < PIECES) {
                 const int j = pw >> 1, half = pw & 1;
-                const unsigned dbase = ((unsigned)(e.slot0 + j * slot_step) * (unsigned)stride) * 4u;
+                const unsigned dbase = ((unsigned)(slot0 + j * slot_step) * (unsigned)stride) * 4u;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int o = row0 + 8 * (16 * q + (lane >> 2)) + 4 * half + (lane & 3);
-                    const int in = o + e.s0 + j;
+                    const int in = o + s0 + j;
                     const bool ok = ((unsigned)in < (unsigned)n_in) & (o < n_out);
-                    rw_lds_load_b32(ar, abuf + 1024u * (unsigned)pw + 256u * (unsigned)q,
+                    rw_lds_load_b32(ar_all, abuf + 1024u * (unsigned)pw + 256u * (unsigned)q,
                                     ok ? dbase + (unsigned)(ashift ? in : o) * 4u : RW_OOB);
                 }
             }
@@ -426,10 +438,10 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
         }
         // (the range check of a buffer load counts the scalar offset in: every column gets a resource of its
         // own that ends with the column's last row)
-        rw_load_own_checked<Q, 0>(v, rw_rsrc(xcol0 + colb[0] / 4u, (unsigned)n_in * 4u));
-        rw_load_own_checked<Q, 1>(v, rw_rsrc(xcol0 + colb[1] / 4u, (unsigned)n_in * 4u));
-        rw_load_own_checked<Q, 2>(v, rw_rsrc(xcol0 + colb[2] / 4u, (unsigned)n_in * 4u));
-        rw_load_own_checked<Q, 3>(v, rw_rsrc(xcol0 + colb[3] / 4u, (unsigned)n_in * 4u));
+        rw_load_own_checked<Q, 0>(v, rw_rsrc(xcol0 + column_bytes(0) / 4u, (unsigned)n_in * 4u));
+        rw_load_own_checked<Q, 1>(v, rw_rsrc(xcol0 + column_bytes(1) / 4u, (unsigned)n_in * 4u));
+        rw_load_own_checked<Q, 2>(v, rw_rsrc(xcol0 + column_bytes(2) / 4u, (unsigned)n_in * 4u));
+        rw_load_own_checked<Q, 3>(v, rw_rsrc(xcol0 + column_bytes(3) / 4u, (unsigned)n_in * 4u));
     };
 
     asm volatile(RW_DEFS ".irp i,0,1,2,3,4,5,6,7,8,9,10,11,12,13,14,15,16,17,18,19,20,21,22,23,24,25,26,27,28,29,30,31\n"
@@ -442,27 +454,20 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
     // of loads per chunk whatever happens and the waits count exactly).
     bool exact = false;         // the loads in flight behind those of the chunk about to be computed are the NLOADS of one statement
     if (nk > 0) {
-        const Entry e0 = entry(0);
-        if (whole(e0)) rw_request_now<LCK, 0>(x_voff, a_voff, request(e0, 0, true));
-        else request_checked(e0, std::integral_constant<int, 0>{});
+        const Next n0 = prepare(0, 0);
+        if (!n0.checked) rw_request_now<LCK, 0>(x_voff, a_voff, n0.rq);
+        else request_checked(n0.at, std::integral_constant<int, 0>{});
         if (nk > 1) {
-            const Entry e1 = entry(1);
-            if (whole(e1)) {
-                rw_request_now<LCK, 1>(x_voff, a_voff, request(e1, 1, true));
+            const Next n1 = prepare(1, 1);
+            if (!n1.checked) {
+                rw_request_now<LCK, 1>(x_voff, a_voff, n1.rq);
                 exact = true;
             } else {
-                request_checked(e1, std::integral_constant<int, 1>{});
+                request_checked(n1.at, std::integral_constant<int, 1>{});
             }
         }
     }
-    // what the statement of a step requests (chunk i + 2), prepared one step ahead -- behind the arithmetic of
-    // the step before, where the waves wait for each other anyway
-    struct Next { RwRequest rq; Entry e; bool checked; };
-    auto prepare = [&](int ii, int q) __attribute__((always_inline)) {
-        const Entry e = entry(ii);
-        const bool there = ii < nk, w = whole(e);
-        return Next{request(e, q, there && w), e, there && !w};
-    };
+    // what the statement of a step requests (chunk i + 2) is prepared one step ahead
     Next nx = prepare(2, 2);
     auto step = [&](int i, auto p_c) __attribute__((always_inline)) {
         constexpr int P = decltype(p_c)::value, Q = (P + 2) % 3;
@@ -474,7 +479,7 @@ __global__ __launch_bounds__(64 * RW_WAVES) void spmm_rows_kernel(
         else rw_compute<LCK, P, 1>(aread, x_voff, a_voff, nx.rq);
         exact = true;
         if (nx.checked) {
-            request_checked(nx.e, std::integral_constant<int, Q>{});
+            request_checked(nx.at, std::integral_constant<int, Q>{});
             exact = false;
         }
         nx = prepare(i + 3, P);

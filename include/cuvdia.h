@@ -155,15 +155,11 @@ long long cuvdia_plan_walk_launch(const int *offsets_host, int nd, int stride, i
  * beta == 0 follows the reference HOST rule (spmv.cu:152-156): dst is
  * overwritten and never read, so it may hold NaN.  batch == 0 is a no-op.
  * B and dst must not overlap.
- * Non-finite values in B: the generic kernels, like the reference's host
- * loop, multiply exactly the stored elements.  The tiled kernels process
- * every chunk of the run table as if it had the table's longest length,
- * with zeros for the missing diagonals; when a table mixes chunk lengths
- * (e.g. offsets -3..3 together with 100, 101) a shorter chunk therefore
- * multiplies a few rows of B next to its own by zero, and an Inf or NaN in
- * such a row turns into NaN in result rows that do not reference it.  Tables
- * whose chunks all have one length (any 2-d window pattern) are not
- * affected. */
+ * Non-finite values in B: every kernel family multiplies exactly the stored
+ * elements, as the reference's host loop does (spmv.cu:183-197): an Inf or
+ * NaN in a row of B reaches the result rows that reference that row and no
+ * other (chunks shorter than the table's longest run only the diagonals
+ * they have). */
 int cuvdia_spmm_f32(const cuvdia_desc *desc, const float *A_vals_device,
                     const float *B_device, long long ldb,
                     float *dst_device, long long ldd, int batch,

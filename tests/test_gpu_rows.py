@@ -55,3 +55,28 @@ def test_rows_matches_the_oracle(oracle, gu, h, w, px, fs, channels, batch, tran
     assert ran == _lib.PATH_ROWS
     _, ran = gu.check_prod(oracle, A, B, dst, trans, 0.75, -1.5, _lib.PATH_ROWS, "rows scaled")
     assert ran == _lib.PATH_ROWS
+
+
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_rows_non_finite_values_reach_only_the_rows_that_use_them(oracle, gu, trans):
+    """Inf and NaN in B, in the interior and in the first and last rows of the operand (the chunks there are
+    fetched element by element, with zeros where a row does not exist): the masks of NaN and +-Inf equal the
+    oracle's."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(82)
+    h = w = 5000
+    A = _window_dia(oracle, rng, h, w, 50, 7)
+    B, _ = _operands(rng, A, 33, trans)
+    B[2000, 3] = np.inf
+    B[1, 20] = np.nan
+    B[h - 2, 5] = -np.inf
+    B[777, 32] = np.nan
+    with np.errstate(invalid="ignore"):
+        ref = oracle.prod(A, B, None, trans)
+    got, ran = gu.gpu_prod(A, B, None, trans, 1.0, 0.0, _lib.PATH_ROWS)
+    assert ran == _lib.PATH_ROWS
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    assert np.array_equal(np.isposinf(got), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(got), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    np.testing.assert_allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-5)

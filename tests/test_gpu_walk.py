@@ -207,3 +207,29 @@ def test_walk_on_random_window_shapes(oracle, gu, seed):
         print(what, flush=True)
         _, ran = gu.check_prod(oracle, A, B, None if beta == 0.0 else dst, trans, alpha, beta, _lib.PATH_WALK, what)
         assert ran == _lib.PATH_WALK
+
+
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_walk_non_finite_values_reach_only_the_rows_that_use_them(oracle, gu, trans):
+    """Inf and NaN in B, in the interior and in the first and last rows of the operand: the walking kernel stages
+    zeros for rows outside the operand and for diagonal slots outside the matrix, and no such zero may meet a
+    non-finite dense value that the oracle's loop over stored elements does not touch."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(81)
+    px, fs, batch = 64, 7, 70
+    n = px * px
+    A = _window_dia(oracle, rng, n, n, px, fs)
+    B, _ = _operands(rng, A, batch, trans)
+    B[2000, 3] = np.inf
+    B[1, 40] = np.nan
+    B[n - 2, 5] = -np.inf
+    B[777, 69] = np.nan
+    with np.errstate(invalid="ignore"):
+        ref = oracle.prod(A, B, None, trans)
+    got, ran = gu.gpu_prod(A, B, None, trans, 1.0, 0.0, _lib.PATH_WALK)
+    assert ran == _lib.PATH_WALK
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    assert np.array_equal(np.isposinf(got), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(got), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    np.testing.assert_allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-5)
