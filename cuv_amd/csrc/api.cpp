@@ -42,8 +42,6 @@ thread_local std::string t_hip_error;
 // one batch column on each of 64 lanes.
 constexpr int SPMM_TILED_MIN_BATCH = 24;
 // The rows-along-lanes kernel is the automatic choice from this many of its tiles (workgroups) and this batch.
-constexpr long long SPMM_ROWS_MIN_TILES = 1LL << 40;     // (not chosen automatically until measured)
-constexpr int SPMM_ROWS_MIN_BATCH = 32;
 // Largest h, w and |offset| the kernels' 32-bit row arithmetic allows.
 constexpr long long DIM_LIMIT = 1LL << 30;
 
@@ -135,7 +133,7 @@ const char *cuvdia_last_hip_error(void) { return t_hip_error.c_str(); }
 int cuvdia_set_path(int path)
 {
     if (path != CUVDIA_PATH_AUTO && path != CUVDIA_PATH_GENERIC && path != CUVDIA_PATH_TILED &&
-        path != CUVDIA_PATH_TILED_NOWALK && path != CUVDIA_PATH_WALK && path != CUVDIA_PATH_ROWS)
+        path != CUVDIA_PATH_TILED_NOWALK && path != CUVDIA_PATH_WALK)
         return CUVDIA_EINVAL;
     g_path.store(path);
     return CUVDIA_OK;
@@ -399,25 +397,6 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const fl
 
     const int forced = g_path.load();
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // The rows-along-lanes kernel: plain products of tables it serves (spmm_rows_ok).  Chosen when asked for,
-    // and by itself for products large enough to fill the chip with its tiles several times over.
-    {
-        const bool plain = bias == nullptr && act == CUVDIA_ACT_NONE;
-        const bool rows_possible = plain && spmm_rows_ok(desc->view, ldb, ldd, trans);
-        if (forced == CUVDIA_PATH_ROWS && !rows_possible) return CUVDIA_EUNSUPPORTED;
-        bool rows = forced == CUVDIA_PATH_ROWS;
-        if (forced == CUVDIA_PATH_AUTO && rows_possible) {
-            const int lck = trans ? desc->view.max_len_t : desc->view.max_len_n;
-            const long long tiles = ((long long)n_out + spmm_rows_tile_rows(lck) - 1) / spmm_rows_tile_rows(lck) *
-                                    (((long long)batch + 31) / 32);
-            rows = tiles >= SPMM_ROWS_MIN_TILES && batch >= SPMM_ROWS_MIN_BATCH;
-        }
-        if (rows) {
-            const hipError_t e = launch_spmm_rows(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, s);
-            t_last_path = CUVDIA_PATH_ROWS;
-            return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "spmm kernel launch");
-        }
-    }
     const bool tiled_possible = spmm_tiled_ok(desc->view, ldb, ldd, trans);
     bool tiled;
     if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
@@ -509,8 +488,7 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
         }
     }
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK ||
-        forced == CUVDIA_PATH_ROWS) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {
@@ -678,7 +656,7 @@ int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals, const int *offsets_host
 
     // the kernel family is chosen by the rule of cuvdia_spmm_layer_f32
     const int forced = g_path.load();
-    if (forced == CUVDIA_PATH_WALK || forced == CUVDIA_PATH_ROWS) return CUVDIA_EUNSUPPORTED;
+    if (forced == CUVDIA_PATH_WALK) return CUVDIA_EUNSUPPORTED;
     const bool tiled_possible = spmm_tiled_ok(view, ldb, ldd, trans);
     bool tiled;
     if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK) {

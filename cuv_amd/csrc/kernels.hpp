@@ -79,18 +79,6 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
                              float alpha, float beta, SpEpilogue ep, hipStream_t stream,
                              int walk = 0, bool *walked = nullptr);
 
-// The product for large operands with the ROWS along the lanes (spmm_rows.hip): a lane owns 8 rows x 4 batch
-// columns of sums, the diagonal values are its own, and every FMA runs on three plain vector registers in
-// different register banks -- twice the issue rate of the broadcast form the tiled kernels use.  Serves tables
-// whose chunks all have 7 or 13 diagonals at evenly spaced ascending table positions (2-d window patterns),
-// row_fact 1, no fused epilogue.  spmm_rows_ok: can it serve these operands; spmm_rows_tile_rows: output rows
-// per workgroup for a chunk length.
-bool spmm_rows_ok(const DiaView &A, long long ldb, long long ldd, bool trans);
-int spmm_rows_tile_rows(int lck);
-hipError_t launch_spmm_rows(const DiaView &A, const float *vals, const float *B, long long ldb,
-                            float *dst, long long ldd, int batch, bool trans,
-                            float alpha, float beta, hipStream_t stream);
-
 // m = mw*M[i] - lr*(dW[i] + l2*W[i]); W[i] += m; M[i] = m, i < n.
 hipError_t launch_momentum(float *W, float *M, const float *dW, long long n, float lr, float mw, float l2,
                            hipStream_t stream);

@@ -52,7 +52,6 @@ extern "C" {
 #define CUVDIA_PATH_TILED    2  /* LDS-staged, register-blocked kernels (rf == 1) */
 #define CUVDIA_PATH_WALK     3  /* of the tiled family: the walking kernel for window tables (products only) */
 #define CUVDIA_PATH_TILED_NOWALK 4  /* the tiled family without its walking kernel (products only)         */
-#define CUVDIA_PATH_ROWS     5  /* the rows-along-lanes kernel for large products of window tables (products only) */
 
 /* Activation applied by cuvdia_spmm_bias_act_f32. */
 #define CUVDIA_ACT_NONE      0
