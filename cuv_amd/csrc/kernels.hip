@@ -1499,8 +1499,8 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
 
     // dense rows: instruction i = wave + WAVES it of a block stages pieces 64 i .. 64 i + 63, piece p = XQ * column + quad
     constexpr int XIT = (XQ + WAVES - 1) / WAVES;
-    // A lane's share of the requests is recomputed from its lane number for every block (a few integer
-    // operations) rather than kept in registers across the walk: the running sums need them.
+    // A lane's share of the requests at the operand's ends is recomputed from its lane number for every block (a
+    // few integer operations) rather than kept in registers across the walk: the running sums need them.
     auto lane_now = [&]() __attribute__((always_inline)) {
         int l = lane;
         asm volatile("" : "+v"(l));
@@ -1519,6 +1519,27 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
     // piece / XQ == (piece * XQ_RECIP) >> 16 (checked below), a 24-bit multiplication at full rate
     constexpr unsigned XQ_RECIP = (65536u + XQ - 1) / XQ;
     static_assert(64 * XIT * WAVES <= 2048 && recip16_exact(XQ, XQ_RECIP, 2048), "piece / XQ by multiplication");
+    // What a lane adds to the byte offset of a block that lies wholly inside the operand -- all but the few at
+    // its ends -- is the same for the whole walk: its piece's column and place in the column for the dense rows,
+    // its diagonal and rows for the values.  Kept in registers (5), a request of such a block costs one vector
+    // addition instead of a dozen operations; the offsets stay vector offsets, so the buffer's range check
+    // still answers anything out of range with zeros.
+    constexpr int AIT = (K * S::AI + WAVES - 1) / WAVES;
+    unsigned x_lane[XIT], a_lane[AIT];
+#pragma unroll
+    for (int it = 0; it < XIT; ++it) {
+        const int piece = 64 * (wave + WAVES * it) + lane;
+        const int col = (int)(__umul24((unsigned)piece, XQ_RECIP) >> 16);
+        x_lane[it] = wave + WAVES * it < XQ
+                         ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) + 16u * (unsigned)(piece - col * XQ)
+                         : OOB_OFFSET;
+    }
+#pragma unroll
+    for (int k = 0; k < AIT; ++k) {
+        const int n = wave + WAVES * k, h = n % S::AI;
+        const int j = h * S::DPI + lane / (ROWS / 4);
+        a_lane[k] = (n < K * S::AI && j < LCK) ? (unsigned)(16 * (lane % (ROWS / 4)) + j * astep4) : OOB_OFFSET;
+    }
     // Requests block number i = u * ngroups + g (step u, group g) into buffer i & 1: its dense
     // rows and, for every tile m = u - dy that exists, the values of chunk (g, dy) for the tile's rows.
     auto issue = [&](int i, int u, int g) __attribute__((always_inline)) {
@@ -1526,16 +1547,24 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         if (a0 + ROWS + LCK - 1 <= 0 || a0 >= n_in) return;          // wholly outside: nothing to stage (see apply)
         const unsigned buf = lds0 + (unsigned)(i & 1) * BUF_BYTES;
         const int a0p = a0 - SH;                                     // a multiple of 4
-        const int ln = lane_now();
+        if ((a0p >= 0) & (a0p + 4 * XQ <= n_in)) {
+            // every staged piece exists
 #pragma unroll
-        for (int it = 0; it < XIT; ++it) {
-            if (wave + WAVES * it < XQ) {
-                const int piece = 64 * (wave + WAVES * it) + ln;
-                const int col = (int)(__umul24((unsigned)piece, XQ_RECIP) >> 16);
-                const int r = a0p + 4 * (piece - col * XQ);
-                const unsigned x_col = (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u);
-                const bool ok = (r >= 0) & (r + 4 <= n_in);
-                lds_load_b128(xq, buf + 1024u * (unsigned)(wave + WAVES * it), ok ? x_col + (unsigned)(r * 4) : OOB_OFFSET, 0u);
+            for (int it = 0; it < XIT; ++it)
+                if (wave + WAVES * it < XQ)
+                    lds_load_b128(xq, buf + 1024u * (unsigned)(wave + WAVES * it), x_lane[it] + (unsigned)(a0p * 4), 0u);
+        } else {
+            const int ln = lane_now();
+#pragma unroll
+            for (int it = 0; it < XIT; ++it) {
+                if (wave + WAVES * it < XQ) {
+                    const int piece = 64 * (wave + WAVES * it) + ln;
+                    const int col = (int)(__umul24((unsigned)piece, XQ_RECIP) >> 16);
+                    const int r = a0p + 4 * (piece - col * XQ);
+                    const unsigned x_col = (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u);
+                    const bool ok = (r >= 0) & (r + 4 <= n_in);
+                    lds_load_b128(xq, buf + 1024u * (unsigned)(wave + WAVES * it), ok ? x_col + (unsigned)(r * 4) : OOB_OFFSET, 0u);
+                }
             }
         }
         const bool inside = (a0 >= 0) & (a0 + ROWS + LCK - 1 <= n_in);
@@ -1543,16 +1572,18 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         if (inside) {
             // 16-byte pieces: instruction n = dy * AI + h carries diagonals h*DPI .. of tile u - dy's chunk,
             // lane = (ROWS/4) * diagonal + piece
-            for (int n = wave; n < K * AI; n += WAVES) {
-                const int dy = n / AI, h = n - dy * AI;
+#pragma unroll
+            for (int k = 0; k < AIT; ++k) {
+                const int n = wave + WAVES * k;
+                if (n >= K * AI) break;
+                const int dy = n / AI;
                 const int m = u - dy;
                 if (m < 0 || m >= ntiles) continue;
-                const int j = h * S::DPI + ln / (ROWS / 4), piece = ln % (ROWS / 4);
-                const int row = row_first + m * period + 4 * piece;
-                const unsigned off = (unsigned)(stab[ngroups + g * K + dy] + row * 4 + j * astep4);
-                lds_load_b128(aq, abuf + (unsigned)(n * 1024), j < LCK ? off : OOB_OFFSET, 0u);
+                const unsigned base = (unsigned)(stab[ngroups + g * K + dy] + (row_first + m * period) * 4);   // wave-uniform
+                lds_load_b128(aq, abuf + (unsigned)(n * 1024), a_lane[k] + base, 0u);
             }
         } else {
+            const int ln = lane_now();
             // the block crosses an end of the operand: 4-byte loads, each lane testing its own element.
             // Instruction n = dy * NI + h carries EPI diagonals x ROWS rows, lane = ROWS * diagonal + row.
             constexpr int EPI = 64 / ROWS;                           // diagonals per instruction (1 or 2)
