@@ -89,6 +89,8 @@ def parse():
                          "so that a profiler's per-kernel averages describe the same launches as the headline figures")
     ap.add_argument("--settle-ms", type=float, default=200.0,
                     help="untimed replays of a leg's own launches before it is timed, in ms of GPU time")
+    ap.add_argument("--no-clocks", action="store_true",
+                    help="do not start rocm-smi to read the clocks (for runs under a profiler)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
     return ap.parse_args()
@@ -761,7 +763,8 @@ def main():
     else:
         keep = sets[0]
     # last of the GPU work (a query of the management interface is followed by slower launches for a while)
-    out["clocks"] = read_clocks(torch, lambda: [(up(keep), down(keep), grad(keep)) for _ in range(30)], args.no_graph)
+    if not args.no_clocks:
+        out["clocks"] = read_clocks(torch, lambda: [(up(keep), down(keep), grad(keep)) for _ in range(30)], args.no_graph)
 
     if not args.no_cpu:
         from oracle import oracle as O
