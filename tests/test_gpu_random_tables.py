@@ -75,3 +75,39 @@ def test_random_table(oracle, gu, seed):
     for path in (_lib.PATH_AUTO, _lib.PATH_GENERIC):
         C = oracle.Dia(h, w, offs, A.stride, 1, A.vals.copy() if beta != 0.0 else np.full_like(A.vals, np.nan))
         gu.check_dd2dia(oracle, C, P, Q, alpha / batch, beta, path, "%s, projection, path %d" % (what, path))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_table_non_finite(oracle, gu, seed):
+    """The same tables with a handful of Inf and NaN scattered over the dense operand: the masks of NaN, +Inf and
+    -Inf in both products equal the oracle's (whose loop multiplies exactly the stored elements) on the automatic
+    path and on the generic kernels, and the finite results agree as in the test above."""
+    from cuv_amd import _lib
+    rng, h, w, offs, batch, alpha, beta = _draw(seed)
+    if abs(alpha) < 1e-3:
+        alpha = 1.0
+    what = "seed %d: %dx%d, %d diagonals, batch %d" % (seed, h, w, len(offs), batch)
+    print(what, flush=True)
+    A = oracle.Dia(h, w, offs, None, 1)
+    A.vals[:] = np.nan
+    m = oracle.valid_mask(A)
+    A.vals[m] = rng.uniform(-1, 1, int(m.sum())).astype(np.float32)
+    for trans in ("n", "t"):
+        n_in, n_out = (h, w) if trans == "t" else (w, h)
+        B = np.asfortranarray(rng.uniform(-1, 1, (n_in, batch)).astype(np.float32))
+        for _ in range(6):
+            B[int(rng.integers(0, n_in)), int(rng.integers(0, batch))] = rng.choice([np.inf, -np.inf, np.nan])
+        B[0, 0], B[n_in - 1, batch - 1] = np.inf, np.nan          # the operand's corners
+        dst = None if beta == 0.0 else np.asfortranarray(rng.uniform(-1, 1, (n_out, batch)).astype(np.float32))
+        with np.errstate(invalid="ignore"):
+            ref = oracle.prod(A, B, dst, trans, alpha, beta)
+        fin = np.isfinite(ref)
+        with np.errstate(invalid="ignore"):
+            mag = oracle.prod_mag(A, B, dst, trans, alpha, beta)
+        for path in (_lib.PATH_AUTO, _lib.PATH_GENERIC):
+            got, _ = gu.gpu_prod(A, B, dst, trans, alpha, beta, path)
+            tag = "%s, '%s', path %d" % (what, trans, path)
+            assert np.array_equal(np.isnan(got), np.isnan(ref)), tag
+            assert np.array_equal(np.isposinf(got), np.isposinf(ref)), tag
+            assert np.array_equal(np.isneginf(got), np.isneginf(ref)), tag
+            gu.assert_close_mag(got[fin], ref[fin], mag[fin], tag)
