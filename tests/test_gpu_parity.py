@@ -304,6 +304,46 @@ def test_non_finite_values_with_chunks_of_mixed_length(oracle, gu, offs, trans):
             np.testing.assert_allclose(got[fin], ref[fin], rtol=1e-4, atol=1e-5, err_msg=what)
 
 
+@pytest.mark.parametrize("offs", [[dy * 32 + dx for dy in range(-2, 3) for dx in range(-2, 3)],
+                                  list(range(-3, 4)) + [100, 101],
+                                  [dy * 512 + dx for dy in range(-1, 2) for dx in range(-3, 4)]],
+                         ids=["5x5 window", "7+2", "rows 512 apart"])
+def test_projection_non_finite_values_reach_only_the_slots_that_use_them(oracle, gu, offs):
+    """Inf and NaN in either dense operand of densedense_to_dia: a stored element (i, j) sums A[i, b] * B[j, b]
+    over the batch, so a non-finite A[i0, b0] reaches the stored slots of row i0 and a non-finite B[j0, b0] those
+    of column j0 -- and nothing else, although the tiled kernel also forms products for positions that hold no
+    matrix element (chunk positions past a short chunk's length, band rows outside B) and drops them.  Masks of
+    NaN and +-Inf over the valid slots equal the oracle's on both kernel families; padding slots keep their bits."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(len(offs) + 7)
+    h = w = 2048
+    batch = 72
+    C = _rand_dia(oracle, rng, h, w, offs)
+    P = np.asfortranarray(rng.uniform(-1, 1, (h, batch)).astype(np.float32))
+    Q = np.asfortranarray(rng.uniform(-1, 1, (w, batch)).astype(np.float32))
+    P[700, 5] = np.inf
+    P[3, 70] = np.nan
+    Q[1200, 9] = -np.inf
+    Q[w - 2, 0] = np.nan
+    Q[0, 33] = np.inf
+    valid = oracle.valid_mask(C)
+    for alpha, beta in ((1.0 / batch, 0.0), (0.5, 0.9)):
+        with np.errstate(invalid="ignore"):
+            ref = oracle.dd2dia(C, P, Q, alpha, beta)
+        assert 0 < (~np.isfinite(ref[valid])).sum() < 6 * len(offs)
+        for path in _paths(1):
+            got, ran = gu.gpu_dd2dia(C, P, Q, alpha, beta, path)
+            assert ran == path
+            what = "path %d, beta %g" % (path, beta)
+            assert np.array_equal(got[~valid].view(np.uint32), C.vals[~valid].view(np.uint32)), what
+            g, r = got[valid], ref[valid]
+            assert np.array_equal(np.isnan(g), np.isnan(r)), what
+            assert np.array_equal(np.isposinf(g), np.isposinf(r)), what
+            assert np.array_equal(np.isneginf(g), np.isneginf(r)), what
+            fin = np.isfinite(r)
+            np.testing.assert_allclose(g[fin], r[fin], rtol=1e-4, atol=1e-5, err_msg=what)
+
+
 def test_batch_zero_and_errors(oracle, gu):
     import ctypes
     import torch
