@@ -649,6 +649,10 @@ def test_avg_diagonals_errors(oracle, gu):
     (32, 16, [-3, -2, -1, 0, 1, 2, 3], 6),
     (700, 650, [d * 25 + e for d in range(-2, 3) for e in range(-2, 3)], 96),
     (1024, 1024, [dy * 32 + dx for dy in range(-3, 4) for dx in range(-3, 4)], 128),
+    # chunks of different lengths (the kernel variant that skips the diagonals a short chunk does not have)
+    (900, 900, list(range(-8, -1)) + list(range(0, 8)) + [100, 101] + [300], 70),
+    # more than 64 chunks of mixed lengths (the chunk table in four register sets)
+    (1500, 1500, [o for k in range(70) for o in ((9 * k - 300,) if k % 3 else (9 * k - 300, 9 * k - 299))], 40),
 ])
 def test_prod_bias_sigmoid(oracle, gu, h, w, offs, batch, trans):
     """dst = sigmoid(beta*dst + alpha*op(A)*B + bias) in one launch against the
