@@ -598,17 +598,17 @@ __device__ __forceinline__ void spmm_rows_range_upto(float (&acc)[T], const SpWi
         spmm_rows_range_upto<LCK, T, J + 1, J1>(acc, win, len);
     }
 }
-// diagonals J .. J1 - 1 of a chunk of `len` diagonals: the straight-line block for a full chunk, the guarded
-// one otherwise.  MIXED = false: the kernel for tables all of whose chunks have LCK diagonals (every window table),
-// which carries neither the test nor the second block.
+// diagonals J .. J1 - 1 of a chunk of `len` diagonals.  MIXED = false: the kernel for tables all of whose chunks
+// have LCK diagonals (every window table): the straight-line block, no test.  MIXED = true: the guarded block for
+// every chunk, full ones included (a second, straight-line copy for those made the variants for LCK >= 10 spill
+// up to 60 registers; the tests are 2 scalar instructions per diagonal).
 template <int LCK, int T, int J, int J1, bool MIXED>
 __device__ __forceinline__ void spmm_rows_chunk(float (&acc)[T], const SpWindow<LCK, T> &win, int len)
 {
     if constexpr (LCK == 1 || !MIXED) {
         spmm_rows_range<LCK, T, J, J1>(acc, win);
     } else {
-        if (len == LCK) spmm_rows_range<LCK, T, J, J1>(acc, win);
-        else spmm_rows_range_upto<LCK, T, J, J1>(acc, win, len);
+        spmm_rows_range_upto<LCK, T, J, J1>(acc, win, len);
     }
 }
 
