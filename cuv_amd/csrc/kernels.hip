@@ -1530,7 +1530,8 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
     for (int it = 0; it < XIT; ++it) {
         const int piece = 64 * (wave + WAVES * it) + lane;
         const int col = (int)(__umul24((unsigned)piece, XQ_RECIP) >> 16);
-        x_lane[it] = wave + WAVES * it < XQ
+        // (a column's last piece exists only to keep the pitch odd: where no window reaches it, it is not fetched)
+        x_lane[it] = ((wave + WAVES * it < XQ) & (4 * (piece - col * XQ) < S::XNEED))
                          ? (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u) + 16u * (unsigned)(piece - col * XQ)
                          : OOB_OFFSET;
     }
@@ -1562,7 +1563,7 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
                     const int col = (int)(__umul24((unsigned)piece, XQ_RECIP) >> 16);
                     const int r = a0p + 4 * (piece - col * XQ);
                     const unsigned x_col = (unsigned)min(col, cols_here - 1) * ((unsigned)ldx * 4u);
-                    const bool ok = (r >= 0) & (r + 4 <= n_in);
+                    const bool ok = (r >= 0) & (r + 4 <= n_in) & (4 * (piece - col * XQ) < S::XNEED);
                     lds_load_b128(xq, buf + 1024u * (unsigned)(wave + WAVES * it), ok ? x_col + (unsigned)(r * 4) : OOB_OFFSET, 0u);
                 }
             }
