@@ -327,8 +327,10 @@ int cuvdia_desc_create(cuvdia_desc **out, const int *offsets_host, int nd,
     d->view.pair_delta_max = pair_delta_max(cp, un);
     d->view.single_units_dev = reinterpret_cast<const Unit *>(base + us_at);
     auto walk_view = [&](const WalkPlan &p, size_t at) {
-        return p.ok ? WalkView{reinterpret_cast<const int *>(base + at), p.ngroups, p.period, p.s0, p.k, p.lck, p.astep4}
-                    : WalkView{nullptr, 0, 0, 0, 0, 0, 0};
+        bool rows4 = true;
+        for (int r : p.group_rows) rows4 = rows4 && r % 4 == 0;
+        return p.ok ? WalkView{reinterpret_cast<const int *>(base + at), p.ngroups, p.period, p.s0, p.k, p.lck, p.astep4, rows4}
+                    : WalkView{nullptr, 0, 0, 0, 0, 0, 0, false};
     };
     d->view.walk_n = walk_view(wn, wn_at);
     d->view.walk_t = walk_view(wt, wt_at);
@@ -498,14 +500,23 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipSuccess;
+    bool windowed = false;
     if (!tiled) {
         e = launch_dd2dia_generic(desc->view, C_vals, A, lda, B, ldb, batch, alpha, beta, s);
     } else {
-        for (int c0 = 0; c0 < batch && e == hipSuccess; c0 += slab)
+        const int window = forced == CUVDIA_PATH_WALK ? 1 : forced == CUVDIA_PATH_TILED_NOWALK ? -1 : 0;
+        for (int c0 = 0; c0 < batch && e == hipSuccess; c0 += slab) {
+            bool this_one = false;
             e = launch_dd2dia_tiled(desc->view, C_vals, A + (long long)c0 * lda, lda, B + (long long)c0 * ldb, ldb,
-                                    std::min(slab, batch - c0), alpha, c0 == 0 ? beta : 1.f, s);
+                                    std::min(slab, batch - c0), alpha, c0 == 0 ? beta : 1.f, s, window, &this_one);
+            windowed = windowed || this_one;
+        }
+        if (window > 0 && e == hipErrorNotSupported) {
+            (void)hipGetLastError();
+            return CUVDIA_EUNSUPPORTED;
+        }
     }
-    t_last_path = tiled ? CUVDIA_PATH_TILED : CUVDIA_PATH_GENERIC;
+    t_last_path = !tiled ? CUVDIA_PATH_GENERIC : windowed ? CUVDIA_PATH_WALK : CUVDIA_PATH_TILED;
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "dd2dia kernel launch");
 }
 

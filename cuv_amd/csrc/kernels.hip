@@ -21,8 +21,8 @@
 //           each acc = fma(a, b, acc); total = ((p0 + p1) + p2) + p3.
 //           A chunk pair: eight sums s_q over g = q (mod 8);
 //           p_q = s_q + s_{q+4}, then total as above.
-//           C = beta*C + alpha*total.  The generic kernel sums the batch
-//           serially in ascending column order.
+//           C = beta*C + alpha*total.  The generic kernel and the window-table
+//           kernel sum the batch serially in ascending column order.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -31,9 +31,10 @@
 
 #include "kernels.hpp"
 
-// This file is compiled five times (CUVDIA_PART = 1 .. 5, see the Makefile), each translation unit
+// This file is compiled six times (CUVDIA_PART = 1 .. 6, see the Makefile), each translation unit
 // instantiating one share of the kernel templates, so that the shares compile in parallel: parts 1 - 3 hold
-// the tiled SpMM kernels by longest chunk (1 - 5, 6 - 9, 10 - 13), part 5 the walking SpMM kernels, part 4
+// the tiled SpMM kernels by longest chunk (1 - 5, 6 - 9, 10 - 13), part 5 the walking SpMM kernels, part 6
+// the window-table projection, part 4
 // everything else.  Without the macro one unit holds everything.
 #ifndef CUVDIA_PART
 #define CUVDIA_PART 0
@@ -2174,6 +2175,7 @@ __device__ __forceinline__ void dd2dia_unit(
 
 // Shape of the blocks the projection's tiles are numbered in (see the kernel): units per block and row tiles per
 // block, 64 positions or nearly.
+constexpr int DW_MIN_WGS = 768;               // below this the window-table projection leaves CUs short of work
 constexpr int DD_BLOCKED_MIN_TILES = 1024;   // launches of more than a few rounds number their tiles in blocks
 struct DdBlock {
     __host__ __device__ static int units(int nunits) { return nunits < 16 ? nunits : 16; }
@@ -2240,6 +2242,246 @@ __global__ __launch_bounds__((PAIRS && WIDE != DD_SHIFTED) ? 512 : 256) void dd2
     if (row0 >= h) return;
     dd2dia_unit<LC, 1, AVEC, DD_NARROW, !PAIRS || WIDE == DD_SHIFTED>(lds, row0, chunks + c1, chunks + c1, C, stride, A, lda, B, ldb, h, w, batch,
                              alpha, beta, a_bytes, b_bytes, c_bytes);
+}
+
+// ------------------------------------------------------- window-table dd2dia --
+//
+// The projection for *window* tables (plan_walk: k window rows `period` rows apart, every chunk LC <= 8 shifts,
+// repeated for every group), tiled in the plane the window lives in.  Row i of A is position (y, x) =
+// (i / period, i mod period); slot (dy, j) of group g pairs it with row i + s0 + group_rows[g] + dy * period + j of
+// B.  A workgroup owns a tile of 4 x 64 positions -- wave = one y, 64 consecutive x -- for up to 8 window rows
+// (DYB; a taller window is served by several workgroups per tile) and walks the batch in groups of 4 columns.
+// Per group it stages, with loads that write LDS directly,
+//   * its 4 x 64 values of A per column (16 pieces of 16 bytes per y), and
+//   * the 4 + rows - 1 stretches of B that its window rows reach, 64 + SH + LC - 1 values each (BPR pieces),
+// each value ONCE for all the slots that use it: (256 + 10 * 72) * 4 B per column for 49 * 256 FMAs of a 7 x 7
+// window, a third of what 256 rows cost the chunk-by-chunk kernel above (3 KB per 14 * 248 FMAs).  The stretches
+// start at the multiple of 4 at or below their first row (SH = s0 mod 4, the same for every group: a template
+// parameter, so a lane's window keeps static register indices); with row counts that are multiples of 4 every
+// 16-byte piece lies wholly inside its column or outside, and the pieces outside are requested out of range and
+// arrive as zeros.
+// Lane = (role r = lane / 16, xg = lane mod 16): positions x = 64 tx + 4 xg .. + 3 of the wave's y, window rows
+// dy = 2r and 2r + 1 of the workgroup's eight: 2 x 4 x LC running sums, one 16-byte read of A and two windows
+// of B (4 + LC - 1 values each, WQ 16-byte reads) per column.  Two LDS buffers: while group i is applied, group
+// i + 1 lands; one wait and one barrier per group.  A lane's share of a group's requests is the same for the
+// whole walk up to the column step, so its byte offsets are computed once; everything, column included, goes
+// into the vector offset, which the buffer's range check covers.
+//
+// Accumulation order per slot: batch columns ascending, acc = fma(a, b, acc); C = beta*C + alpha*acc.
+template <int LC, int SH>
+struct DwShape {
+    static constexpr int WAVES = 4, TX = 64, COLS = 4, DYB = 8;
+    static constexpr int WIN = SH + 4 + LC - 1;                  // values of a lane's window, from its first piece
+    static constexpr int WQ = (WIN + 3) / 4;                     // .. as 16-byte reads
+    static constexpr int BPR = TX / 4 + WQ - 1;                  // pieces per staged stretch of B
+    static constexpr int NBR_MAX = WAVES - 1 + DYB;              // stretches per column
+    static constexpr int B_PIECES = (COLS * NBR_MAX * BPR + 63) / 64 * 64;
+    static constexpr int A_PIECES = COLS * WAVES * (TX / 4);
+    static constexpr int BUF_PIECES = B_PIECES + A_PIECES;
+    static constexpr int NI_MAX = BUF_PIECES / 64;               // load instructions per group
+    static constexpr int NIT = (NI_MAX + WAVES - 1) / WAVES;     // .. per wave
+    static_assert(A_PIECES % 64 == 0 && LC >= 1 && LC <= CHUNK_MAX && SH >= 0 && SH < 4, "shape");
+    static_assert(2 * BUF_PIECES * 16 <= 40 * 1024, "four workgroups share a CU's LDS");
+};
+
+template <int LC, int SH>
+__global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
+    const int *__restrict__ tab,            // group_rows[ngroups], then 4 * element offset of chunk (g, dy)'s first slot
+    int ngroups, int K, int period, int s0, int astep, float *__restrict__ C,
+    const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
+    int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes, unsigned c_bytes,
+    int txn, int tyn, int ndb)
+{
+    typedef DwShape<LC, SH> S;
+    constexpr int WAVES = S::WAVES, COLS = S::COLS, DYB = S::DYB, WQ = S::WQ, BPR = S::BPR, NIT = S::NIT;
+    __shared__ __attribute__((aligned(16))) float lds[2][S::BUF_PIECES * 4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    typedef const int __attribute__((address_space(4))) *sc_int_ptr;
+    const sc_int_ptr stab = (sc_int_ptr)tab;
+
+    // workgroup -> (group, block of window rows, tile row, tile column), the tile column fastest: the 64
+    // workgroups an XCD receives together are a band of neighbouring tiles, which share their stretches of B
+    int rest = xcd_tile(blockIdx.x, gridDim.x);
+    const int tx = rest % txn; rest /= txn;
+    const int ty = rest % tyn; rest /= tyn;
+    const int db = rest % ndb;
+    const int g = rest / ndb;
+    const int kb = min(DYB, K - DYB * db);                    // window rows served here
+    const int nbr = WAVES - 1 + kb;                           // stretches of B per column
+    const int i_tile = 4 * ty * period + S::TX * tx;          // the tile's first row of A
+    const int s_g = s0 + stab[g] + DYB * db * period;         // shift of this block's first slot
+    const int b_tile = i_tile + s_g - SH;                     // first staged row of B, a multiple of 4
+    // every slot of the workgroup pairs rows of A with rows [b_tile, b_hi) of B: nothing to do when none exists
+    const int b_hi = b_tile + (nbr - 1) * period + 4 * BPR;
+    if (i_tile >= h || b_hi <= 0 || b_tile >= w) return;
+
+    // This lane's requests of a group: instruction s = wave + WAVES * it carries pieces 64 s .. 64 s + 63 of the
+    // buffer -- B's first ((column, stretch, piece), nib instructions), then A's ((column, y, piece)).
+    const int npb = COLS * nbr * BPR;
+    const int nib = (npb + 63) / 64;
+    const int ni = nib + S::A_PIECES / 64;
+    unsigned v_lane[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+        const int s = wave + WAVES * it;
+        unsigned v = OOB_OFFSET;
+        if (s < nib) {
+            const int p = 64 * s + lane;
+            const int col = p / (nbr * BPR), rem = p - col * (nbr * BPR);
+            const int row = rem / BPR, pc = rem - row * BPR;
+            const int idx = b_tile + row * period + 4 * pc;
+            if ((p < npb) & (idx >= 0) & (idx + 4 <= w)) v = (unsigned)(col * (int)ldb + idx) * 4u;
+        } else if (s < ni) {
+            const int col = s - nib, row = lane >> 4, pc = lane & 15;
+            const int idx = i_tile + row * period + 4 * pc;
+            if (idx + 4 <= h) v = (unsigned)(col * (int)lda + idx) * 4u;
+        }
+        v_lane[it] = v;
+    }
+    const sp_int4 bq = raw_rsrc(B, b_bytes), aq = raw_rsrc(A, a_bytes);
+    const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
+    constexpr unsigned BUF_BYTES = S::BUF_PIECES * 16u;
+    const unsigned b_step = (unsigned)ldb * (4u * COLS), a_step = (unsigned)lda * (4u * COLS);    // bytes per group
+    // Requests the next group into buffer `par` and moves the lane's offsets one group on.  (An offset that is
+    // out of range stays so: it starts at 2^31, and all the steps of a walk add up to less than an operand's size.)
+    auto issue = [&](int par) __attribute__((always_inline)) {
+        const unsigned buf = lds0 + (unsigned)par * BUF_BYTES;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int s = wave + WAVES * it;
+            if (s < nib) {
+                lds_load_b128(bq, buf + 1024u * (unsigned)s, v_lane[it], 0u);
+                v_lane[it] += b_step;
+            } else if (s < ni) {
+                lds_load_b128(aq, buf + (unsigned)S::B_PIECES * 16u + 1024u * (unsigned)(s - nib), v_lane[it], 0u);
+                v_lane[it] += a_step;
+            }
+        }
+    };
+
+    const int role = lane >> 4, xg = lane & 15;
+    // floats from a buffer's start to this lane's windows (column 0) and to its piece of A
+    int w_off[2];
+#pragma unroll
+    for (int n = 0; n < 2; ++n) w_off[n] = ((wave + min(2 * role + n, kb - 1)) * BPR + xg) * 4;
+    const int col_floats = nbr * BPR * 4;
+    const int a_off = S::B_PIECES * 4 + (wave * 16 + xg) * 4;
+
+    float acc[2][4][LC];
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int j = 0; j < LC; ++j) acc[n][t][j] = 0.f;
+
+    struct Win { float v[WQ * 4]; };
+    auto read_win = [&](Win &win, const float *buf, int c, int n) __attribute__((always_inline)) {
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        const v4f *p4 = reinterpret_cast<const v4f *>(buf + c * col_floats + w_off[n]);
+#pragma unroll
+        for (int q = 0; q < WQ; ++q) {
+            v4f v = p4[q];
+            // (the window's first and last values may be unused: without this the compiler fetches the others
+            // one by one, and four-byte reads 16 bytes apart share their banks four ways)
+            asm volatile("" : "+v"(v));
+            win.v[4 * q + 0] = v.x; win.v[4 * q + 1] = v.y; win.v[4 * q + 2] = v.z; win.v[4 * q + 3] = v.w;
+        }
+    };
+    auto fmas = [&](int n, const float4 &a, const Win &win) __attribute__((always_inline)) {
+        const float av[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int j = 0; j < LC; ++j) acc[n][t][j] = __builtin_fmaf(av[t], win.v[SH + t + j], acc[n][t][j]);
+    };
+    // One group: the second window of a column and the next column's first are read while the FMAs of the
+    // window before them run.
+    auto apply = [&](const float *buf) __attribute__((always_inline)) {
+        Win w0, w1;
+        float4 a0, a1;
+        a0 = *reinterpret_cast<const float4 *>(buf + a_off);
+        read_win(w0, buf, 0, 0);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            float4 &ac = (c & 1) ? a1 : a0;
+            float4 &an = (c & 1) ? a0 : a1;
+            read_win(w1, buf, c, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            fmas(0, ac, w0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (c + 1 < COLS) {
+                an = *reinterpret_cast<const float4 *>(buf + a_off + (c + 1) * 256);
+                read_win(w0, buf, c + 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            fmas(1, ac, w1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    const int ngr = batch / COLS;
+    issue(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int gi = 0; gi < ngr; ++gi) {
+        if (gi + 1 < ngr) issue((gi + 1) & 1);
+        apply(&lds[gi & 1][0]);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // Results: 4 consecutive rows of every slot per lane, one 16-byte store where all four exist.
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    typedef unsigned sp_u4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t cr = make_rsrc(C, c_bytes);
+    const int o = i_tile + wave * period + 4 * xg;              // the lane's first row of A
+    const bool x_ok = S::TX * tx + 4 * xg < period;             // (a narrower last tile column: the positions past the
+                                                                // row belong to the next row's first tile)
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+        const int dyl = 2 * role + n;
+        const bool dy_ok = dyl < kb;
+        const int dy = DYB * db + (dy_ok ? dyl : 0);
+        const int e0 = tab[ngroups + g * K + dy] / 4 + o;       // element of slot j = 0 for row o
+        const int in0 = o + s_g + dyl * period;                 // the row of B that row o meets in slot j = 0
+#pragma unroll
+        for (int j = 0; j < LC; ++j) {
+            bool ok[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) ok[t] = dy_ok & x_ok & (o + t < h) & ((unsigned)(in0 + j + t) < (unsigned)w);
+            const bool all4 = ok[0] & ok[1] & ok[2] & ok[3];
+            const bool part = (ok[0] | ok[1] | ok[2] | ok[3]) & !all4;
+            const unsigned off = (unsigned)(e0 + j * astep) * 4u;
+            const bool any_part = __builtin_amdgcn_ballot_w64(part) != 0ull;       // wave-uniform
+            float r[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) r[t] = alpha * acc[n][t][j];
+            if (beta != 0.f) {
+                const f4u old4 = __builtin_bit_cast(f4u, __builtin_amdgcn_raw_buffer_load_b128(cr, all4 ? off : OOB_OFFSET, 0, 0));
+                float old[4] = {old4.x, old4.y, old4.z, old4.w};
+                if (any_part) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const float v = buffer_load_f32(cr, (part & ok[t]) ? off + 4u * t : OOB_OFFSET);
+                        old[t] = part ? v : old[t];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) r[t] = beta * old[t] + alpha * acc[n][t][j];
+            }
+            __builtin_amdgcn_raw_buffer_store_b128(sp_u4{__builtin_bit_cast(unsigned, r[0]), __builtin_bit_cast(unsigned, r[1]),
+                                                         __builtin_bit_cast(unsigned, r[2]), __builtin_bit_cast(unsigned, r[3])},
+                                                   cr, all4 ? off : OOB_OFFSET, 0, 2);
+            if (any_part) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, r[t]), cr,
+                                                          (part & ok[t]) ? off + 4u * t : OOB_OFFSET, 0, 2);
+            }
+        }
+    }
 }
 
 }  // namespace
@@ -2323,6 +2565,22 @@ struct WalkLaunch {
     hipStream_t stream;
 };
 hipError_t spmm_walk_launch(const WalkLaunch &L);
+// The window-table projection's launch (its unit instantiates the kernel for every chunk length and alignment).
+struct DwLaunch {
+    const int *tab;
+    int ngroups, k, period, s0, astep, lck;
+    float *vals;
+    const float *A;
+    long long lda;
+    const float *B;
+    long long ldb;
+    int h, w, batch;
+    float alpha, beta;
+    unsigned a_bytes, b_bytes, c_bytes;
+    int txn, tyn, ndb;
+    hipStream_t stream;
+};
+hipError_t dd2dia_window_launch(const DwLaunch &L);
 hipError_t spmm_tiled_launch_1_5(const SpLaunch &L);
 hipError_t spmm_tiled_launch_6_9(const SpLaunch &L);
 hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
@@ -2400,6 +2658,33 @@ hipError_t spmm_walk_launch(const WalkLaunch &L)
     else if (L.lck == 5) hipLaunchKernelGGL((spmm_walk_kernel<5, 5, 8, 2>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
     else hipLaunchKernelGGL((spmm_walk_kernel<3, 3, 8, 3>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
 #undef CUVDIA_WALK_ARGS
+    return hipGetLastError();
+}
+#endif
+#if CUVDIA_IN_PART(6)
+hipError_t dd2dia_window_launch(const DwLaunch &L)
+{
+    const long long blocks = (long long)L.ngroups * L.ndb * L.tyn * L.txn;
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)blocks);
+    const int sh = ((L.s0 % 4) + 4) % 4;
+#define CUVDIA_DW_ARGS L.tab, L.ngroups, L.k, L.period, L.s0, L.astep, L.vals, L.A, L.lda, L.B, L.ldb, L.h, L.w, L.batch, \
+                       L.alpha, L.beta, L.a_bytes, L.b_bytes, L.c_bytes, L.txn, L.tyn, L.ndb
+#define CUVDIA_DW_LAUNCH(LC)                                                                                          \
+    case LC:                                                                                                          \
+        if (sh == 0) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 0>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS); \
+        else if (sh == 1) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 1>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS); \
+        else if (sh == 2) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 2>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS); \
+        else hipLaunchKernelGGL((dd2dia_window_kernel<LC, 3>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS);        \
+        break;
+    note_kernel("dd2dia_window_kernel<%d, %d>", L.lck, sh);
+    switch (L.lck) {
+        CUVDIA_DW_LAUNCH(2) CUVDIA_DW_LAUNCH(3) CUVDIA_DW_LAUNCH(4) CUVDIA_DW_LAUNCH(5)
+        CUVDIA_DW_LAUNCH(6) CUVDIA_DW_LAUNCH(7) CUVDIA_DW_LAUNCH(8)
+        default: return hipErrorNotSupported;
+    }
+#undef CUVDIA_DW_LAUNCH
+#undef CUVDIA_DW_ARGS
     return hipGetLastError();
 }
 #endif
@@ -2570,10 +2855,47 @@ int dd2dia_slab_columns(const DiaView &C, long long lda, long long ldb)
     return whole >= DD2DIA_SLAB_MIN ? (int)std::min<long long>(whole, 1 << 30) : 0;
 }
 
+// Workgroups of the window-table projection on these operands, 0 where it does not apply: no window table,
+// chunks longer than CHUNK_MAX or shorter than 2, a period, group rows or row counts that are no multiples of 4
+// (its 16-byte pieces then straddle the operands' ends), a batch that is no multiple of its 4-column groups.
+long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn, int *tyn, int *ndb)
+{
+    const WalkView &wk = C.walk_n;
+    if (wk.tab_dev == nullptr || wk.lck < 2 || wk.lck > CHUNK_MAX || !wk.rows4 || wk.period % 4 != 0 ||
+        C.h % 4 != 0 || C.w % 4 != 0 || batch < 4 || batch % 4 != 0 || wk.astep4 % 4 != 0)
+        return 0;
+    const long long image_rows = ((long long)C.h + wk.period - 1) / wk.period;
+    const long long tx = ((long long)wk.period + 63) / 64, ty = (image_rows + 3) / 4, db = (wk.k + 7) / 8;
+    const long long total = tx * ty * db * wk.ngroups;
+    if (total > 0x7fffffffLL || (long long)4 * ty * wk.period + 64 * tx >= (1LL << 30)) return 0;
+    if (txn) *txn = (int)tx;
+    if (tyn) *tyn = (int)ty;
+    if (ndb) *ndb = (int)db;
+    return total;
+}
+
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
-                               float alpha, float beta, hipStream_t stream)
+                               float alpha, float beta, hipStream_t stream, int window, bool *windowed)
 {
+    if (windowed) *windowed = false;
+    if (window >= 0) {
+        int txn = 0, tyn = 0, ndb = 0;
+        const long long wgs = dd2dia_window_workgroups(C, batch, &txn, &tyn, &ndb);
+        // By size: the tiles must fill the chip (four workgroups per CU), and maps narrower than a tile's 64
+        // positions would leave lanes idle.
+        if (wgs > 0 && (window > 0 || (wgs >= DW_MIN_WGS && C.walk_n.period >= 64))) {
+            const WalkView &wk = C.walk_n;
+            const DwLaunch L{wk.tab_dev, wk.ngroups, wk.k, wk.period, wk.s0, wk.astep4 / 4, wk.lck, vals, A, lda, B, ldb,
+                             C.h, C.w, batch, alpha, beta,
+                             (unsigned)((((long long)batch - 1) * lda + C.h) * 4),
+                             (unsigned)((((long long)batch - 1) * ldb + C.w) * 4),
+                             (unsigned)((long long)C.nd * C.stride * 4), txn, tyn, ndb, stream};
+            if (windowed) *windowed = true;
+            return dd2dia_window_launch(L);
+        }
+    }
+    if (window > 0) return hipErrorNotSupported;
     // 16-byte loads of A need an aligned base and leading dimension and whole
     // groups of 4 rows; row tiles start at multiples of 256 and lanes at
     // multiples of 4 rows.

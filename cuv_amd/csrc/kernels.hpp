@@ -14,6 +14,7 @@ namespace cuvdia {
 struct WalkView {
     const int *tab_dev;          // group_rows[ngroups], then aoff4[ngroups * k]
     int ngroups, period, s0, k, lck, astep4;
+    bool rows4;                  // every group_rows[g] is a multiple of 4
 };
 
 struct DiaView {
@@ -107,9 +108,15 @@ int dd2dia_slab_columns(const DiaView &C, long long lda, long long ldb);
 // Same contract, row_fact == 1 only: a workgroup owns 256 rows of one run
 // chunk; each lane keeps 4 rows x (longest chunk) diagonals of partial sums,
 // the four waves split the batch and are summed through LDS in wave order.
+// Window tables whose tiles fill the chip go to the window-table projection (a tile of 4 x 64 positions of the
+// window's plane per workgroup, both operands staged once for all the slots of up to 8 window rows).
+// `window`: 0 -- that choice is made by size; 1 -- that kernel or hipErrorNotSupported; -1 -- never.
+// *windowed (if not null) tells which ran.
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
-                               float alpha, float beta, hipStream_t stream);
+                               float alpha, float beta, hipStream_t stream, int window = 0, bool *windowed = nullptr);
+// Workgroups of the window-table projection for these operands (0: it does not apply).
+long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn = nullptr, int *tyn = nullptr, int *ndb = nullptr);
 
 // The allocation-free entry point keeps its device tables in a static device
 // array instead of a descriptor's allocation: the offset table at byte 0 (up

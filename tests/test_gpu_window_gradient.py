@@ -1,0 +1,161 @@
+"""The window-table projection kernel against the CPU oracle.
+
+Window tables (k window rows of up to 8 consecutive diagonals, `period` rows apart) whose tiles fill the chip
+are served by workgroups that own a tile of 4 x 64 positions of the window's plane.  The tests force that
+kernel (the path switch the walking product uses) on sizes the oracle finishes in seconds, with NaN in every
+padding slot of the destination, and check what the automatic choice does on both sides of its size rule and
+that tables the kernel does not serve are refused when it is forced.  Tolerance: the fp32 bar of
+_gpu_util.assert_close_mag (1e-5 of the sum of |terms| per element).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gu():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    import _gpu_util
+    return _gpu_util
+
+
+def _dia(o, rng, h, w, offsets):
+    d = o.Dia(h, w, np.asarray(offsets, np.int32), None, 1)
+    d.vals[:] = np.nan
+    m = o.valid_mask(d)
+    d.vals[m] = rng.uniform(-1, 1, int(m.sum())).astype(np.float32)
+    return d
+
+
+def _operands(rng, C, batch):
+    A = np.asfortranarray(rng.uniform(-1, 1, (C.h, batch)).astype(np.float32))
+    B = np.asfortranarray(rng.uniform(-1, 1, (C.w, batch)).astype(np.float32))
+    return A, B
+
+
+def _last_kernel():
+    from cuv_amd import _lib
+    return _lib.lib().cuvdia_last_kernel().decode()
+
+
+def _window(px, rows, cols, first_dy, first_dx, channels=1, map_elems=None):
+    map_elems = px * px if map_elems is None else map_elems
+    return [c * map_elems + (first_dy + dy) * px + first_dx + dx
+            for c in range(channels) for dy in range(rows) for dx in range(cols)]
+
+
+# px (period), rows of A, rows of B, window rows x columns, first dy, first dx, channels, batch
+CASES = [
+    (64, 64 * 12, 64 * 12, 7, 7, -3, -3, 1, 8),        # the centred 7 x 7, one tile column
+    (128, 128 * 9, 128 * 9, 7, 7, -3, -3, 1, 12),      # two tile columns, a last tile row of one map row
+    (72, 72 * 10, 72 * 10, 5, 5, -2, -2, 1, 20),       # a narrower last tile column
+    (64, 64 * 8, 64 * 8, 3, 3, -1, -1, 1, 4),          # a single group of columns
+    (64, 64 * 8, 64 * 11, 4, 8, 0, 0, 1, 16),          # chunks of 8, window rows all below, a wider B
+    (64, 64 * 11, 64 * 8, 2, 6, -1, -5, 1, 16),        # a taller A, alignment shift 3
+    (96, 96 * 8, 96 * 8, 11, 3, -5, -1, 1, 8),         # 11 window rows: two blocks of window rows
+    (64, 64 * 16, 64 * 16, 7, 7, -3, -3, 2, 8),        # two groups (channels)
+    (64, 64 * 12 - 4, 64 * 12 - 8, 5, 7, -2, -3, 1, 8),    # row counts that end inside a map row
+]
+
+
+@pytest.mark.parametrize("px,h,w,rows,cols,dy0,dx0,channels,batch", CASES)
+def test_window_projection_matches_the_oracle(oracle, gu, px, h, w, rows, cols, dy0, dx0, channels, batch):
+    from cuv_amd import _lib
+    rng = np.random.default_rng(px + h + w + rows * 7 + cols + batch)
+    offsets = _window(px, rows, cols, dy0, dx0, channels, map_elems=(h // channels) // 4 * 4)
+    C = _dia(oracle, rng, h, w, offsets)
+    A, B = _operands(rng, C, batch)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_WALK, "window beta0")
+    assert ran == _lib.PATH_WALK and _last_kernel().startswith("dd2dia_window_kernel<%d," % cols)
+    C.vals[oracle.valid_mask(C)] = rng.uniform(-1, 1, int(oracle.valid_mask(C).sum())).astype(np.float32)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0 / batch, 0.9, _lib.PATH_WALK, "window scaled")
+    assert ran == _lib.PATH_WALK
+
+
+def test_window_projection_with_padded_operands_and_a_table_in_descending_order(oracle, gu):
+    """Leading dimensions larger than the row counts (rows of the next column follow a column's last row at a
+    distance), and the offsets listed from the last to the first."""
+    import torch
+    from cuv_amd import _lib, dia as D
+    rng = np.random.default_rng(11)
+    px, n, batch = 64, 64 * 10, 12
+    offsets = _window(px, 7, 7, -3, -3)[::-1]
+    C = _dia(oracle, rng, n, n, offsets)
+    A, B = _operands(rng, C, batch)
+    ref = oracle.dd2dia(C, A, B, 0.5, 0.0)
+    L = _lib.lib()
+    Cd = gu.make_dev_dia(C)
+    lda, ldb = n + 12, n + 20
+    Ad = torch.full((batch + 2, lda), float("nan"), dtype=torch.float32, device="cuda:0")
+    Bd = torch.full((batch + 2, ldb), float("nan"), dtype=torch.float32, device="cuda:0")
+    Ad[1:batch + 1, :n] = D.to_device_colmajor(A)
+    Bd[1:batch + 1, :n] = D.to_device_colmajor(B)
+    L.cuvdia_set_path(_lib.PATH_WALK)
+    try:
+        D.densedense_to_dia(Cd, D.dev_block_descriptor_f(Cd), Ad[1:batch + 1, :n], Bd[1:batch + 1, :n], 0.5, 0.0)
+        assert L.cuvdia_last_path() == _lib.PATH_WALK
+    finally:
+        L.cuvdia_set_path(_lib.PATH_AUTO)
+    got = Cd.pull()
+    valid = oracle.valid_mask(C)
+    mag = oracle.dd2dia_f64(type(C)(C.h, C.w, C.offsets, C.stride, C.rf, np.abs(C.vals)), np.abs(A), np.abs(B), 0.5, 0.0)
+    gu.assert_close_mag(got[valid], ref[valid], mag[valid], "padded operands")
+    assert np.isnan(got[~valid]).all()
+
+
+def test_non_finite_values_stay_in_the_slots_that_use_them(oracle, gu):
+    """An infinity in A and a NaN in B reach exactly the slots whose sums contain them."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(3)
+    px, n, batch = 64, 64 * 9, 8
+    C = _dia(oracle, rng, n, n, _window(px, 7, 7, -3, -3))
+    A, B = _operands(rng, C, batch)
+    A[5 * px + 17, 3] = np.inf
+    B[2 * px + 40, 6] = np.nan
+    B[0, 0] = np.inf
+    A[n - 1, batch - 1] = -np.inf
+    got, ran = gu.gpu_dd2dia(C, A, B, 1.0, 0.0, _lib.PATH_WALK)
+    assert ran == _lib.PATH_WALK
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = oracle.dd2dia(C, A, B, 1.0, 0.0)
+    valid = oracle.valid_mask(C)
+    fin = np.isfinite(ref) & valid
+    assert np.array_equal(np.isnan(got[valid]), np.isnan(ref[valid]))
+    assert np.array_equal(np.isposinf(got[valid]), np.isposinf(ref[valid]))
+    assert np.array_equal(np.isneginf(got[valid]), np.isneginf(ref[valid]))
+    assert (~np.isfinite(ref[valid])).sum() > 0
+    np.testing.assert_allclose(got[fin], ref[fin], rtol=0, atol=1e-4)
+
+
+def test_the_choice_by_size_and_the_refusals(oracle, gu):
+    from cuv_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(21)
+    # 768 tiles: taken by size
+    px, n, batch = 256, 256 * 768, 4
+    C = _dia(oracle, rng, n, n, _window(px, 3, 3, -1, -1))
+    A, B = _operands(rng, C, batch)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_AUTO, "taken by size")
+    assert ran == _lib.PATH_WALK and _last_kernel().startswith("dd2dia_window_kernel<3,")
+    # the same table on fewer rows: left to the chunk-by-chunk kernel, which agrees
+    n = 256 * 64
+    C = _dia(oracle, rng, n, n, _window(px, 3, 3, -1, -1))
+    A, B = _operands(rng, C, batch)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_AUTO, "left alone")
+    assert ran == _lib.PATH_TILED and _last_kernel().startswith("dd2dia_tiled_kernel")
+    # forced on what it does not serve: a batch that is no multiple of 4, a period that is none, no window table
+    for offsets, b in ((_window(256, 3, 3, -1, -1), 6), (_window(254, 3, 3, -1, -1), 8), ([-5, -1, 0, 1, 9], 8)):
+        C = _dia(oracle, rng, n, n, offsets)
+        A, B = _operands(rng, C, b)
+        Cd = gu.make_dev_dia(C)
+        from cuv_amd import dia as D
+        Ad, Bd = D.to_device_colmajor(A), D.to_device_colmajor(B)
+        L.cuvdia_set_path(_lib.PATH_WALK)
+        try:
+            with pytest.raises(_lib.CuvDiaError) as err:
+                D.densedense_to_dia(Cd, D.dev_block_descriptor_f(Cd), Ad, Bd, 1.0, 0.0)
+        finally:
+            L.cuvdia_set_path(_lib.PATH_AUTO)
+        assert err.value.code == _lib.EUNSUPPORTED
