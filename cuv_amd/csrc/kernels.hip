@@ -2175,7 +2175,7 @@ __device__ __forceinline__ void dd2dia_unit(
 
 // Shape of the blocks the projection's tiles are numbered in (see the kernel): units per block and row tiles per
 // block, 64 positions or nearly.
-constexpr int DW_MIN_WGS = 768;               // below this the window-table projection leaves CUs short of work
+constexpr int DW_MIN_WGS = 768;               // workgroups from which the window-table projection of a 7 x 7 window is ahead
 constexpr int DD_BLOCKED_MIN_TILES = 1024;   // launches of more than a few rounds number their tiles in blocks
 struct DdBlock {
     __host__ __device__ static int units(int nunits) { return nunits < 16 ? nunits : 16; }
@@ -2262,15 +2262,21 @@ __global__ __launch_bounds__((PAIRS && WIDE != DD_SHIFTED) ? 512 : 256) void dd2
 // arrive as zeros.
 // Lane = (role r = lane / 16, xg = lane mod 16): positions x = 64 tx + 4 xg .. + 3 of the wave's y, window rows
 // dy = 2r and 2r + 1 of the workgroup's eight: 2 x 4 x LC running sums, one 16-byte read of A and two windows
-// of B (4 + LC - 1 values each, WQ 16-byte reads) per column.  Two LDS buffers: while group i is applied, group
-// i + 1 lands; one wait and one barrier per group.  A lane's share of a group's requests is the same for the
+// of B (4 + LC - 1 values each, WQ 16-byte reads) per column.  A ring of NBUF LDS buffers: while group i is
+// applied, the groups up to i + NBUF - 1 land; one wait and one barrier per group.  (Two buffers of 4 columns
+// measured best: with 4 buffers of 2 columns -- half as much again in flight in the same LDS -- the 512 x 512
+// map at batch 512 took 344 us instead of 315, with 3 buffers of 4 columns, which leave room for 2 or 3
+// workgroups per CU, 424.  What bounds the kernel at those sizes is the operands' one trip from memory:
+// with neither FMAs nor LDS reads it takes 288 us.)  A lane's share of a group's requests is the same for the
 // whole walk up to the column step, so its byte offsets are computed once; everything, column included, goes
 // into the vector offset, which the buffer's range check covers.
 //
 // Accumulation order per slot: batch columns ascending, acc = fma(a, b, acc); C = beta*C + alpha*acc.
 template <int LC, int SH>
 struct DwShape {
-    static constexpr int WAVES = 4, TX = 64, COLS = 4, DYB = 8;
+    static constexpr int WAVES = 4, TX = 64, DYB = 8;
+    static constexpr int COLS = 4;                               // batch columns per staged group
+    static constexpr int NBUF = 2;                               // LDS buffers: the group applied + those in flight
     static constexpr int WIN = SH + 4 + LC - 1;                  // values of a lane's window, from its first piece
     static constexpr int WQ = (WIN + 3) / 4;                     // .. as 16-byte reads
     static constexpr int BPR = TX / 4 + WQ - 1;                  // pieces per staged stretch of B
@@ -2281,8 +2287,19 @@ struct DwShape {
     static constexpr int NI_MAX = BUF_PIECES / 64;               // load instructions per group
     static constexpr int NIT = (NI_MAX + WAVES - 1) / WAVES;     // .. per wave
     static_assert(A_PIECES % 64 == 0 && LC >= 1 && LC <= CHUNK_MAX && SH >= 0 && SH < 4, "shape");
-    static_assert(2 * BUF_PIECES * 16 <= 40 * 1024, "four workgroups share a CU's LDS");
+    static_assert(NBUF >= 2 && NBUF * BUF_PIECES * 16 <= 40 * 1024, "four workgroups share a CU's LDS");
+    static_assert((NBUF - 2) * NIT <= 8, "the waits name up to eight requests left in flight");
 };
+
+// calls body(gi + I, I) for I = 0 .. N-1 while gi + I < n: the position in the ring is a compile-time constant
+template <int N, int I, class F>
+__device__ __forceinline__ void dw_ring(F &body, int gi, int n)
+{
+    if constexpr (I < N) {
+        if (gi + I < n) body(gi + I, std::integral_constant<int, I>{});
+        dw_ring<N, I + 1>(body, gi, n);
+    }
+}
 
 template <int LC, int SH>
 __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
@@ -2294,7 +2311,7 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
 {
     typedef DwShape<LC, SH> S;
     constexpr int WAVES = S::WAVES, COLS = S::COLS, DYB = S::DYB, WQ = S::WQ, BPR = S::BPR, NIT = S::NIT;
-    __shared__ __attribute__((aligned(16))) float lds[2][S::BUF_PIECES * 4];
+    __shared__ __attribute__((aligned(16))) float lds[S::NBUF][S::BUF_PIECES * 4];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     typedef const int __attribute__((address_space(4))) *sc_int_ptr;
@@ -2421,16 +2438,39 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
         }
     };
 
+    // The ring: group gi is applied out of buffer gi mod NBUF while the groups up to gi + NBUF - 1 are in flight or
+    // landed.  At a group's end everything but the requests of the groups after the next has to have arrived: this
+    // wave's share of a group is n_mine instructions, and they complete in order.
     const int ngr = batch / COLS;
-    issue(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const int n_mine = (ni - wave + WAVES - 1) / WAVES;
+    auto wait_leaving_groups = [&](int groups) __attribute__((always_inline)) {
+        switch (groups * n_mine) {
+            case 0: asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)" ::: "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory"); break;
+            case 3: asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory"); break;
+            case 4: asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory"); break;
+            case 5: asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory"); break;
+            case 6: asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory"); break;
+            case 7: asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory"); break;
+        }
+    };
+    constexpr int NBUF = S::NBUF;
+    for (int k = 0; k < NBUF - 1; ++k)
+        if (k < ngr) issue(k);
+    wait_leaving_groups(min(NBUF - 2, ngr - 1));
     __syncthreads();
-    for (int gi = 0; gi < ngr; ++gi) {
-        if (gi + 1 < ngr) issue((gi + 1) & 1);
-        apply(&lds[gi & 1][0]);
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    auto body = [&](int gi, auto cur_c) __attribute__((always_inline)) {
+        constexpr int cur = decltype(cur_c)::value;
+        // (the buffer the group before this one was applied from: every wave left it at the last barrier)
+        if (gi + NBUF - 1 < ngr) issue((cur + NBUF - 1) % NBUF);
+        apply(&lds[cur][0]);
+        wait_leaving_groups(max(0, min(NBUF - 2, ngr - 2 - gi)));
         __syncthreads();
-    }
+    };
+#pragma clang loop unroll(disable)
+    for (int gi = 0; gi < ngr; gi += NBUF) dw_ring<NBUF, 0>(body, gi, ngr);
 
     // Results: 4 consecutive rows of every slot per lane, one 16-byte store where all four exist.
     typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -2882,9 +2922,14 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     if (window >= 0) {
         int txn = 0, tyn = 0, ndb = 0;
         const long long wgs = dd2dia_window_workgroups(C, batch, &txn, &tyn, &ndb);
-        // By size: the tiles must fill the chip (four workgroups per CU), and maps narrower than a tile's 64
-        // positions would leave lanes idle.
-        if (wgs > 0 && (window > 0 || (wgs >= DW_MIN_WGS && C.walk_n.period >= 64))) {
+        // By size: the tiles must fill the chip (four workgroups per CU) -- the smaller the window, the less a tile
+        // saves over the chunk-by-chunk kernel and the more tiles it takes (measured on 7 x 7, 5 x 5 and 3 x 3
+        // windows of maps 256 to 1024 wide at batch 32 to 512: ahead from 768, 1024 and 1536 tiles on, the 3 x 3 only
+        // from batch 128) -- and maps narrower than a tile's 64 positions would leave lanes idle.
+        const int slots = C.walk_n.k * C.walk_n.lck;
+        const long long min_wgs = slots >= 49 ? DW_MIN_WGS : slots >= 25 ? DW_MIN_WGS * 4 / 3 : DW_MIN_WGS * 2;
+        const bool by_size = wgs >= min_wgs && C.walk_n.period >= 64 && (slots >= 25 || batch >= 128);
+        if (wgs > 0 && (window > 0 || by_size)) {
             const WalkView &wk = C.walk_n;
             const DwLaunch L{wk.tab_dev, wk.ngroups, wk.k, wk.period, wk.s0, wk.astep4 / 4, wk.lck, vals, A, lda, B, ldb,
                              C.h, C.w, batch, alpha, beta,

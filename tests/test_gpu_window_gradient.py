@@ -133,12 +133,17 @@ def test_the_choice_by_size_and_the_refusals(oracle, gu):
     from cuv_amd import _lib
     L = _lib.lib()
     rng = np.random.default_rng(21)
-    # 768 tiles: taken by size
-    px, n, batch = 256, 256 * 768, 4
-    C = _dia(oracle, rng, n, n, _window(px, 3, 3, -1, -1))
+    # 1024 tiles of a 5 x 5 window: taken by size
+    px, n, batch = 256, 256 * 1024, 4
+    C = _dia(oracle, rng, n, n, _window(px, 5, 5, -2, -2))
     A, B = _operands(rng, C, batch)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_AUTO, "taken by size")
-    assert ran == _lib.PATH_WALK and _last_kernel().startswith("dd2dia_window_kernel<3,")
+    assert ran == _lib.PATH_WALK and _last_kernel().startswith("dd2dia_window_kernel<5,")
+    # as many tiles of a 3 x 3 window at a small batch: not taken
+    C = _dia(oracle, rng, n, n, _window(px, 3, 3, -1, -1))
+    A, B = _operands(rng, C, batch)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_AUTO, "small window, small batch")
+    assert ran == _lib.PATH_TILED
     # the same table on fewer rows: left to the chunk-by-chunk kernel, which agrees
     n = 256 * 64
     C = _dia(oracle, rng, n, n, _window(px, 3, 3, -1, -1))
