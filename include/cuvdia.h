@@ -50,8 +50,9 @@ extern "C" {
 #define CUVDIA_PATH_AUTO     0  /* pick by shape (default)                        */
 #define CUVDIA_PATH_GENERIC  1  /* one-thread-per-output kernels, any row_fact    */
 #define CUVDIA_PATH_TILED    2  /* LDS-staged, register-blocked kernels (rf == 1) */
-#define CUVDIA_PATH_WALK     3  /* of the tiled family: the walking kernel for window tables (products only) */
-#define CUVDIA_PATH_TILED_NOWALK 4  /* the tiled family without its walking kernel (products only)         */
+#define CUVDIA_PATH_WALK     3  /* of the tiled family: the kernels for window tables (the walking product, the
+                                 * projection tiled in the window's plane)                                  */
+#define CUVDIA_PATH_TILED_NOWALK 4  /* the tiled family without its kernels for window tables                  */
 
 /* Activation applied by cuvdia_spmm_bias_act_f32. */
 #define CUVDIA_ACT_NONE      0
@@ -236,7 +237,12 @@ int cuvdia_learn_step_weight_decay_momentum_f32(float *W_device, float *momentum
  * A is h x batch (lda >= h), B is w x batch (ldb >= w).  beta == 0 never
  * reads C.  batch == 0 scales C by beta (zero-fills valid slots if beta == 0).
  * A batch whose operands are larger than 2 GiB is worked in several launches
- * on `stream`, slab of columns after slab, each adding to C. */
+ * on `stream`, slab of columns after slab, each adding to C.
+ * Summation order per slot: see kernels.hip; the kernel for large window
+ * tables (cuvdia_last_path() == CUVDIA_PATH_WALK) adds the batch columns in
+ * ascending order into one sum, the chunk-by-chunk kernel into four or eight
+ * partial sums: their results differ by rounding, both within 1e-5 of the
+ * sum of |terms| of the reference's host result. */
 int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals_device,
                       const float *A_device, long long lda,
                       const float *B_device, long long ldb, int batch,
@@ -311,15 +317,18 @@ int cuvdia_cache_clear(void);
  * run both families on the same inputs).  CUVDIA_PATH_TILED on a request the
  * tiled kernels cannot serve (row_fact > 1) returns CUVDIA_EUNSUPPORTED from
  * the compute call.  CUVDIA_PATH_WALK and CUVDIA_PATH_TILED_NOWALK choose
- * inside the tiled family for the products (cuvdia_spmm_*): the walking
- * kernel whatever the product's size (CUVDIA_EUNSUPPORTED when the table is
- * no window table it serves), or never; densedense_to_dia treats both as
- * CUVDIA_PATH_TILED. */
+ * inside the tiled family: the kernel for window tables whatever the size
+ * of the operands (CUVDIA_EUNSUPPORTED when it does not serve the request:
+ * for a product, a table that is no window table with a walking kernel; for
+ * densedense_to_dia, one that is no window table of chunks of 2 to 8
+ * diagonals, a period, channel distances or row counts that are no
+ * multiples of 4, or a batch that is none), or never. */
 int cuvdia_set_path(int path);
 
 /* Which family the most recent compute call on this thread launched
  * (CUVDIA_PATH_GENERIC, CUVDIA_PATH_TILED or -- a product served by the
- * walking kernel -- CUVDIA_PATH_WALK; 0 before any call). */
+ * walking kernel, a projection served by the kernel tiled in the window's
+ * plane -- CUVDIA_PATH_WALK; 0 before any call). */
 int cuvdia_last_path(void);
 
 /* Name of the kernel the most recent compute call on this thread launched
