@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libcuvdia.so")
 OK = 0
 EINVAL, ESHAPE, EHIP, ENOMEM, EUNSUPPORTED, ENODEVICE, ETOOLARGE = -1, -2, -3, -4, -5, -6, -7
 ACT_NONE, ACT_SIGMOID, ACT_SIGMOID_SAMPLE = 0, 1, 2
-PATH_AUTO, PATH_GENERIC, PATH_TILED, PATH_WALK, PATH_TILED_NOWALK = 0, 1, 2, 3, 4
+PATH_AUTO, PATH_GENERIC, PATH_TILED, PATH_WALK, PATH_TILED_NOWALK, PATH_WINDOW = 0, 1, 2, 3, 4, 5
 
 _lib = None
 

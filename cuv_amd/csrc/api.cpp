@@ -133,7 +133,7 @@ const char *cuvdia_last_hip_error(void) { return t_hip_error.c_str(); }
 int cuvdia_set_path(int path)
 {
     if (path != CUVDIA_PATH_AUTO && path != CUVDIA_PATH_GENERIC && path != CUVDIA_PATH_TILED &&
-        path != CUVDIA_PATH_TILED_NOWALK && path != CUVDIA_PATH_WALK)
+        path != CUVDIA_PATH_TILED_NOWALK && path != CUVDIA_PATH_WALK && path != CUVDIA_PATH_WINDOW)
         return CUVDIA_EINVAL;
     g_path.store(path);
     return CUVDIA_OK;
@@ -401,7 +401,8 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const fl
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool tiled_possible = spmm_tiled_ok(desc->view, ldb, ldd, trans);
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK ||
+        forced == CUVDIA_PATH_WINDOW) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {
@@ -410,7 +411,8 @@ int cuvdia_spmm_layer_f32(const cuvdia_desc *desc, const float *A_vals, const fl
         tiled = tiled_possible && batch >= SPMM_TILED_MIN_BATCH;
     }
     bool walked = false;
-    const int walk = forced == CUVDIA_PATH_WALK ? 1 : forced == CUVDIA_PATH_TILED_NOWALK ? -1 : 0;
+    const int walk = forced == CUVDIA_PATH_WALK ? 1
+                     : (forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WINDOW) ? -1 : 0;
     const hipError_t e = tiled
         ? launch_spmm_tiled(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s, walk, &walked)
         : launch_spmm_generic(desc->view, A_vals, B, ldb, dst, ldd, batch, trans, alpha, beta, ep, s);
@@ -490,7 +492,8 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
         }
     }
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK ||
+        forced == CUVDIA_PATH_WINDOW) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {
@@ -504,7 +507,8 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
     if (!tiled) {
         e = launch_dd2dia_generic(desc->view, C_vals, A, lda, B, ldb, batch, alpha, beta, s);
     } else {
-        const int window = forced == CUVDIA_PATH_WALK ? 1 : forced == CUVDIA_PATH_TILED_NOWALK ? -1 : 0;
+        const int window = forced == CUVDIA_PATH_WINDOW ? 1
+                           : (forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WALK) ? -1 : 0;
         for (int c0 = 0; c0 < batch && e == hipSuccess; c0 += slab) {
             bool this_one = false;
             e = launch_dd2dia_tiled(desc->view, C_vals, A + (long long)c0 * lda, lda, B + (long long)c0 * ldb, ldb,
@@ -516,7 +520,7 @@ int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals, const float *A, lo
             return CUVDIA_EUNSUPPORTED;
         }
     }
-    t_last_path = !tiled ? CUVDIA_PATH_GENERIC : windowed ? CUVDIA_PATH_WALK : CUVDIA_PATH_TILED;
+    t_last_path = !tiled ? CUVDIA_PATH_GENERIC : windowed ? CUVDIA_PATH_WINDOW : CUVDIA_PATH_TILED;
     return e == hipSuccess ? CUVDIA_OK : hip_fail(e, "dd2dia kernel launch");
 }
 
@@ -670,7 +674,7 @@ int cuvdia_spmm_offsets_noalloc_f32(const float *A_vals, const int *offsets_host
     if (forced == CUVDIA_PATH_WALK) return CUVDIA_EUNSUPPORTED;
     const bool tiled_possible = spmm_tiled_ok(view, ldb, ldd, trans);
     bool tiled;
-    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK) {
+    if (forced == CUVDIA_PATH_TILED || forced == CUVDIA_PATH_TILED_NOWALK || forced == CUVDIA_PATH_WINDOW) {
         if (!tiled_possible) return CUVDIA_EUNSUPPORTED;
         tiled = true;
     } else if (forced == CUVDIA_PATH_GENERIC) {

@@ -2441,7 +2441,9 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
     // The ring: group gi is applied out of buffer gi mod NBUF while the groups up to gi + NBUF - 1 are in flight or
     // landed.  At a group's end everything but the requests of the groups after the next has to have arrived: this
     // wave's share of a group is n_mine instructions, and they complete in order.
-    const int ngr = batch / COLS;
+    // (the columns of a last, partial group past the batch start a whole column past the last one: out of the
+    // resources' range, they arrive as zeros and add nothing)
+    const int ngr = (batch + COLS - 1) / COLS;
     const int n_mine = (ni - wave + WAVES - 1) / WAVES;
     auto wait_leaving_groups = [&](int groups) __attribute__((always_inline)) {
         switch (groups * n_mine) {
@@ -2897,12 +2899,12 @@ int dd2dia_slab_columns(const DiaView &C, long long lda, long long ldb)
 
 // Workgroups of the window-table projection on these operands, 0 where it does not apply: no window table,
 // chunks longer than CHUNK_MAX or shorter than 2, a period, group rows or row counts that are no multiples of 4
-// (its 16-byte pieces then straddle the operands' ends), a batch that is no multiple of its 4-column groups.
+// (its 16-byte pieces then straddle the operands' ends).
 long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn, int *tyn, int *ndb)
 {
     const WalkView &wk = C.walk_n;
     if (wk.tab_dev == nullptr || wk.lck < 2 || wk.lck > CHUNK_MAX || !wk.rows4 || wk.period % 4 != 0 ||
-        C.h % 4 != 0 || C.w % 4 != 0 || batch < 4 || batch % 4 != 0 || wk.astep4 % 4 != 0)
+        C.h % 4 != 0 || C.w % 4 != 0 || batch < 1 || wk.astep4 % 4 != 0)
         return 0;
     const long long image_rows = ((long long)C.h + wk.period - 1) / wk.period;
     const long long tx = ((long long)wk.period + 63) / 64, ty = (image_rows + 3) / 4, db = (wk.k + 7) / 8;

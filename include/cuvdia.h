@@ -50,9 +50,9 @@ extern "C" {
 #define CUVDIA_PATH_AUTO     0  /* pick by shape (default)                        */
 #define CUVDIA_PATH_GENERIC  1  /* one-thread-per-output kernels, any row_fact    */
 #define CUVDIA_PATH_TILED    2  /* LDS-staged, register-blocked kernels (rf == 1) */
-#define CUVDIA_PATH_WALK     3  /* of the tiled family: the kernels for window tables (the walking product, the
-                                 * projection tiled in the window's plane)                                  */
+#define CUVDIA_PATH_WALK     3  /* of the tiled family: the walking kernel for window tables (products only) */
 #define CUVDIA_PATH_TILED_NOWALK 4  /* the tiled family without its kernels for window tables                  */
+#define CUVDIA_PATH_WINDOW   5  /* of the tiled family: the projection tiled in the window's plane (window tables) */
 
 /* Activation applied by cuvdia_spmm_bias_act_f32. */
 #define CUVDIA_ACT_NONE      0
@@ -239,7 +239,7 @@ int cuvdia_learn_step_weight_decay_momentum_f32(float *W_device, float *momentum
  * A batch whose operands are larger than 2 GiB is worked in several launches
  * on `stream`, slab of columns after slab, each adding to C.
  * Summation order per slot: see kernels.hip; the kernel for large window
- * tables (cuvdia_last_path() == CUVDIA_PATH_WALK) adds the batch columns in
+ * tables (cuvdia_last_path() == CUVDIA_PATH_WINDOW) adds the batch columns in
  * ascending order into one sum, the chunk-by-chunk kernel into four or eight
  * partial sums: their results differ by rounding, both within 1e-5 of the
  * sum of |terms| of the reference's host result. */
@@ -316,19 +316,22 @@ int cuvdia_cache_clear(void);
 /* Forces a kernel family for subsequent calls (process-wide; tests use it to
  * run both families on the same inputs).  CUVDIA_PATH_TILED on a request the
  * tiled kernels cannot serve (row_fact > 1) returns CUVDIA_EUNSUPPORTED from
- * the compute call.  CUVDIA_PATH_WALK and CUVDIA_PATH_TILED_NOWALK choose
- * inside the tiled family: the kernel for window tables whatever the size
- * of the operands (CUVDIA_EUNSUPPORTED when it does not serve the request:
- * for a product, a table that is no window table with a walking kernel; for
- * densedense_to_dia, one that is no window table of chunks of 2 to 8
- * diagonals, a period, channel distances or row counts that are no
- * multiples of 4, or a batch that is none), or never. */
+ * the compute call.  CUVDIA_PATH_WALK, CUVDIA_PATH_WINDOW and
+ * CUVDIA_PATH_TILED_NOWALK choose inside the tiled family: a kernel for
+ * window tables whatever the size of the operands, or none of them.
+ * CUVDIA_PATH_WALK: the walking product (CUVDIA_EUNSUPPORTED for a table
+ * that is no window table with a walking kernel; densedense_to_dia treats it
+ * as CUVDIA_PATH_TILED_NOWALK).  CUVDIA_PATH_WINDOW: the kernels tiled in the
+ * window's plane, which serve densedense_to_dia (CUVDIA_EUNSUPPORTED when
+ * they do not serve the request: no window table of chunks of 2 to 8
+ * diagonals, a period, channel distances or row counts that are no multiples
+ * of 4); the products treat it as CUVDIA_PATH_TILED_NOWALK. */
 int cuvdia_set_path(int path);
 
 /* Which family the most recent compute call on this thread launched
- * (CUVDIA_PATH_GENERIC, CUVDIA_PATH_TILED or -- a product served by the
- * walking kernel, a projection served by the kernel tiled in the window's
- * plane -- CUVDIA_PATH_WALK; 0 before any call). */
+ * (CUVDIA_PATH_GENERIC, CUVDIA_PATH_TILED, CUVDIA_PATH_WALK for a product
+ * served by the walking kernel, CUVDIA_PATH_WINDOW for a projection served
+ * by the kernel tiled in the window's plane; 0 before any call). */
 int cuvdia_last_path(void);
 
 /* Name of the kernel the most recent compute call on this thread launched

@@ -2,7 +2,7 @@
 
 Window tables (k window rows of up to 8 consecutive diagonals, `period` rows apart) whose tiles fill the chip
 are served by workgroups that own a tile of 4 x 64 positions of the window's plane.  The tests force that
-kernel (the path switch the walking product uses) on sizes the oracle finishes in seconds, with NaN in every
+kernel (CUVDIA_PATH_WINDOW) on sizes the oracle finishes in seconds, with NaN in every
 padding slot of the destination, and check what the automatic choice does on both sides of its size rule and
 that tables the kernel does not serve are refused when it is forced.  Tolerance: the fp32 bar of
 _gpu_util.assert_close_mag (1e-5 of the sum of |terms| per element).
@@ -49,9 +49,9 @@ def _window(px, rows, cols, first_dy, first_dx, channels=1, map_elems=None):
 # px (period), rows of A, rows of B, window rows x columns, first dy, first dx, channels, batch
 CASES = [
     (64, 64 * 12, 64 * 12, 7, 7, -3, -3, 1, 8),        # the centred 7 x 7, one tile column
-    (128, 128 * 9, 128 * 9, 7, 7, -3, -3, 1, 12),      # two tile columns, a last tile row of one map row
-    (72, 72 * 10, 72 * 10, 5, 5, -2, -2, 1, 20),       # a narrower last tile column
-    (64, 64 * 8, 64 * 8, 3, 3, -1, -1, 1, 4),          # a single group of columns
+    (128, 128 * 9, 128 * 9, 7, 7, -3, -3, 1, 13),      # two tile columns, a last tile row of one map row, a ragged batch
+    (72, 72 * 10, 72 * 10, 5, 5, -2, -2, 1, 22),       # a narrower last tile column
+    (64, 64 * 8, 64 * 8, 3, 3, -1, -1, 1, 3),          # less than one group of columns
     (64, 64 * 8, 64 * 11, 4, 8, 0, 0, 1, 16),          # chunks of 8, window rows all below, a wider B
     (64, 64 * 11, 64 * 8, 2, 6, -1, -5, 1, 16),        # a taller A, alignment shift 3
     (96, 96 * 8, 96 * 8, 11, 3, -5, -1, 1, 8),         # 11 window rows: two blocks of window rows
@@ -67,11 +67,11 @@ def test_window_projection_matches_the_oracle(oracle, gu, px, h, w, rows, cols, 
     offsets = _window(px, rows, cols, dy0, dx0, channels, map_elems=(h // channels) // 4 * 4)
     C = _dia(oracle, rng, h, w, offsets)
     A, B = _operands(rng, C, batch)
-    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_WALK, "window beta0")
-    assert ran == _lib.PATH_WALK and _last_kernel().startswith("dd2dia_window_kernel<%d," % cols)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_WINDOW, "window beta0")
+    assert ran == _lib.PATH_WINDOW and _last_kernel().startswith("dd2dia_window_kernel<%d," % cols)
     C.vals[oracle.valid_mask(C)] = rng.uniform(-1, 1, int(oracle.valid_mask(C).sum())).astype(np.float32)
-    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0 / batch, 0.9, _lib.PATH_WALK, "window scaled")
-    assert ran == _lib.PATH_WALK
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0 / batch, 0.9, _lib.PATH_WINDOW, "window scaled")
+    assert ran == _lib.PATH_WINDOW
 
 
 def test_window_projection_with_padded_operands_and_a_table_in_descending_order(oracle, gu):
@@ -92,10 +92,10 @@ def test_window_projection_with_padded_operands_and_a_table_in_descending_order(
     Bd = torch.full((batch + 2, ldb), float("nan"), dtype=torch.float32, device="cuda:0")
     Ad[1:batch + 1, :n] = D.to_device_colmajor(A)
     Bd[1:batch + 1, :n] = D.to_device_colmajor(B)
-    L.cuvdia_set_path(_lib.PATH_WALK)
+    L.cuvdia_set_path(_lib.PATH_WINDOW)
     try:
         D.densedense_to_dia(Cd, D.dev_block_descriptor_f(Cd), Ad[1:batch + 1, :n], Bd[1:batch + 1, :n], 0.5, 0.0)
-        assert L.cuvdia_last_path() == _lib.PATH_WALK
+        assert L.cuvdia_last_path() == _lib.PATH_WINDOW
     finally:
         L.cuvdia_set_path(_lib.PATH_AUTO)
     got = Cd.pull()
@@ -116,8 +116,8 @@ def test_non_finite_values_stay_in_the_slots_that_use_them(oracle, gu):
     B[2 * px + 40, 6] = np.nan
     B[0, 0] = np.inf
     A[n - 1, batch - 1] = -np.inf
-    got, ran = gu.gpu_dd2dia(C, A, B, 1.0, 0.0, _lib.PATH_WALK)
-    assert ran == _lib.PATH_WALK
+    got, ran = gu.gpu_dd2dia(C, A, B, 1.0, 0.0, _lib.PATH_WINDOW)
+    assert ran == _lib.PATH_WINDOW
     with np.errstate(invalid="ignore", over="ignore"):
         ref = oracle.dd2dia(C, A, B, 1.0, 0.0)
     valid = oracle.valid_mask(C)
@@ -138,7 +138,7 @@ def test_the_choice_by_size_and_the_refusals(oracle, gu):
     C = _dia(oracle, rng, n, n, _window(px, 5, 5, -2, -2))
     A, B = _operands(rng, C, batch)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_AUTO, "taken by size")
-    assert ran == _lib.PATH_WALK and _last_kernel().startswith("dd2dia_window_kernel<5,")
+    assert ran == _lib.PATH_WINDOW and _last_kernel().startswith("dd2dia_window_kernel<5,")
     # as many tiles of a 3 x 3 window at a small batch: not taken
     C = _dia(oracle, rng, n, n, _window(px, 3, 3, -1, -1))
     A, B = _operands(rng, C, batch)
@@ -150,14 +150,14 @@ def test_the_choice_by_size_and_the_refusals(oracle, gu):
     A, B = _operands(rng, C, batch)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_AUTO, "left alone")
     assert ran == _lib.PATH_TILED and _last_kernel().startswith("dd2dia_tiled_kernel")
-    # forced on what it does not serve: a batch that is no multiple of 4, a period that is none, no window table
-    for offsets, b in ((_window(256, 3, 3, -1, -1), 6), (_window(254, 3, 3, -1, -1), 8), ([-5, -1, 0, 1, 9], 8)):
+    # forced on what it does not serve: window rows of 9 diagonals, a period that is no multiple of 4, no window table
+    for offsets, b in ((_window(256, 2, 9, -1, -4), 8), (_window(254, 3, 3, -1, -1), 8), ([-5, -1, 0, 1, 9], 8)):
         C = _dia(oracle, rng, n, n, offsets)
         A, B = _operands(rng, C, b)
         Cd = gu.make_dev_dia(C)
         from cuv_amd import dia as D
         Ad, Bd = D.to_device_colmajor(A), D.to_device_colmajor(B)
-        L.cuvdia_set_path(_lib.PATH_WALK)
+        L.cuvdia_set_path(_lib.PATH_WINDOW)
         try:
             with pytest.raises(_lib.CuvDiaError) as err:
                 D.densedense_to_dia(Cd, D.dev_block_descriptor_f(Cd), Ad, Bd, 1.0, 0.0)
