@@ -50,6 +50,8 @@ def lib():
     L.cuvdia_plan_walk.argtypes = [ip, c_int, c_int, c_int, ip, ip, ip, ip]
     L.cuvdia_plan_walk_launch.argtypes = [ip, c_int, c_int, c_int, c_int, c_int, c_int]
     L.cuvdia_plan_walk_launch.restype = c_ll
+    L.cuvdia_plan_window_launch.argtypes = [ip, c_int, c_int, c_int, c_int, c_int]
+    L.cuvdia_plan_window_launch.restype = c_ll
     L.cuvdia_last_kernel.argtypes = []
     L.cuvdia_last_kernel.restype = ctypes.c_char_p
     L.cuvdia_desc_create.argtypes = [ctypes.POINTER(c_vp), ip, c_int, c_int, c_int, c_int, c_int]

@@ -213,6 +213,33 @@ long long cuvdia_plan_walk_launch(const int *offsets_host, int nd, int stride, i
     return workgroups;
 }
 
+long long cuvdia_plan_window_launch(const int *offsets_host, int nd, int stride, int h, int w, int batch)
+{
+    if (!offsets_host || nd < 1 || batch < 0) return CUVDIA_EINVAL;
+    if (const int rc = validate_shape(offsets_host, nd, h, w, stride, 1)) return rc;
+    WalkPlan wp;
+    DiaView view{};
+    try {
+        const std::vector<Chunk> chunks = plan_chunks(offsets_host, nd, false, SP_CHUNK_MAX);
+        plan_walk(chunks, stride, false, wp);
+        const std::vector<Chunk> cp = plan_chunks(offsets_host, nd, false, CHUNK_MAX);
+        view.max_len_p = 0;
+        for (const Chunk &c : cp) view.max_len_p = std::max(view.max_len_p, c.len);
+    } catch (const std::bad_alloc &) {
+        return CUVDIA_ENOMEM;
+    }
+    if (!wp.ok || batch < 1) return 0;
+    // the conditions of the automatic choice in cuvdia_dd2dia_f32, for packed operands
+    static const int not_null = 0;          // the planner only asks whether the table is a window table
+    bool rows4 = true;
+    for (int r : wp.group_rows) rows4 = rows4 && r % 4 == 0;
+    view.h = h; view.w = w; view.nd = nd; view.stride = stride; view.rf = 1;
+    view.walk_n = WalkView{&not_null, wp.ngroups, wp.period, wp.s0, wp.k, wp.lck, wp.astep4, rows4};
+    if (!dd2dia_tiled_ok(view, h, w, batch)) return 0;
+    const long long workgroups = dd2dia_window_workgroups(view, batch);
+    return workgroups > 0 && dd2dia_window_by_size(view, batch, workgroups) ? workgroups : 0;
+}
+
 int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap)
 {
     if (!offsets_host || nd < 1) return CUVDIA_EINVAL;

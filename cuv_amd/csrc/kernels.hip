@@ -2916,6 +2916,18 @@ long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn, int *t
     return total;
 }
 
+// Whether the automatic choice takes the window-table projection.  By size: the tiles must fill the chip (four
+// workgroups per CU) -- the smaller the window, the less a tile saves over the chunk-by-chunk kernel and the more
+// tiles it takes (measured on 7 x 7, 5 x 5 and 3 x 3 windows of maps 256 to 1024 wide at batch 32 to 512: ahead
+// from 768, 1024 and 1536 tiles on, the 3 x 3 only from batch 128) -- and maps narrower than a tile's 64
+// positions would leave lanes idle.
+bool dd2dia_window_by_size(const DiaView &C, int batch, long long workgroups)
+{
+    const int slots = C.walk_n.k * C.walk_n.lck;
+    const long long min_wgs = slots >= 49 ? DW_MIN_WGS : slots >= 25 ? DW_MIN_WGS * 4 / 3 : DW_MIN_WGS * 2;
+    return workgroups >= min_wgs && C.walk_n.period >= 64 && (slots >= 25 || batch >= 128);
+}
+
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
                                const float *B, long long ldb, int batch,
                                float alpha, float beta, hipStream_t stream, int window, bool *windowed)
@@ -2924,14 +2936,7 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     if (window >= 0) {
         int txn = 0, tyn = 0, ndb = 0;
         const long long wgs = dd2dia_window_workgroups(C, batch, &txn, &tyn, &ndb);
-        // By size: the tiles must fill the chip (four workgroups per CU) -- the smaller the window, the less a tile
-        // saves over the chunk-by-chunk kernel and the more tiles it takes (measured on 7 x 7, 5 x 5 and 3 x 3
-        // windows of maps 256 to 1024 wide at batch 32 to 512: ahead from 768, 1024 and 1536 tiles on, the 3 x 3 only
-        // from batch 128) -- and maps narrower than a tile's 64 positions would leave lanes idle.
-        const int slots = C.walk_n.k * C.walk_n.lck;
-        const long long min_wgs = slots >= 49 ? DW_MIN_WGS : slots >= 25 ? DW_MIN_WGS * 4 / 3 : DW_MIN_WGS * 2;
-        const bool by_size = wgs >= min_wgs && C.walk_n.period >= 64 && (slots >= 25 || batch >= 128);
-        if (wgs > 0 && (window > 0 || by_size)) {
+        if (wgs > 0 && (window > 0 || dd2dia_window_by_size(C, batch, wgs))) {
             const WalkView &wk = C.walk_n;
             const DwLaunch L{wk.tab_dev, wk.ngroups, wk.k, wk.period, wk.s0, wk.astep4 / 4, wk.lck, vals, A, lda, B, ldb,
                              C.h, C.w, batch, alpha, beta,

@@ -117,6 +117,8 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
                                float alpha, float beta, hipStream_t stream, int window = 0, bool *windowed = nullptr);
 // Workgroups of the window-table projection for these operands (0: it does not apply).
 long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn = nullptr, int *tyn = nullptr, int *ndb = nullptr);
+// Whether the automatic choice takes that kernel for a launch of so many workgroups.
+bool dd2dia_window_by_size(const DiaView &C, int batch, long long workgroups);
 
 // The allocation-free entry point keeps its device tables in a static device
 // array instead of a descriptor's allocation: the offset table at byte 0 (up

@@ -115,6 +115,20 @@ int cuvdia_plan_chunks(const int *offsets_host, int nd, int transposed,
  * the block list built in src/cuv/matrix_ops/densedense_to_sparse.cu:123-171. */
 int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap);
 
+/* Pure host function: does the automatic choice of cuvdia_dd2dia_f32 run the
+ * kernel tiled in the window's plane for an h x w matrix with this table
+ * (row_fact 1) and `batch` packed dense columns?  Returns the number of
+ * workgroups of that launch (tiles of 4 x 64 positions x blocks of 8 window
+ * rows x channel groups), or 0 when the chunk-by-chunk kernel serves: the
+ * table is no window table (see cuvdia_plan_walk) of chunks of 2 to 8
+ * diagonals, the period, a channel distance or a row count is no multiple of
+ * 4, the period is below 64, or the launch has too few workgroups to fill
+ * the chip (768 for windows of 49 slots or more, 1024 from 25 slots, 1536 --
+ * and a batch of at least 128 -- below).  Negative: an error.
+ * cuvdia_set_path(CUVDIA_PATH_WINDOW) waives the conditions on the period's
+ * size, the workgroups and the batch.  No counterpart in the reference. */
+long long cuvdia_plan_window_launch(const int *offsets_host, int nd, int stride, int h, int w, int batch);
+
 /* Pure host function: is the offset table a *window table* -- k window rows of
  * lck consecutive offsets, `period` rows apart, repeated for every one of
  * ngroups groups (channel shifts); the pattern filter_factory builds

@@ -303,3 +303,45 @@ def test_walk_launch_depends_on_the_shape_too():
     # argument errors
     assert _walk_launch(offs, n, n, n, -1) == _lib.EINVAL
     assert _walk_launch(offs, n - 8, n, n, 128) < 0          # stride shorter than the diagonals
+
+
+def _window_launch(offs, stride, h, w, batch):
+    from cuv_amd import _lib
+    offs = np.ascontiguousarray(offs, np.int32)
+    ip = ctypes.POINTER(ctypes.c_int)
+    return _lib.lib().cuvdia_plan_window_launch(offs.ctypes.data_as(ip), offs.size, stride, h, w, batch)
+
+
+def test_window_projection_launch_by_table_shape_and_size():
+    """The projection tiled in the window's plane: tiles of 4 x 64 positions, taken from 768 (49 slots), 1024
+    (25 slots) or 1536 tiles and batch 128 (fewer slots) on; period, channel distances and row counts multiples
+    of 4; chunks of 2 to 8 diagonals."""
+    from cuv_amd import _lib, workloads as W
+    n = 512 * 512
+    offs = W.window_offsets(512, 7)
+    assert _window_launch(offs, n, n, n, 128) == 8 * 128            # 8 tile columns x 128 tile rows
+    assert _window_launch(offs, n, n, n, 3) == 8 * 128              # any batch
+    assert _window_launch(offs, n, n - 4, n - 8, 128) == 8 * 128    # row counts multiples of 4
+    assert _window_launch(offs, n, n - 2, n, 128) == 0
+    assert _window_launch(offs, n, n, n - 6, 128) == 0
+    # 448-wide map: 7 x 112 = 784 tiles -- taken; 384-wide: 576 -- left to the chunk-by-chunk kernel
+    assert _window_launch(W.window_offsets(448, 7), 448 * 448, 448 * 448, 448 * 448, 64) == 784
+    assert _window_launch(W.window_offsets(384, 7), 384 * 384, 384 * 384, 384 * 384, 64) == 0
+    # 5 x 5 from 1024 tiles, 3 x 3 from 1536 and batch 128
+    assert _window_launch(W.window_offsets(448, 5), 448 * 448, 448 * 448, 448 * 448, 64) == 0
+    assert _window_launch(W.window_offsets(512, 5), n, n, n, 64) == 1024
+    assert _window_launch(W.window_offsets(512, 3), n, n, n, 512) == 0
+    assert _window_launch(W.window_offsets(640, 3), 640 * 640, 640 * 640, 640 * 640, 128) == 10 * 160
+    assert _window_launch(W.window_offsets(640, 3), 640 * 640, 640 * 640, 640 * 640, 64) == 0
+    # four channels of a 256-wide map: 4 tile columns x 256 tile rows x 4 groups
+    offs4 = W.window_offsets(256, 7, 4)
+    assert _window_launch(offs4, 4 * 256 * 256, 4 * 256 * 256, 4 * 256 * 256, 32) == 4 * 256 * 4
+    # 13 window rows: two blocks of window rows per tile -- but 13 diagonals per row are not served
+    assert _window_launch(W.window_offsets(512, 13), n, n, n, 128) == 0
+    tall = [dy * 512 + dx for dy in range(-6, 7) for dx in range(-3, 4)]
+    assert _window_launch(tall, n, n, n, 128) == 2 * 8 * 128
+    # a period that is no multiple of 4; no window table; the headline layer (64 tiles)
+    assert _window_launch(W.window_offsets(510, 7), 510 * 510, 510 * 510, 510 * 510, 128) == 0
+    assert _window_launch([-5, -1, 0, 1, 9], n, n, n, 128) == 0
+    assert _window_launch(W.window_offsets(128, 7), 128 * 128, 128 * 128, 128 * 128, 128) == 0
+    assert _lib.lib().cuvdia_plan_window_launch(None, 3, 16, 16, 16, 8) == _lib.EINVAL
