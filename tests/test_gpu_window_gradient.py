@@ -164,3 +164,69 @@ def test_the_choice_by_size_and_the_refusals(oracle, gu):
         finally:
             L.cuvdia_set_path(_lib.PATH_AUTO)
         assert err.value.code == _lib.EUNSUPPORTED
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_window_shapes(oracle, gu, seed):
+    """Seeded window tables nobody picked by hand: period, window, first shift, channel groups, row counts and batch
+    drawn at random within what the kernel serves."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(1000 + seed)
+    px = 4 * int(rng.integers(16, 50))
+    rows, cols = int(rng.integers(2, 12)), int(rng.integers(2, 9))
+    dy0, dx0 = -int(rng.integers(0, rows)), -int(rng.integers(0, cols))
+    channels = int(rng.choice([1, 1, 2, 3]))
+    map_rows = rows + int(rng.integers(4, 12))
+    map_elems = px * map_rows
+    h = channels * map_elems - 4 * int(rng.integers(0, 3))
+    w = channels * map_elems - 4 * int(rng.integers(0, 3))
+    batch = int(rng.choice([1, 3, 4, 7, 8, 17, 32]))
+    C = _dia(oracle, rng, h, w, _window(px, rows, cols, dy0, dx0, channels, map_elems))
+    A, B = _operands(rng, C, batch)
+    alpha, beta = float(rng.choice([1.0, -0.5, 1.0 / batch])), float(rng.choice([0.0, 0.9, -1.5]))
+    _, ran = gu.check_dd2dia(oracle, C, A, B, alpha, beta, _lib.PATH_WINDOW, "random window %d" % seed)
+    assert ran == _lib.PATH_WINDOW
+
+
+def test_a_sweep_size_against_sampled_exact_sums_and_the_chunk_kernel(gu):
+    """512 x 512 map, 7 x 7 window, batch 32 -- a size the automatic choice gives to this kernel and the oracle
+    would take minutes for: 4000 stored slots drawn at random are compared with their sums in fp64, the padding
+    slots must keep their NaN, and the whole result must lie within rounding of the chunk-by-chunk kernel's."""
+    import torch
+    from cuv_amd import _lib, dia as D, workloads as W
+    rng = np.random.default_rng(7)
+    px, batch = 512, 32
+    n = px * px
+    offs = W.window_offsets(px, 7)
+    A = np.asfortranarray(rng.uniform(-1, 1, (n, batch)).astype(np.float32))
+    B = np.asfortranarray(rng.uniform(-1, 1, (n, batch)).astype(np.float32))
+    Ad, Bd = D.to_device_colmajor(A), D.to_device_colmajor(B)
+    L = _lib.lib()
+    results = {}
+    for path in (_lib.PATH_AUTO, _lib.PATH_TILED_NOWALK):
+        C = D.dev_dia_matrix_f(n, n, len(offs), n, 1, device="cuda:0")
+        C.set_offsets(offs)
+        C.vec.fill_(float("nan"))
+        L.cuvdia_set_path(path)
+        try:
+            D.densedense_to_dia(C, D.dev_block_descriptor_f(C), Ad, Bd, 0.5, 0.0)
+            ran = L.cuvdia_last_path()
+        finally:
+            L.cuvdia_set_path(_lib.PATH_AUTO)
+        results[path] = (C.pull().reshape(len(offs), n), ran)
+    got, ran = results[_lib.PATH_AUTO]
+    assert ran == _lib.PATH_WINDOW
+    other, ran = results[_lib.PATH_TILED_NOWALK]
+    assert ran == _lib.PATH_TILED
+    i = np.arange(n)
+    valid = np.stack([(i + k >= 0) & (i + k < n) for k in offs])
+    assert np.isnan(got[~valid]).all() and np.isfinite(got[valid]).all()
+    # every term is below 1 in magnitude: 1e-5 of the batch bounds 1e-5 of the sum of |terms|
+    assert np.abs(got[valid] - other[valid]).max() <= 1e-5 * 0.5 * batch
+    d = rng.integers(0, len(offs), 4000)
+    r = rng.integers(0, n, 4000)
+    keep = valid[d, r]
+    d, r = d[keep], r[keep]
+    exact = 0.5 * np.einsum("ij,ij->i", A[r].astype(np.float64), B[r + offs[d]].astype(np.float64))
+    mag = 0.5 * np.einsum("ij,ij->i", np.abs(A[r]).astype(np.float64), np.abs(B[r + offs[d]]).astype(np.float64))
+    assert (np.abs(got[d, r] - exact) <= 1e-5 * mag + 1e-30).all()
