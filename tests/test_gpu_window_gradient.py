@@ -230,3 +230,45 @@ def test_a_sweep_size_against_sampled_exact_sums_and_the_chunk_kernel(gu):
     exact = 0.5 * np.einsum("ij,ij->i", A[r].astype(np.float64), B[r + offs[d]].astype(np.float64))
     mag = 0.5 * np.einsum("ij,ij->i", np.abs(A[r]).astype(np.float64), np.abs(B[r + offs[d]]).astype(np.float64))
     assert (np.abs(got[d, r] - exact) <= 1e-5 * mag + 1e-30).all()
+
+
+def test_window_projection_under_graph_capture_and_replay(oracle, gu):
+    """The kernel recorded into a HIP graph and replayed with the program's own eager work between the replays:
+    every replay equals the eager result (beta != 0: the destination is restored before each replay)."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    rng = np.random.default_rng(12)
+    px, n, batch = 64, 64 * 12, 20
+    C = _dia(oracle, rng, n, n, _window(px, 5, 5, -2, -2))
+    A, B = _operands(rng, C, batch)
+    Ad, Bd = D.to_device_colmajor(A), D.to_device_colmajor(B)
+    L = _lib.lib()
+    L.cuvdia_set_path(_lib.PATH_WINDOW)
+    try:
+        Ce = gu.make_dev_dia(C)
+        start = Ce.vec.clone()
+        D.densedense_to_dia(Ce, D.dev_block_descriptor_f(Ce), Ad, Bd, 0.25, 0.9)
+        assert L.cuvdia_last_path() == _lib.PATH_WINDOW
+        eager = Ce.vec.clone()
+        Cg = gu.make_dev_dia(C)
+        bd = D.dev_block_descriptor_f(Cg)
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            D.densedense_to_dia(Cg, bd, Ad, Bd, 0.25, 0.9, sync=False)      # warm-up on a side stream
+        torch.cuda.current_stream().wait_stream(s)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            D.densedense_to_dia(Cg, bd, Ad, Bd, 0.25, 0.9, sync=False)
+        for rep in range(3):
+            Cg.vec.copy_(start)
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(Cg.vec.view(torch.int32), eager.view(torch.int32)), "replay %d differs from the eager call" % rep
+    finally:
+        L.cuvdia_set_path(_lib.PATH_AUTO)
+    ref = oracle.dd2dia(C, A, B, 0.25, 0.9)
+    valid = oracle.valid_mask(C)
+    mag = oracle.dd2dia_f64(type(C)(C.h, C.w, C.offsets, C.stride, C.rf, np.abs(C.vals)), np.abs(A), np.abs(B), 0.25, 0.9)
+    gu.assert_close_mag(eager.cpu().numpy()[valid], ref[valid], mag[valid], "eager")
