@@ -2301,8 +2301,11 @@ __device__ __forceinline__ void dw_ring(F &body, int gi, int n)
     }
 }
 
-template <int LC, int SH>
-__global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
+// SUBS: the batch is cut into SUBS ranges of whole groups, each worked by 4 waves of the workgroup's 4 SUBS with
+// staging buffers of their own (launches of few tiles: 2 or 4 ranges keep 16 waves on every CU where one
+// range per tile would leave most of the chip idle).  The ranges' sums meet in LDS at the end, in range order.
+template <int LC, int SH, int SUBS>
+__global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
     const int *__restrict__ tab,            // group_rows[ngroups], then 4 * element offset of chunk (g, dy)'s first slot
     int ngroups, int K, int period, int s0, int astep, float *__restrict__ C,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
@@ -2311,9 +2314,13 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
 {
     typedef DwShape<LC, SH> S;
     constexpr int WAVES = S::WAVES, COLS = S::COLS, DYB = S::DYB, WQ = S::WQ, BPR = S::BPR, NIT = S::NIT;
-    __shared__ __attribute__((aligned(16))) float lds[S::NBUF][S::BUF_PIECES * 4];
+    static_assert(SUBS == 1 || SUBS == 2 || SUBS == 4, "batch ranges per workgroup");
+    __shared__ __attribute__((aligned(16))) float lds_all[SUBS][S::NBUF][S::BUF_PIECES * 4];
+    static_assert((SUBS - 1) * WAVES * 4 * LC * 64 <= SUBS * S::NBUF * S::BUF_PIECES * 4, "the ranges' sums fit the staging buffers");
     const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sub = wave_all / WAVES, wave = wave_all % WAVES;      // batch range, wave within it
+    float (*lds)[S::BUF_PIECES * 4] = lds_all[sub];
     typedef const int __attribute__((address_space(4))) *sc_int_ptr;
     const sc_int_ptr stab = (sc_int_ptr)tab;
 
@@ -2338,6 +2345,9 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
     const int npb = COLS * nbr * BPR;
     const int nib = (npb + 63) / 64;
     const int ni = nib + S::A_PIECES / 64;
+    // groups per batch range (the same for every range: a range that ends past the batch works on zeros there)
+    const int ngr = ((batch + COLS - 1) / COLS + SUBS - 1) / SUBS;
+    const int col_first = sub * ngr * COLS;
     unsigned v_lane[NIT];
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
@@ -2348,16 +2358,17 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
             const int col = p / (nbr * BPR), rem = p - col * (nbr * BPR);
             const int row = rem / BPR, pc = rem - row * BPR;
             const int idx = b_tile + row * period + 4 * pc;
-            if ((p < npb) & (idx >= 0) & (idx + 4 <= w)) v = (unsigned)(col * (int)ldb + idx) * 4u;
+            if ((p < npb) & (idx >= 0) & (idx + 4 <= w)) v = (unsigned)((col_first + col) * (int)ldb + idx) * 4u;
         } else if (s < ni) {
             const int col = s - nib, row = lane >> 4, pc = lane & 15;
             const int idx = i_tile + row * period + 4 * pc;
-            if (idx + 4 <= h) v = (unsigned)(col * (int)lda + idx) * 4u;
+            if (idx + 4 <= h) v = (unsigned)((col_first + col) * (int)lda + idx) * 4u;
         }
         v_lane[it] = v;
     }
     const sp_int4 bq = raw_rsrc(B, b_bytes), aq = raw_rsrc(A, a_bytes);
-    const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
+    const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds_all[0][0][0] +
+                          (unsigned)sub * (S::NBUF * S::BUF_PIECES * 16u);
     constexpr unsigned BUF_BYTES = S::BUF_PIECES * 16u;
     const unsigned b_step = (unsigned)ldb * (4u * COLS), a_step = (unsigned)lda * (4u * COLS);    // bytes per group
     // Requests the next group into buffer `par` and moves the lane's offsets one group on.  (An offset that is
@@ -2441,9 +2452,8 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
     // The ring: group gi is applied out of buffer gi mod NBUF while the groups up to gi + NBUF - 1 are in flight or
     // landed.  At a group's end everything but the requests of the groups after the next has to have arrived: this
     // wave's share of a group is n_mine instructions, and they complete in order.
-    // (the columns of a last, partial group past the batch start a whole column past the last one: out of the
-    // resources' range, they arrive as zeros and add nothing)
-    const int ngr = (batch + COLS - 1) / COLS;
+    // (columns past the batch start a whole column past the last one: out of the resources' range, they arrive
+    // as zeros and add nothing)
     const int n_mine = (ni - wave + WAVES - 1) / WAVES;
     auto wait_leaving_groups = [&](int groups) __attribute__((always_inline)) {
         switch (groups * n_mine) {
@@ -2473,6 +2483,36 @@ __global__ __launch_bounds__(256, 4) void dd2dia_window_kernel(
     };
 #pragma clang loop unroll(disable)
     for (int gi = 0; gi < ngr; gi += NBUF) dw_ring<NBUF, 0>(body, gi, ngr);
+
+    // The ranges' sums meet: half of them at a time (one of a lane's two window rows), ranges 1 .. SUBS - 1 write,
+    // range 0 adds them in range order.  (Every wave has passed the loop's last barrier: the buffers are free.)
+    if constexpr (SUBS > 1) {
+        float *red = &lds_all[0][0][0];
+        constexpr int PER_WAVE = 4 * LC * 64;
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            if (sub > 0) {
+                float *dst = red + ((sub - 1) * WAVES + wave) * PER_WAVE + lane;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int j = 0; j < LC; ++j) dst[(t * LC + j) * 64] = acc[n][t][j];
+            }
+            __syncthreads();
+            if (sub == 0) {
+#pragma unroll
+                for (int r = 1; r < SUBS; ++r) {
+                    const float *src = red + ((r - 1) * WAVES + wave) * PER_WAVE + lane;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+#pragma unroll
+                        for (int j = 0; j < LC; ++j) acc[n][t][j] += src[(t * LC + j) * 64];
+                }
+            }
+            __syncthreads();
+        }
+        if (sub > 0) return;
+    }
 
     // Results: 4 consecutive rows of every slot per lane, one 16-byte store where all four exist.
     typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -2620,6 +2660,7 @@ struct DwLaunch {
     float alpha, beta;
     unsigned a_bytes, b_bytes, c_bytes;
     int txn, tyn, ndb;
+    int subs;                   // batch ranges per workgroup: 1, 2 or 4
     hipStream_t stream;
 };
 hipError_t dd2dia_window_launch(const DwLaunch &L);
@@ -2712,20 +2753,27 @@ hipError_t dd2dia_window_launch(const DwLaunch &L)
     const int sh = ((L.s0 % 4) + 4) % 4;
 #define CUVDIA_DW_ARGS L.tab, L.ngroups, L.k, L.period, L.s0, L.astep, L.vals, L.A, L.lda, L.B, L.ldb, L.h, L.w, L.batch, \
                        L.alpha, L.beta, L.a_bytes, L.b_bytes, L.c_bytes, L.txn, L.tyn, L.ndb
+#define CUVDIA_DW_LAUNCH_SUBS(LC, SUBS)                                                                               \
+    do {                                                                                                              \
+        if (sh == 0) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 0, SUBS>), grid, dim3(256 * SUBS), 0, L.stream, CUVDIA_DW_ARGS); \
+        else if (sh == 1) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 1, SUBS>), grid, dim3(256 * SUBS), 0, L.stream, CUVDIA_DW_ARGS); \
+        else if (sh == 2) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 2, SUBS>), grid, dim3(256 * SUBS), 0, L.stream, CUVDIA_DW_ARGS); \
+        else hipLaunchKernelGGL((dd2dia_window_kernel<LC, 3, SUBS>), grid, dim3(256 * SUBS), 0, L.stream, CUVDIA_DW_ARGS); \
+    } while (0)
 #define CUVDIA_DW_LAUNCH(LC)                                                                                          \
     case LC:                                                                                                          \
-        if (sh == 0) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 0>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS); \
-        else if (sh == 1) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 1>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS); \
-        else if (sh == 2) hipLaunchKernelGGL((dd2dia_window_kernel<LC, 2>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS); \
-        else hipLaunchKernelGGL((dd2dia_window_kernel<LC, 3>), grid, dim3(256), 0, L.stream, CUVDIA_DW_ARGS);        \
+        if (L.subs == 4) CUVDIA_DW_LAUNCH_SUBS(LC, 4);                                                                \
+        else if (L.subs == 2) CUVDIA_DW_LAUNCH_SUBS(LC, 2);                                                           \
+        else CUVDIA_DW_LAUNCH_SUBS(LC, 1);                                                                            \
         break;
-    note_kernel("dd2dia_window_kernel<%d, %d>", L.lck, sh);
+    note_kernel("dd2dia_window_kernel<%d, %d, %d>", L.lck, sh, L.subs);
     switch (L.lck) {
         CUVDIA_DW_LAUNCH(2) CUVDIA_DW_LAUNCH(3) CUVDIA_DW_LAUNCH(4) CUVDIA_DW_LAUNCH(5)
         CUVDIA_DW_LAUNCH(6) CUVDIA_DW_LAUNCH(7) CUVDIA_DW_LAUNCH(8)
         default: return hipErrorNotSupported;
     }
 #undef CUVDIA_DW_LAUNCH
+#undef CUVDIA_DW_LAUNCH_SUBS
 #undef CUVDIA_DW_ARGS
     return hipGetLastError();
 }
@@ -2916,16 +2964,30 @@ long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn, int *t
     return total;
 }
 
-// Whether the automatic choice takes the window-table projection.  By size: the tiles must fill the chip (four
-// workgroups per CU) -- the smaller the window, the less a tile saves over the chunk-by-chunk kernel and the more
-// tiles it takes (measured on 7 x 7, 5 x 5 and 3 x 3 windows of maps 256 to 1024 wide at batch 32 to 512: ahead
-// from 768, 1024 and 1536 tiles on, the 3 x 3 only from batch 128) -- and maps narrower than a tile's 64
-// positions would leave lanes idle.
+// Batch ranges per workgroup the window-table projection runs with on a launch of so many workgroups (tiles):
+// 1 when the tiles alone fill the chip (four workgroups of 4 waves per CU), 2 or 4 when it takes that many ranges
+// of the batch per tile to get there.  The smaller the window, the less a tile saves over the chunk-by-chunk
+// kernel and the more tiles it takes (measured on 7 x 7, 5 x 5 and 3 x 3 windows of maps 256 to 1024 wide at
+// batch 32 to 512: ahead from 768, 1024 and 1536 tiles on, the 3 x 3 only from batch 128).
+int dd2dia_window_subs(const DiaView &C, long long workgroups)
+{
+    const int slots = C.walk_n.k * C.walk_n.lck;
+    const long long min_wgs = slots >= 49 ? DW_MIN_WGS : slots >= 25 ? DW_MIN_WGS * 4 / 3 : DW_MIN_WGS * 2;
+    return workgroups >= min_wgs ? 1 : 2 * workgroups >= min_wgs ? 2 : 4;
+}
+// Whether the automatic choice takes the window-table projection: enough tiles to fill the chip and a map no
+// narrower than a tile's 64 positions (lanes would idle).  With 2 or 4 batch ranges per tile only windows of 49
+// slots or more, and two ranges only from batch 512 on: a 7 x 7 window on a 256-wide map (256 tiles, 4 ranges)
+// measured 1.2 - 1.5 times the chunk-by-chunk kernel's rate at batch 32 to 2048, on 320- and 384-wide maps (400 and
+// 576 tiles, 2 ranges) 1.1 - 1.6 times from batch 512 and 0.86 - 0.98 below; 5 x 5 windows on those maps 0.6 - 1.0.
 bool dd2dia_window_by_size(const DiaView &C, int batch, long long workgroups)
 {
     const int slots = C.walk_n.k * C.walk_n.lck;
     const long long min_wgs = slots >= 49 ? DW_MIN_WGS : slots >= 25 ? DW_MIN_WGS * 4 / 3 : DW_MIN_WGS * 2;
-    return workgroups >= min_wgs && C.walk_n.period >= 64 && (slots >= 25 || batch >= 128);
+    const int subs = dd2dia_window_subs(C, workgroups);
+    if (subs * workgroups < min_wgs || C.walk_n.period < 64) return false;
+    if (subs == 1) return slots >= 25 || batch >= 128;
+    return slots >= 49 && batch >= (subs == 2 ? 512 : 32);
 }
 
 hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, long long lda,
@@ -2942,7 +3004,8 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
                              C.h, C.w, batch, alpha, beta,
                              (unsigned)((((long long)batch - 1) * lda + C.h) * 4),
                              (unsigned)((((long long)batch - 1) * ldb + C.w) * 4),
-                             (unsigned)((long long)C.nd * C.stride * 4), txn, tyn, ndb, stream};
+                             (unsigned)((long long)C.nd * C.stride * 4), txn, tyn, ndb,
+                             dd2dia_window_subs(C, wgs), stream};
             if (windowed) *windowed = true;
             return dd2dia_window_launch(L);
         }

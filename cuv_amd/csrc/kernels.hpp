@@ -119,6 +119,8 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
 long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn = nullptr, int *tyn = nullptr, int *ndb = nullptr);
 // Whether the automatic choice takes that kernel for a launch of so many workgroups.
 bool dd2dia_window_by_size(const DiaView &C, int batch, long long workgroups);
+// Batch ranges per workgroup (1, 2 or 4) of such a launch.
+int dd2dia_window_subs(const DiaView &C, long long workgroups);
 
 // The allocation-free entry point keeps its device tables in a static device
 // array instead of a descriptor's allocation: the offset table at byte 0 (up

@@ -123,8 +123,10 @@ int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap
  * table is no window table (see cuvdia_plan_walk) of chunks of 2 to 8
  * diagonals, the period, a channel distance or a row count is no multiple of
  * 4, the period is below 64, or the launch has too few workgroups to fill
- * the chip (768 for windows of 49 slots or more, 1024 from 25 slots, 1536 --
- * and a batch of at least 128 -- below).  Negative: an error.
+ * the chip: 768 for windows of 49 slots or more -- or 384 at a batch of at
+ * least 512, or 192 at a batch of at least 32: a workgroup then works two or
+ * four ranges of the batch side by side --, 1024 from 25 slots, 1536 and a
+ * batch of at least 128 below.  Negative: an error.
  * cuvdia_set_path(CUVDIA_PATH_WINDOW) waives the conditions on the period's
  * size, the workgroups and the batch.  No counterpart in the reference. */
 long long cuvdia_plan_window_launch(const int *offsets_host, int nd, int stride, int h, int w, int batch);

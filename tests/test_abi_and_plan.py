@@ -313,9 +313,9 @@ def _window_launch(offs, stride, h, w, batch):
 
 
 def test_window_projection_launch_by_table_shape_and_size():
-    """The projection tiled in the window's plane: tiles of 4 x 64 positions, taken from 768 (49 slots), 1024
-    (25 slots) or 1536 tiles and batch 128 (fewer slots) on; period, channel distances and row counts multiples
-    of 4; chunks of 2 to 8 diagonals."""
+    """The projection tiled in the window's plane: tiles of 4 x 64 positions, taken from 768 (49 slots; fewer with
+    two or four batch ranges per tile), 1024 (25 slots) or 1536 tiles and batch 128 (fewer slots) on; period,
+    channel distances and row counts multiples of 4; chunks of 2 to 8 diagonals."""
     from cuv_amd import _lib, workloads as W
     n = 512 * 512
     offs = W.window_offsets(512, 7)
@@ -324,9 +324,15 @@ def test_window_projection_launch_by_table_shape_and_size():
     assert _window_launch(offs, n, n - 4, n - 8, 128) == 8 * 128    # row counts multiples of 4
     assert _window_launch(offs, n, n - 2, n, 128) == 0
     assert _window_launch(offs, n, n, n - 6, 128) == 0
-    # 448-wide map: 7 x 112 = 784 tiles -- taken; 384-wide: 576 -- left to the chunk-by-chunk kernel
+    # 448-wide map: 7 x 112 = 784 tiles -- taken; 384-wide: 576 -- with two batch ranges per tile, from batch 512;
+    # 256-wide: 256 -- with four, from batch 32; 192-wide: 144 -- left to the chunk-by-chunk kernel
     assert _window_launch(W.window_offsets(448, 7), 448 * 448, 448 * 448, 448 * 448, 64) == 784
     assert _window_launch(W.window_offsets(384, 7), 384 * 384, 384 * 384, 384 * 384, 64) == 0
+    assert _window_launch(W.window_offsets(384, 7), 384 * 384, 384 * 384, 384 * 384, 512) == 576
+    assert _window_launch(W.window_offsets(256, 7), 256 * 256, 256 * 256, 256 * 256, 32) == 256
+    assert _window_launch(W.window_offsets(256, 7), 256 * 256, 256 * 256, 256 * 256, 16) == 0
+    assert _window_launch(W.window_offsets(256, 5), 256 * 256, 256 * 256, 256 * 256, 1024) == 0
+    assert _window_launch(W.window_offsets(192, 7), 192 * 192, 192 * 192, 192 * 192, 1024) == 0
     # 5 x 5 from 1024 tiles, 3 x 3 from 1536 and batch 128
     assert _window_launch(W.window_offsets(448, 5), 448 * 448, 448 * 448, 448 * 448, 64) == 0
     assert _window_launch(W.window_offsets(512, 5), n, n, n, 64) == 1024

@@ -45,7 +45,7 @@ def test_projection_walks_a_batch_beyond_2_gib_in_slabs():
     C = new_dia(c0)
     bd = D.dev_block_descriptor_f(C)
     D.densedense_to_dia(C, bd, P, Q, alpha, beta)
-    assert L.cuvdia_last_path() == _lib.PATH_TILED, "the large batch must not fall back to the generic kernel"
+    assert L.cuvdia_last_path() in (_lib.PATH_TILED, _lib.PATH_WINDOW), "the large batch must not fall back to the generic kernel"
     got = C.vec.view(nd, n)
     assert bool(torch.isnan(got[~valid]).all()), "padding slots were written"
     assert bool(torch.isfinite(got[valid]).all()), "padding slots were read"

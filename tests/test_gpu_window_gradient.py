@@ -57,6 +57,8 @@ CASES = [
     (96, 96 * 8, 96 * 8, 11, 3, -5, -1, 1, 8),         # 11 window rows: two blocks of window rows
     (64, 64 * 16, 64 * 16, 7, 7, -3, -3, 2, 8),        # two groups (channels)
     (64, 64 * 12 - 4, 64 * 12 - 8, 5, 7, -2, -3, 1, 8),    # row counts that end inside a map row
+    (64, 64 * 1600, 64 * 1600, 7, 7, -3, -3, 1, 9),    # 400 tiles: two batch ranges per workgroup (the cases above: four)
+    (64, 64 * 3200, 64 * 3200, 7, 7, -3, -3, 1, 5),    # 800 tiles: one
 ]
 
 
@@ -69,6 +71,8 @@ def test_window_projection_matches_the_oracle(oracle, gu, px, h, w, rows, cols, 
     A, B = _operands(rng, C, batch)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_WINDOW, "window beta0")
     assert ran == _lib.PATH_WINDOW and _last_kernel().startswith("dd2dia_window_kernel<%d," % cols)
+    tiles = -(-px // 64) * -(-(-(-h // px)) // 4) * -(-rows // 8) * channels
+    assert _last_kernel().endswith(", %d>" % (1 if tiles >= 768 else 2 if tiles >= 384 else 4)) or cols != 7 or rows != 7
     C.vals[oracle.valid_mask(C)] = rng.uniform(-1, 1, int(oracle.valid_mask(C).sum())).astype(np.float32)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0 / batch, 0.9, _lib.PATH_WINDOW, "window scaled")
     assert ran == _lib.PATH_WINDOW
@@ -150,6 +154,13 @@ def test_the_choice_by_size_and_the_refusals(oracle, gu):
     A, B = _operands(rng, C, batch)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_AUTO, "left alone")
     assert ran == _lib.PATH_TILED and _last_kernel().startswith("dd2dia_tiled_kernel")
+    # 256 tiles of a 7 x 7 window at batch 32: taken with four batch ranges per workgroup
+    n = 64 * 1024
+    C = _dia(oracle, rng, n, n, _window(64, 7, 7, -3, -3))
+    A, B = _operands(rng, C, 32)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0 / 32, 0.9, _lib.PATH_AUTO, "four ranges")
+    assert ran == _lib.PATH_WINDOW and _last_kernel() == "dd2dia_window_kernel<7, 1, 4>"
+    n = 256 * 64
     # forced on what it does not serve: window rows of 9 diagonals, a period that is no multiple of 4, no window table
     for offsets, b in ((_window(256, 2, 9, -1, -4), 8), (_window(254, 3, 3, -1, -1), 8), ([-5, -1, 0, 1, 9], 8)):
         C = _dia(oracle, rng, n, n, offsets)
