@@ -22,7 +22,9 @@
 //           A chunk pair: eight sums s_q over g = q (mod 8);
 //           p_q = s_q + s_{q+4}, then total as above.
 //           C = beta*C + alpha*total.  The generic kernel and the window-table
-//           kernel sum the batch serially in ascending column order.
+//           kernel sum the batch serially in ascending column order (the latter,
+//           on launches of few tiles, as 2 or 4 ranges of the batch whose sums
+//           are added in range order).
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -2271,7 +2273,9 @@ __global__ __launch_bounds__((PAIRS && WIDE != DD_SHIFTED) ? 512 : 256) void dd2
 // whole walk up to the column step, so its byte offsets are computed once; everything, column included, goes
 // into the vector offset, which the buffer's range check covers.
 //
-// Accumulation order per slot: batch columns ascending, acc = fma(a, b, acc); C = beta*C + alpha*acc.
+// Accumulation order per slot: batch columns ascending, acc = fma(a, b, acc); C = beta*C + alpha*acc.  With
+// SUBS batch ranges per workgroup (see the kernel): p_r over range r's columns ascending, then
+// acc = ((p_0 + p_1) + p_2) + p_3.
 template <int LC, int SH>
 struct DwShape {
     static constexpr int WAVES = 4, TX = 64, DYB = 8;

@@ -256,9 +256,10 @@ int cuvdia_learn_step_weight_decay_momentum_f32(float *W_device, float *momentum
  * on `stream`, slab of columns after slab, each adding to C.
  * Summation order per slot: see kernels.hip; the kernel for large window
  * tables (cuvdia_last_path() == CUVDIA_PATH_WINDOW) adds the batch columns in
- * ascending order into one sum, the chunk-by-chunk kernel into four or eight
- * partial sums: their results differ by rounding, both within 1e-5 of the
- * sum of |terms| of the reference's host result. */
+ * ascending order into one sum (on launches of few tiles: into two or four
+ * sums over consecutive ranges of the batch), the chunk-by-chunk kernel into
+ * four or eight interleaved partial sums: their results differ by rounding,
+ * both within 1e-5 of the sum of |terms| of the reference's host result. */
 int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals_device,
                       const float *A_device, long long lda,
                       const float *B_device, long long ldb, int batch,
