@@ -292,6 +292,31 @@ TEST_CASE(locally_connected_layer)
     delete W;
 }
 
+TEST_CASE(locally_connected_layer_window_projection)
+{
+    // the same on a 64 x 128 map with a 7 x 7 window, the projection through its kernel tiled in the window's plane
+    // (taken by itself from 192 tiles of 4 x 64 positions on; forced here on 32)
+    filter_factory<float, host_memory_space> ff(64, 128, 7, 1, 1);
+    dia_matrix<float, host_memory_space> *W = ff.get_dia();
+    const int N = W->h(), batch = 32;
+    for (int i = 0; i < (int)W->vec().size(); i++) W->vec()[i] = 0.01f * (float)((i * 37) % 101 + 1);
+    tensor<float, host_memory_space, column_major> V(N, batch), H(N, batch);
+    for (int i = 0; i < N * batch; i++) { V[i] = (float)((i * 13) % 7) / 7.f; H[i] = (float)((i * 29) % 11) / 11.f; }
+    dia_matrix<float, dev_memory_space> Wd(N, N, W->num_dia(), W->stride(), 1);
+    convert(Wd, *W);
+    tensor<float, dev_memory_space, column_major> Vd(V.shape()), Hd(H.shape());
+    convert(Vd, V); convert(Hd, H);
+    CHECK(cuvdia_set_path(CUVDIA_PATH_WINDOW) == CUVDIA_OK);
+    densedense_to_dia(Wd, Hd, Vd, 1.f / batch, 0.9f);
+    const int ran = cuvdia_last_path();
+    CHECK(cuvdia_set_path(CUVDIA_PATH_AUTO) == CUVDIA_OK);
+    CHECK(ran == CUVDIA_PATH_WINDOW);
+    host_block_descriptor<float> bdh(*W);
+    cuv_oracle::densedense_to_dia(*W, bdh, H, V, 1.f / batch, 0.9f);
+    MAT_CMP(*W, Wd, 0.01f);
+    delete W;
+}
+
 int main(int argc, char **argv)
 {
     initCUDA(CUDA_TEST_DEVICE);
