@@ -21,8 +21,8 @@ def gu():
     return _gpu_util
 
 
-def _dia(o, rng, h, w, offsets):
-    d = o.Dia(h, w, np.asarray(offsets, np.int32), None, 1)
+def _dia(o, rng, h, w, offsets, stride=None):
+    d = o.Dia(h, w, np.asarray(offsets, np.int32), stride, 1)
     d.vals[:] = np.nan
     m = o.valid_mask(d)
     d.vals[m] = rng.uniform(-1, 1, int(m.sum())).astype(np.float32)
@@ -192,7 +192,11 @@ def test_random_window_shapes(oracle, gu, seed):
     h = channels * map_elems - 4 * int(rng.integers(0, 3))
     w = channels * map_elems - 4 * int(rng.integers(0, 3))
     batch = int(rng.choice([1, 3, 4, 7, 8, 17, 32]))
-    C = _dia(oracle, rng, h, w, _window(px, rows, cols, dy0, dx0, channels, map_elems))
+    offsets = _window(px, rows, cols, dy0, dx0, channels, map_elems)
+    if seed % 3 == 0:
+        offsets = offsets[::-1]                                        # listed from the last to the first
+    stride = max(h, w) + int(rng.choice([0, 0, 1, 3, 4, 13]))         # (a stride that is no multiple of 4: the 16-byte
+    C = _dia(oracle, rng, h, w, offsets, stride)                       # stores then start at any 4-byte boundary)
     A, B = _operands(rng, C, batch)
     alpha, beta = float(rng.choice([1.0, -0.5, 1.0 / batch])), float(rng.choice([0.0, 0.9, -1.5]))
     _, ran = gu.check_dd2dia(oracle, C, A, B, alpha, beta, _lib.PATH_WINDOW, "random window %d" % seed)
