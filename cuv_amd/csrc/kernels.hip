@@ -2305,7 +2305,7 @@ __device__ __forceinline__ void dw_ring(F &body, int gi, int n)
     }
 }
 
-// SUBS: the batch is cut into SUBS ranges of whole groups, each worked by 4 waves of the workgroup's 4 SUBS with
+// SUBS: the batch is cut into SUBS ranges of whole groups, each worked by 4 of the workgroup's 4 x SUBS waves with
 // staging buffers of their own (launches of few tiles: 2 or 4 ranges keep 16 waves on every CU where one
 // range per tile would leave most of the chip idle).  The ranges' sums meet in LDS at the end, in range order.
 template <int LC, int SH, int SUBS>
