@@ -2525,6 +2525,8 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
     const int o = i_tile + wave * period + 4 * xg;              // the lane's first row of A
     const bool x_ok = S::TX * tx + 4 * xg < period;             // (a narrower last tile column: the positions past the
                                                                 // row belong to the next row's first tile)
+    // (A window row's old values are all requested before the first of them is used: a request per slot, waited
+    // for and stored before the next, cost the workgroup LC round trips to memory in a row.)
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
         const int dyl = 2 * role + n;
@@ -2532,39 +2534,58 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
         const int dy = DYB * db + (dy_ok ? dyl : 0);
         const int e0 = tab[ngroups + g * K + dy] / 4 + o;       // element of slot j = 0 for row o
         const int in0 = o + s_g + dyl * period;                 // the row of B that row o meets in slot j = 0
+        unsigned off[LC], okbits[LC];
+        f4u old4[LC];
+        bool any_part = false;                                  // wave-uniform: some lane has a partly valid group of 4
 #pragma unroll
         for (int j = 0; j < LC; ++j) {
-            bool ok[4];
+            unsigned bits = 0;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) ok[t] = dy_ok & x_ok & (o + t < h) & ((unsigned)(in0 + j + t) < (unsigned)w);
-            const bool all4 = ok[0] & ok[1] & ok[2] & ok[3];
-            const bool part = (ok[0] | ok[1] | ok[2] | ok[3]) & !all4;
-            const unsigned off = (unsigned)(e0 + j * astep) * 4u;
-            const bool any_part = __builtin_amdgcn_ballot_w64(part) != 0ull;       // wave-uniform
-            float r[4];
+            for (int t = 0; t < 4; ++t)
+                bits |= (unsigned)(dy_ok & x_ok & (o + t < h) & ((unsigned)(in0 + j + t) < (unsigned)w)) << t;
+            okbits[j] = bits;
+            off[j] = (unsigned)(e0 + j * astep) * 4u;
+            any_part = any_part || __builtin_amdgcn_ballot_w64(bits != 0u && bits != 15u) != 0ull;
+            old4[j] = f4u{0.f, 0.f, 0.f, 0.f};
+            if (beta != 0.f)
+                old4[j] = __builtin_bit_cast(f4u, __builtin_amdgcn_raw_buffer_load_b128(cr, bits == 15u ? off[j] : OOB_OFFSET, 0, 0));
+        }
+        if (!any_part) {
+            // every lane's groups of 4 are whole or empty: nothing but the stores, no wait between them
 #pragma unroll
-            for (int t = 0; t < 4; ++t) r[t] = alpha * acc[n][t][j];
-            if (beta != 0.f) {
-                const f4u old4 = __builtin_bit_cast(f4u, __builtin_amdgcn_raw_buffer_load_b128(cr, all4 ? off : OOB_OFFSET, 0, 0));
-                float old[4] = {old4.x, old4.y, old4.z, old4.w};
-                if (any_part) {
+            for (int j = 0; j < LC; ++j) {
+                float r[4];
+                const float old[4] = {old4[j].x, old4[j].y, old4[j].z, old4[j].w};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) r[t] = (beta == 0.f) ? alpha * acc[n][t][j] : beta * old[t] + alpha * acc[n][t][j];
+                __builtin_amdgcn_raw_buffer_store_b128(sp_u4{__builtin_bit_cast(unsigned, r[0]), __builtin_bit_cast(unsigned, r[1]),
+                                                             __builtin_bit_cast(unsigned, r[2]), __builtin_bit_cast(unsigned, r[3])},
+                                                       cr, okbits[j] == 15u ? off[j] : OOB_OFFSET, 0, 2);
+            }
+        } else {
+            // workgroups at the matrix's first and last rows: the partly valid groups row by row
+#pragma unroll
+            for (int j = 0; j < LC; ++j) {
+                const bool all4 = okbits[j] == 15u;
+                const bool part = okbits[j] != 0u && !all4;
+                float old[4] = {old4[j].x, old4[j].y, old4[j].z, old4[j].w};
+                if (beta != 0.f) {
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        const float v = buffer_load_f32(cr, (part & ok[t]) ? off + 4u * t : OOB_OFFSET);
+                        const float v = buffer_load_f32(cr, (part && ((okbits[j] >> t) & 1u)) ? off[j] + 4u * t : OOB_OFFSET);
                         old[t] = part ? v : old[t];
                     }
                 }
+                float r[4];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) r[t] = beta * old[t] + alpha * acc[n][t][j];
-            }
-            __builtin_amdgcn_raw_buffer_store_b128(sp_u4{__builtin_bit_cast(unsigned, r[0]), __builtin_bit_cast(unsigned, r[1]),
-                                                         __builtin_bit_cast(unsigned, r[2]), __builtin_bit_cast(unsigned, r[3])},
-                                                   cr, all4 ? off : OOB_OFFSET, 0, 2);
-            if (any_part) {
+                for (int t = 0; t < 4; ++t) r[t] = (beta == 0.f) ? alpha * acc[n][t][j] : beta * old[t] + alpha * acc[n][t][j];
+                __builtin_amdgcn_raw_buffer_store_b128(sp_u4{__builtin_bit_cast(unsigned, r[0]), __builtin_bit_cast(unsigned, r[1]),
+                                                             __builtin_bit_cast(unsigned, r[2]), __builtin_bit_cast(unsigned, r[3])},
+                                                       cr, all4 ? off[j] : OOB_OFFSET, 0, 2);
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, r[t]), cr,
-                                                          (part & ok[t]) ? off + 4u * t : OOB_OFFSET, 0, 2);
+                                                          (part && ((okbits[j] >> t) & 1u)) ? off[j] + 4u * t : OOB_OFFSET, 0, 2);
             }
         }
     }
