@@ -2362,11 +2362,14 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
             const int col = p / (nbr * BPR), rem = p - col * (nbr * BPR);
             const int row = rem / BPR, pc = rem - row * BPR;
             const int idx = b_tile + row * period + 4 * pc;
-            if ((p < npb) & (idx >= 0) & (idx + 4 <= w)) v = (unsigned)((col_first + col) * (int)ldb + idx) * 4u;
+            // (64-bit: a column past the batch may lie past 2^31 bytes; it is out of range either way)
+            const long long at = ((long long)(col_first + col) * ldb + idx) * 4;
+            if ((p < npb) & (idx >= 0) & (idx + 4 <= w) & (at < (long long)OOB_OFFSET)) v = (unsigned)at;
         } else if (s < ni) {
             const int col = s - nib, row = lane >> 4, pc = lane & 15;
             const int idx = i_tile + row * period + 4 * pc;
-            if (idx + 4 <= h) v = (unsigned)((col_first + col) * (int)lda + idx) * 4u;
+            const long long at = ((long long)(col_first + col) * lda + idx) * 4;
+            if ((idx + 4 <= h) & (at < (long long)OOB_OFFSET)) v = (unsigned)at;
         }
         v_lane[it] = v;
     }
@@ -3022,7 +3025,9 @@ hipError_t launch_dd2dia_tiled(const DiaView &C, float *vals, const float *A, lo
     if (windowed) *windowed = false;
     if (window >= 0) {
         int txn = 0, tyn = 0, ndb = 0;
-        const long long wgs = dd2dia_window_workgroups(C, batch, &txn, &tyn, &ndb);
+        long long wgs = dd2dia_window_workgroups(C, batch, &txn, &tyn, &ndb);
+        // (a lane's byte offsets run up to 16 columns past the batch and must stay below 2^32)
+        if (((long long)batch + 16) * std::max(lda, ldb) * 4 >= (1LL << 32)) wgs = 0;
         if (wgs > 0 && (window > 0 || dd2dia_window_by_size(C, batch, wgs))) {
             const WalkView &wk = C.walk_n;
             const DwLaunch L{wk.tab_dev, wk.ngroups, wk.k, wk.period, wk.s0, wk.astep4 / 4, wk.lck, vals, A, lda, B, ldb,
