@@ -2177,6 +2177,7 @@ __device__ __forceinline__ void dd2dia_unit(
 
 // Shape of the blocks the projection's tiles are numbered in (see the kernel): units per block and row tiles per
 // block, 64 positions or nearly.
+constexpr int DW_LONG_ROWS = 7;              // window rows per workgroup of the projection's kernel for rows of 9 to 13 diagonals
 constexpr int DW_MIN_WGS = 768;               // workgroups from which the window-table projection of a 7 x 7 window is ahead
 constexpr int DD_BLOCKED_MIN_TILES = 1024;   // launches of more than a few rounds number their tiles in blocks
 struct DdBlock {
@@ -2332,9 +2333,9 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
     // workgroups an XCD receives together are a band of neighbouring tiles, which share their stretches of B
     int rest = xcd_tile(blockIdx.x, gridDim.x);
     const int tx = rest % txn; rest /= txn;
-    const int ty = rest % tyn; rest /= tyn;
-    const int db = rest % ndb;
-    const int g = rest / ndb;
+    const int db = rest % ndb; rest /= ndb;
+    const int ty = rest % tyn;
+    const int g = rest / tyn;
     const int kb = min(DYB, K - DYB * db);                    // window rows served here
     const int nbr = WAVES - 1 + kb;                           // stretches of B per column
     const int i_tile = 4 * ty * period + S::TX * tx;          // the tile's first row of A
@@ -2411,25 +2412,29 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
 #pragma unroll
             for (int j = 0; j < LC; ++j) acc[n][t][j] = 0.f;
 
-    struct Win { float v[WQ * 4]; };
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    struct Win { v4f p[WQ]; };
     auto read_win = [&](Win &win, const float *buf, int c, int n) __attribute__((always_inline)) {
-        typedef float v4f __attribute__((ext_vector_type(4)));
         const v4f *p4 = reinterpret_cast<const v4f *>(buf + c * col_floats + w_off[n]);
 #pragma unroll
-        for (int q = 0; q < WQ; ++q) {
-            v4f v = p4[q];
-            // (the window's first and last values may be unused: without this the compiler fetches the others
-            // one by one, and four-byte reads 16 bytes apart share their banks four ways)
-            asm volatile("" : "+v"(v));
-            win.v[4 * q + 0] = v.x; win.v[4 * q + 1] = v.y; win.v[4 * q + 2] = v.z; win.v[4 * q + 3] = v.w;
-        }
+        for (int q = 0; q < WQ; ++q) win.p[q] = p4[q];
     };
-    auto fmas = [&](int n, const float4 &a, const Win &win) __attribute__((always_inline)) {
+    auto fmas = [&](int n, const float4 &a, Win &win) __attribute__((always_inline)) {
         const float av[4] = {a.x, a.y, a.z, a.w};
+        float wv[WQ * 4];
+#pragma unroll
+        for (int q = 0; q < WQ; ++q) {
+            // (The window's first and last values may be unused: without this the compiler fetches the others one
+            // by one, and four-byte reads 16 bytes apart share their banks four ways.  The asm sits where the
+            // window is used, not where it is read: the wait for the read goes with it.)
+            v4f v = win.p[q];
+            asm volatile("" : "+v"(v));
+            wv[4 * q + 0] = v.x; wv[4 * q + 1] = v.y; wv[4 * q + 2] = v.z; wv[4 * q + 3] = v.w;
+        }
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int j = 0; j < LC; ++j) acc[n][t][j] = __builtin_fmaf(av[t], win.v[SH + t + j], acc[n][t][j]);
+            for (int j = 0; j < LC; ++j) acc[n][t][j] = __builtin_fmaf(av[t], wv[SH + t + j], acc[n][t][j]);
     };
     // One group: the second window of a column and the next column's first are read while the FMAs of the
     // window before them run.
@@ -2589,6 +2594,254 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
                 for (int t = 0; t < 4; ++t)
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, r[t]), cr,
                                                           (part && ((okbits[j] >> t) & 1u)) ? off[j] + 4u * t : OOB_OFFSET, 0, 2);
+            }
+        }
+    }
+}
+
+// The same tiling for window rows of 9 to 13 diagonals (a chunk of the products' table: the large layer's 13 x 13
+// window), with the roles turned round: a wave's 2 x 4 x LC sums would not fit its registers, so here a WAVE owns
+// one window row (DwLongShape::WAVES of them per workgroup; a taller window takes several workgroups per tile) and
+// a lane's role is the y of the tile's four: 4 x LC running sums, one 16-byte read of A and one window of B
+// (4 + LC - 1 values) per column.  Staging, ring, waits and the results' way out are those of the kernel above; a
+// wave past the block's last window row only helps with the requests.
+template <int LC, int SH>
+struct DwLongShape {
+    static constexpr int WAVES = DW_LONG_ROWS, YT = 4, TX = 64;
+    static constexpr int COLS = 8;                               // batch columns per staged group
+    static constexpr int NBUF = 2;                               // (3 or 4 buffers of 4 columns measured 3 - 4 % slower)
+    static constexpr int WIN = SH + 4 + LC - 1;
+    static constexpr int WQ = (WIN + 3) / 4;
+    static constexpr int BPR = TX / 4 + WQ - 1;
+    static constexpr int NBR_MAX = YT - 1 + WAVES;
+    static constexpr int B_PIECES = (COLS * NBR_MAX * BPR + 63) / 64 * 64;
+    static constexpr int A_PIECES = COLS * YT * (TX / 4);
+    static constexpr int BUF_PIECES = B_PIECES + A_PIECES;
+    static constexpr int NI_MAX = BUF_PIECES / 64;
+    static constexpr int NIT = (NI_MAX + WAVES - 1) / WAVES;
+    static_assert(A_PIECES % 64 == 0 && LC > CHUNK_MAX && LC <= SP_CHUNK_MAX && SH >= 0 && SH < 4, "shape");
+    static_assert(NBUF >= 2 && NBUF * BUF_PIECES * 16 <= 80 * 1024, "two buffers; two workgroups per CU and to spare");
+};
+
+template <int LC, int SH>
+__global__ __launch_bounds__(64 * DW_LONG_ROWS, 4) void dd2dia_window_long_kernel(
+    const int *__restrict__ tab, int ngroups, int K, int period, int s0, int astep, float *__restrict__ C,
+    const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
+    int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes, unsigned c_bytes,
+    int txn, int tyn, int ndb)
+{
+    typedef DwLongShape<LC, SH> S;
+    constexpr int WAVES = S::WAVES, YT = S::YT, COLS = S::COLS, WQ = S::WQ, BPR = S::BPR, NIT = S::NIT;
+    __shared__ __attribute__((aligned(16))) float lds[S::NBUF][S::BUF_PIECES * 4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    typedef const int __attribute__((address_space(4))) *sc_int_ptr;
+    const sc_int_ptr stab = (sc_int_ptr)tab;
+
+    // workgroup -> (group, tile row, block of window rows, tile column): the blocks of a tile side by side, so that
+    // they find the tile's rows of A and the stretches they share in the XCD's L2
+    int rest = xcd_tile(blockIdx.x, gridDim.x);
+    const int tx = rest % txn; rest /= txn;
+    const int db = rest % ndb; rest /= ndb;
+    const int ty = rest % tyn;
+    const int g = rest / tyn;
+    const int kb = min(WAVES, K - WAVES * db);                // window rows served here
+    const int nbr = YT - 1 + kb;                              // stretches of B per column
+    const int i_tile = YT * ty * period + S::TX * tx;         // the tile's first row of A
+    const int s_g = s0 + stab[g] + WAVES * db * period;       // shift of this block's first slot
+    const int b_tile = i_tile + s_g - SH;                     // first staged row of B, a multiple of 4
+    const int b_hi = b_tile + (nbr - 1) * period + 4 * BPR;
+    if (i_tile >= h || b_hi <= 0 || b_tile >= w) return;
+
+    const int npb = COLS * nbr * BPR;
+    const int nib = (npb + 63) / 64;
+    const int ni = nib + S::A_PIECES / 64;
+    const int ngr = (batch + COLS - 1) / COLS;
+    unsigned v_lane[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+        const int s = wave + WAVES * it;
+        unsigned v = OOB_OFFSET;
+        if (s < nib) {
+            const int p = 64 * s + lane;
+            const int col = p / (nbr * BPR), rem = p - col * (nbr * BPR);
+            const int row = rem / BPR, pc = rem - row * BPR;
+            const int idx = b_tile + row * period + 4 * pc;
+            const long long at = ((long long)col * ldb + idx) * 4;
+            if ((p < npb) & (idx >= 0) & (idx + 4 <= w) & (at < (long long)OOB_OFFSET)) v = (unsigned)at;
+        } else if (s < ni) {
+            const int col = s - nib, row = lane >> 4, pc = lane & 15;
+            const int idx = i_tile + row * period + 4 * pc;
+            const long long at = ((long long)col * lda + idx) * 4;
+            if ((idx + 4 <= h) & (at < (long long)OOB_OFFSET)) v = (unsigned)at;
+        }
+        v_lane[it] = v;
+    }
+    const sp_int4 bq = raw_rsrc(B, b_bytes), aq = raw_rsrc(A, a_bytes);
+    const unsigned lds0 = (unsigned)(unsigned long long)(__attribute__((address_space(3))) float *)&lds[0][0];
+    constexpr unsigned BUF_BYTES = S::BUF_PIECES * 16u;
+    const unsigned b_step = (unsigned)ldb * (4u * COLS), a_step = (unsigned)lda * (4u * COLS);
+    auto issue = [&](int par) __attribute__((always_inline)) {
+        const unsigned buf = lds0 + (unsigned)par * BUF_BYTES;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int s = wave + WAVES * it;
+            if (s < nib) {
+                lds_load_b128(bq, buf + 1024u * (unsigned)s, v_lane[it], 0u);
+                v_lane[it] += b_step;
+            } else if (s < ni) {
+                lds_load_b128(aq, buf + (unsigned)S::B_PIECES * 16u + 1024u * (unsigned)(s - nib), v_lane[it], 0u);
+                v_lane[it] += a_step;
+            }
+        }
+    };
+
+    const int role = lane >> 4, xg = lane & 15;               // role = the lane's y of the tile's four
+    const bool active = wave < kb;                            // (wave-uniform)
+    const int w_off = ((role + min(wave, kb - 1)) * BPR + xg) * 4;
+    const int col_floats = nbr * BPR * 4;
+    const int a_off = S::B_PIECES * 4 + (role * 16 + xg) * 4;
+
+    float acc[4][LC];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int j = 0; j < LC; ++j) acc[t][j] = 0.f;
+
+    // One group.  A column's FMAs run in the order of the window values they use; as soon as a 16-byte piece of the
+    // window has served its last FMA, the same registers take the next column's piece -- one window in registers,
+    // its reads hidden behind the FMAs of the pieces after it.
+    // (The pieces stay whole 16-byte reads because each passes through an empty asm -- see the kernel above -- and
+    // that asm sits where the piece is first used, not where it is read: the wait for the read goes with it.)
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    v4f wv[WQ];
+    auto read_piece = [&](const float *buf, int c, int q) __attribute__((always_inline)) {
+        wv[q] = reinterpret_cast<const v4f *>(buf + c * col_floats + w_off)[q];
+    };
+    auto apply = [&](const float *buf) __attribute__((always_inline)) {
+        float4 a0, a1;
+        a0 = *reinterpret_cast<const float4 *>(buf + a_off);
+#pragma unroll
+        for (int q = 0; q < WQ; ++q) read_piece(buf, 0, q);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            float4 &ac = (c & 1) ? a1 : a0;
+            float4 &an = (c & 1) ? a0 : a1;
+            if (c + 1 < COLS) an = *reinterpret_cast<const float4 *>(buf + a_off + (c + 1) * 256);
+            const float av[4] = {ac.x, ac.y, ac.z, ac.w};
+#pragma unroll
+            for (int q = 0; q < WQ; ++q) {
+                __builtin_amdgcn_sched_barrier(0);
+                v4f v = wv[q];
+                asm volatile("" : "+v"(v));
+                const float win4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int j = 4 * q + e - SH - t;
+                        if (j >= 0 && j < LC) acc[t][j] = __builtin_fmaf(av[t], win4[e], acc[t][j]);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+                if (c + 1 < COLS) read_piece(buf, c + 1, q);
+            }
+        }
+    };
+
+    // The ring (as in the kernel above): group gi is applied out of buffer gi mod NBUF while the groups up to
+    // gi + NBUF - 1 are in flight or landed; at a group's end everything but the requests of the groups after the
+    // next has to have arrived -- this wave's share of a group is n_mine instructions, and they complete in order.
+    constexpr int NBUF = S::NBUF;
+    const int n_mine = (ni - wave + WAVES - 1) / WAVES;
+    auto wait_leaving_groups = [&](int groups) __attribute__((always_inline)) {
+        switch (groups * n_mine) {
+            case 0: asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)" ::: "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory"); break;
+            case 3: asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory"); break;
+            case 4: asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory"); break;
+            case 5: asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory"); break;
+            case 6: asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory"); break;
+            case 7: asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory"); break;
+        }
+    };
+    static_assert((NBUF - 2) * NIT <= 8, "the waits name up to eight requests left in flight");
+    for (int k = 0; k < NBUF - 1; ++k)
+        if (k < ngr) issue(k);
+    wait_leaving_groups(min(NBUF - 2, ngr - 1));
+    __syncthreads();
+    auto body = [&](int gi, auto cur_c) __attribute__((always_inline)) {
+        constexpr int cur = decltype(cur_c)::value;
+        if (gi + NBUF - 1 < ngr) issue((cur + NBUF - 1) % NBUF);
+        if (active) apply(&lds[cur][0]);
+        wait_leaving_groups(max(0, min(NBUF - 2, ngr - 2 - gi)));
+        __syncthreads();
+    };
+#pragma clang loop unroll(disable)
+    for (int gi = 0; gi < ngr; gi += NBUF) dw_ring<NBUF, 0>(body, gi, ngr);
+    if (!active) return;
+
+    // Results: 4 consecutive rows of every slot of the wave's window row per lane.
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    typedef unsigned sp_u4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t cr = make_rsrc(C, c_bytes);
+    const int o = i_tile + role * period + 4 * xg;              // the lane's first row of A
+    const bool x_ok = S::TX * tx + 4 * xg < period;
+    const int dy = WAVES * db + wave;
+    const int e0 = tab[ngroups + g * K + dy] / 4 + o;           // element of slot j = 0 for row o
+    const int in0 = o + s_g + wave * period;                    // the row of B that row o meets in slot j = 0
+    // (half of the window row's slots at a time: their old values, requested together, and the sums share the
+    // registers)
+    constexpr int JH = (LC + 1) / 2;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int j0 = half * JH;
+        unsigned off[JH], okbits[JH];
+        f4u old4[JH];
+        bool any_part = false;
+#pragma unroll
+        for (int jj = 0; jj < JH; ++jj) {
+            const int j = j0 + jj;
+            unsigned bits = 0;
+            if (j < LC) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    bits |= (unsigned)(x_ok & (o + t < h) & ((unsigned)(in0 + j + t) < (unsigned)w)) << t;
+            }
+            okbits[jj] = bits;
+            off[jj] = (unsigned)(e0 + j * astep) * 4u;
+            any_part = any_part || __builtin_amdgcn_ballot_w64(bits != 0u && bits != 15u) != 0ull;
+            old4[jj] = f4u{0.f, 0.f, 0.f, 0.f};
+            if (beta != 0.f)
+                old4[jj] = __builtin_bit_cast(f4u, __builtin_amdgcn_raw_buffer_load_b128(cr, bits == 15u ? off[jj] : OOB_OFFSET, 0, 0));
+        }
+#pragma unroll
+        for (int jj = 0; jj < JH; ++jj) {
+            const int j = j0 + jj;
+            if (j >= LC) continue;
+            const bool all4 = okbits[jj] == 15u;
+            const bool part = okbits[jj] != 0u && !all4;
+            float old[4] = {old4[jj].x, old4[jj].y, old4[jj].z, old4[jj].w};
+            if (any_part && beta != 0.f) {
+                // workgroups at the matrix's first and last rows: the partly valid groups row by row
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const float v = buffer_load_f32(cr, (part && ((okbits[jj] >> t) & 1u)) ? off[jj] + 4u * t : OOB_OFFSET);
+                    old[t] = part ? v : old[t];
+                }
+            }
+            float r[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) r[t] = (beta == 0.f) ? alpha * acc[t][j] : beta * old[t] + alpha * acc[t][j];
+            __builtin_amdgcn_raw_buffer_store_b128(sp_u4{__builtin_bit_cast(unsigned, r[0]), __builtin_bit_cast(unsigned, r[1]),
+                                                         __builtin_bit_cast(unsigned, r[2]), __builtin_bit_cast(unsigned, r[3])},
+                                                   cr, all4 ? off[jj] : OOB_OFFSET, 0, 2);
+            if (any_part) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, r[t]), cr,
+                                                          (part && ((okbits[jj] >> t) & 1u)) ? off[jj] + 4u * t : OOB_OFFSET, 0, 2);
             }
         }
     }
@@ -2794,6 +3047,23 @@ hipError_t dd2dia_window_launch(const DwLaunch &L)
         else if (L.subs == 2) CUVDIA_DW_LAUNCH_SUBS(LC, 2);                                                           \
         else CUVDIA_DW_LAUNCH_SUBS(LC, 1);                                                                            \
         break;
+    if (L.lck > CHUNK_MAX) {
+        if (L.subs != 1) return hipErrorNotSupported;
+        note_kernel("dd2dia_window_long_kernel<%d, %d>", L.lck, sh);
+#define CUVDIA_DWL_LAUNCH(LC)                                                                                          \
+    case LC:                                                                                                           \
+        if (sh == 0) hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 0>), grid, dim3(64 * DwLongShape<LC, 0>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
+        else if (sh == 1) hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 1>), grid, dim3(64 * DwLongShape<LC, 1>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
+        else if (sh == 2) hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 2>), grid, dim3(64 * DwLongShape<LC, 2>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
+        else hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 3>), grid, dim3(64 * DwLongShape<LC, 3>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
+        break;
+        switch (L.lck) {
+            CUVDIA_DWL_LAUNCH(9) CUVDIA_DWL_LAUNCH(10) CUVDIA_DWL_LAUNCH(11) CUVDIA_DWL_LAUNCH(12) CUVDIA_DWL_LAUNCH(13)
+            default: return hipErrorNotSupported;
+        }
+#undef CUVDIA_DWL_LAUNCH
+        return hipGetLastError();
+    }
     note_kernel("dd2dia_window_kernel<%d, %d, %d>", L.lck, sh, L.subs);
     switch (L.lck) {
         CUVDIA_DW_LAUNCH(2) CUVDIA_DW_LAUNCH(3) CUVDIA_DW_LAUNCH(4) CUVDIA_DW_LAUNCH(5)
@@ -2979,11 +3249,12 @@ int dd2dia_slab_columns(const DiaView &C, long long lda, long long ldb)
 long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn, int *tyn, int *ndb)
 {
     const WalkView &wk = C.walk_n;
-    if (wk.tab_dev == nullptr || wk.lck < 2 || wk.lck > CHUNK_MAX || !wk.rows4 || wk.period % 4 != 0 ||
+    if (wk.tab_dev == nullptr || wk.lck < 2 || wk.lck > SP_CHUNK_MAX || !wk.rows4 || wk.period % 4 != 0 ||
         C.h % 4 != 0 || C.w % 4 != 0 || batch < 1 || wk.astep4 % 4 != 0)
         return 0;
     const long long image_rows = ((long long)C.h + wk.period - 1) / wk.period;
-    const long long tx = ((long long)wk.period + 63) / 64, ty = (image_rows + 3) / 4, db = (wk.k + 7) / 8;
+    const long long tx = ((long long)wk.period + 63) / 64, ty = (image_rows + 3) / 4,
+                    db = wk.lck > CHUNK_MAX ? (wk.k + DW_LONG_ROWS - 1) / DW_LONG_ROWS : (wk.k + 7) / 8;
     const long long total = tx * ty * db * wk.ngroups;
     if (total > 0x7fffffffLL || (long long)4 * ty * wk.period + 64 * tx >= (1LL << 30)) return 0;
     if (txn) *txn = (int)tx;
@@ -3001,6 +3272,7 @@ int dd2dia_window_subs(const DiaView &C, long long workgroups)
 {
     const int slots = C.walk_n.k * C.walk_n.lck;
     const long long min_wgs = slots >= 49 ? DW_MIN_WGS : slots >= 25 ? DW_MIN_WGS * 4 / 3 : DW_MIN_WGS * 2;
+    if (C.walk_n.lck > CHUNK_MAX) return 1;            // (rows of 9 to 13 diagonals: one range only)
     return workgroups >= min_wgs ? 1 : 2 * workgroups >= min_wgs ? 2 : 4;
 }
 // Whether the automatic choice takes the window-table projection: enough tiles to fill the chip and a map no
@@ -3013,7 +3285,17 @@ bool dd2dia_window_by_size(const DiaView &C, int batch, long long workgroups)
     const int slots = C.walk_n.k * C.walk_n.lck;
     const long long min_wgs = slots >= 49 ? DW_MIN_WGS : slots >= 25 ? DW_MIN_WGS * 4 / 3 : DW_MIN_WGS * 2;
     const int subs = dd2dia_window_subs(C, workgroups);
-    if (subs * workgroups < min_wgs || C.walk_n.period < 64) return false;
+    if (C.walk_n.period < 64) return false;
+    if (C.walk_n.lck > CHUNK_MAX) {
+        // Rows of 9 to 13 diagonals: a tile saves the more the more units (window rows x groups) shared its rows
+        // under the chunk-by-chunk kernel.  Measured on 9 x 9 to 13 x 13 windows, 1 to 4 channels, maps 128 to 1024
+        // wide, batch 16 to 1024: 1.04 - 1.48 times its rate where taken, 0.75 - 1.0 where not.
+        const int units = C.walk_n.k * C.walk_n.ngroups;
+        if (C.walk_n.period < 192) return false;        // (four channels of 13 x 13 on a 128-wide map: 0.75)
+        if (workgroups >= 4096) return true;
+        return units >= 13 && (workgroups >= 1024 || (workgroups >= 512 && C.walk_n.period >= 256));
+    }
+    if (subs * workgroups < min_wgs) return false;
     if (subs == 1) return slots >= 25 || batch >= 128;
     return slots >= 49 && batch >= (subs == 2 ? 512 : 32);
 }

@@ -119,14 +119,17 @@ int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap
  * kernel tiled in the window's plane for an h x w matrix with this table
  * (row_fact 1) and `batch` packed dense columns?  Returns the number of
  * workgroups of that launch (tiles of 4 x 64 positions x blocks of 8 window
- * rows x channel groups), or 0 when the chunk-by-chunk kernel serves: the
- * table is no window table (see cuvdia_plan_walk) of chunks of 2 to 8
- * diagonals, the period, a channel distance or a row count is no multiple of
- * 4, the period is below 64, or the launch has too few workgroups to fill
- * the chip: 768 for windows of 49 slots or more -- or 384 at a batch of at
- * least 512, or 192 at a batch of at least 32: a workgroup then works two or
- * four ranges of the batch side by side --, 1024 from 25 slots, 1536 and a
- * batch of at least 128 below.  Negative: an error.
+ * rows -- of 7 where a window row has 9 to 13 diagonals -- x channel
+ * groups), or 0 when the chunk-by-chunk kernel serves: the table is no
+ * window table (see cuvdia_plan_walk) of chunks of 2 to 13 diagonals, the
+ * period, a channel distance or a row count is no multiple of 4, the period
+ * is below 64, or the launch has too few workgroups to fill the chip.  For
+ * chunks of up to 8 diagonals: 768 for windows of 49 slots or more -- or 384
+ * at a batch of at least 512, or 192 at a batch of at least 32: a workgroup
+ * then works two or four ranges of the batch side by side --, 1024 from 25
+ * slots, 1536 and a batch of at least 128 below.  For chunks of 9 to 13, on
+ * periods of at least 192: 4096, or 1024 (512 on periods of at least 256)
+ * when window rows x channel groups are at least 13.  Negative: an error.
  * cuvdia_set_path(CUVDIA_PATH_WINDOW) waives the conditions on the period's
  * size, the workgroups and the batch.  No counterpart in the reference. */
 long long cuvdia_plan_window_launch(const int *offsets_host, int nd, int stride, int h, int w, int batch);
@@ -256,8 +259,9 @@ int cuvdia_learn_step_weight_decay_momentum_f32(float *W_device, float *momentum
  * on `stream`, slab of columns after slab, each adding to C.
  * Summation order per slot: see kernels.hip; the kernel for large window
  * tables (cuvdia_last_path() == CUVDIA_PATH_WINDOW) adds the batch columns in
- * ascending order into one sum (on launches of few tiles: into two or four
- * sums over consecutive ranges of the batch), the chunk-by-chunk kernel into
+ * ascending order into one sum (on launches of few tiles of a window with
+ * rows of at most 8 diagonals: into two or four sums over consecutive ranges
+ * of the batch), the chunk-by-chunk kernel into
  * four or eight interleaved partial sums: their results differ by rounding,
  * both within 1e-5 of the sum of |terms| of the reference's host result. */
 int cuvdia_dd2dia_f32(const cuvdia_desc *desc, float *C_vals_device,
@@ -340,7 +344,7 @@ int cuvdia_cache_clear(void);
  * that is no window table with a walking kernel; densedense_to_dia treats it
  * as CUVDIA_PATH_TILED_NOWALK).  CUVDIA_PATH_WINDOW: the kernels tiled in the
  * window's plane, which serve densedense_to_dia (CUVDIA_EUNSUPPORTED when
- * they do not serve the request: no window table of chunks of 2 to 8
+ * they do not serve the request: no window table of chunks of 2 to 13
  * diagonals, a period, channel distances or row counts that are no multiples
  * of 4); the products treat it as CUVDIA_PATH_TILED_NOWALK. */
 int cuvdia_set_path(int path);

@@ -315,7 +315,8 @@ def _window_launch(offs, stride, h, w, batch):
 def test_window_projection_launch_by_table_shape_and_size():
     """The projection tiled in the window's plane: tiles of 4 x 64 positions, taken from 768 (49 slots; fewer with
     two or four batch ranges per tile), 1024 (25 slots) or 1536 tiles and batch 128 (fewer slots) on; period,
-    channel distances and row counts multiples of 4; chunks of 2 to 8 diagonals."""
+    channel distances and row counts multiples of 4; chunks of 2 to 8 diagonals -- and, with a rule of their own,
+    of 9 to 13."""
     from cuv_amd import _lib, workloads as W
     n = 512 * 512
     offs = W.window_offsets(512, 7)
@@ -342,10 +343,19 @@ def test_window_projection_launch_by_table_shape_and_size():
     # four channels of a 256-wide map: 4 tile columns x 256 tile rows x 4 groups
     offs4 = W.window_offsets(256, 7, 4)
     assert _window_launch(offs4, 4 * 256 * 256, 4 * 256 * 256, 4 * 256 * 256, 32) == 4 * 256 * 4
-    # 13 window rows: two blocks of window rows per tile -- but 13 diagonals per row are not served
-    assert _window_launch(W.window_offsets(512, 13), n, n, n, 128) == 0
+    # 13 window rows of 7 diagonals: two blocks of 8 window rows per tile
     tall = [dy * 512 + dx for dy in range(-6, 7) for dx in range(-3, 4)]
     assert _window_launch(tall, n, n, n, 128) == 2 * 8 * 128
+    # window rows of 9 to 13 diagonals: blocks of 7 window rows; on maps at least 192 wide taken from 4096
+    # workgroups, or from 1024 (512 on maps at least 256 wide) when window rows x channel groups are at least 13
+    assert _window_launch(W.window_offsets(512, 13), n, n, n, 128) == 2 * 8 * 128
+    assert _window_launch(W.window_offsets(512, 9), n, n, n, 128) == 0             # 2048 workgroups of 9 units
+    assert _window_launch(W.window_offsets(1024, 9), 4 * n, 4 * n, 4 * n, 32) == 2 * 16 * 256
+    assert _window_launch(W.window_offsets(256, 13), 256 * 256, 256 * 256, 256 * 256, 256) == 2 * 4 * 64
+    assert _window_launch(W.window_offsets(128, 13, 4), 4 * 128 * 128, 4 * 128 * 128, 4 * 128 * 128, 256) == 0
+    assert _window_launch(W.window_offsets(256, 13, 4), 4 * 256 * 256, 4 * 256 * 256, 4 * 256 * 256, 256) == 2 * 4 * 256 * 4
+    assert _window_launch(W.window_offsets(256, 11, 2), 2 * 256 * 256, 2 * 256 * 256, 2 * 256 * 256, 128) == 2 * 4 * 128 * 2
+    assert _window_launch([dy * 512 + dx for dy in range(2) for dx in range(14)], n, n, n, 128) == 0   # rows of 14
     # a period that is no multiple of 4; no window table; the headline layer (64 tiles)
     assert _window_launch(W.window_offsets(510, 7), 510 * 510, 510 * 510, 510 * 510, 128) == 0
     assert _window_launch([-5, -1, 0, 1, 9], n, n, n, 128) == 0

@@ -556,34 +556,38 @@ def test_cfg4_full_size_properties(gu):
     assert float((Y - Yg).abs().max()) <= 1e-5 * float(Yg.abs().max()), "tiled vs generic"
     del Yg, Yt
 
-    # weight gradient: G = proj(X * H^T) on the pattern, beta == 0 over NaN
-    G = new_dia(torch.zeros(nd * n, device=dev))
-    G.vec.fill_(float("nan"))
-    bd = D.dev_block_descriptor_f(G)
-    _lib.check(L.cuvdia_set_path(_lib.PATH_TILED), "set_path")
-    try:
-        D.densedense_to_dia(G, bd, X, H, 1.0 / batch, 0.0)
-        assert L.cuvdia_last_path() == _lib.PATH_TILED
-    finally:
-        L.cuvdia_set_path(_lib.PATH_AUTO)
-    Gv = G.vec.view(nd, n)
-    assert bool(torch.isnan(Gv[~valid]).all()), "padding slots were written"
-    assert bool(torch.isfinite(Gv[valid]).all()), "valid slots not written"
+    # weight gradient: G = proj(X * H^T) on the pattern, beta == 0 over NaN -- through the chunk-by-chunk kernel and
+    # through the kernel tiled in the window's plane, which the automatic choice takes at this size
+    Y2 = torch.full((batch, n), float("nan"), device=dev)
+    run_prod(Y2, A, H, "n", _lib.PATH_TILED)
     src = sample[:, None] + off[None, :]
     ok = (src >= 0) & (src < n)
     xs = X[:, sample].double()                                         # (batch, rows)
     hs = H[:, src.clamp(0, n - 1)].double()                            # (batch, rows, nd)
     ref = torch.einsum("cr,crd->dr", xs, hs) / batch
-    got = Gv[:, sample].double()
-    err = (got - ref).abs()[ok.T]
-    assert float(err.max()) <= 1e-5 * float(ref.abs().max()), "dd2dia sampled slots %.3g" % float(err.max())
-    # <proj(X H^T)/batch, A> == <A*H', X>/batch with H' = H: sum_valid G*A == <Y2, X>/batch, Y2 = A*H
-    Y2 = torch.full((batch, n), float("nan"), device=dev)
-    run_prod(Y2, A, H, "n", _lib.PATH_TILED)
-    lhs = float((torch.nan_to_num(Gv).double() * torch.nan_to_num(A.vec.view(nd, n)).double()).sum())
-    rhs = float((Y2.double() * X.double()).sum()) / batch
-    scale = float((Y2.double().abs() * X.double()).sum()) / batch
-    assert abs(lhs - rhs) <= 1e-5 * scale, ("gradient adjoint identity", lhs, rhs, scale)
+    for forced, expected in ((_lib.PATH_TILED_NOWALK, _lib.PATH_TILED), (_lib.PATH_WINDOW, _lib.PATH_WINDOW),
+                             (_lib.PATH_AUTO, _lib.PATH_WINDOW)):
+        G = new_dia(torch.zeros(nd * n, device=dev))
+        G.vec.fill_(float("nan"))
+        bd = D.dev_block_descriptor_f(G)
+        _lib.check(L.cuvdia_set_path(forced), "set_path")
+        try:
+            D.densedense_to_dia(G, bd, X, H, 1.0 / batch, 0.0)
+            assert L.cuvdia_last_path() == expected, (forced, L.cuvdia_last_kernel())
+        finally:
+            L.cuvdia_set_path(_lib.PATH_AUTO)
+        Gv = G.vec.view(nd, n)
+        assert bool(torch.isnan(Gv[~valid]).all()), "padding slots were written"
+        assert bool(torch.isfinite(Gv[valid]).all()), "valid slots not written"
+        got = Gv[:, sample].double()
+        err = (got - ref).abs()[ok.T]
+        assert float(err.max()) <= 1e-5 * float(ref.abs().max()), "dd2dia sampled slots %.3g" % float(err.max())
+        # <proj(X H^T)/batch, A> == <A*H', X>/batch with H' = H: sum_valid G*A == <Y2, X>/batch, Y2 = A*H
+        lhs = float((torch.nan_to_num(Gv).double() * torch.nan_to_num(A.vec.view(nd, n)).double()).sum())
+        rhs = float((Y2.double() * X.double()).sum()) / batch
+        scale = float((Y2.double().abs() * X.double()).sum()) / batch
+        assert abs(lhs - rhs) <= 1e-5 * scale, ("gradient adjoint identity", forced, lhs, rhs, scale)
+        del G, Gv, bd
 
 
 # ------------------------------------------------------------ avg_diagonals ---

@@ -59,6 +59,12 @@ CASES = [
     (64, 64 * 12 - 4, 64 * 12 - 8, 5, 7, -2, -3, 1, 8),    # row counts that end inside a map row
     (64, 64 * 1600, 64 * 1600, 7, 7, -3, -3, 1, 9),    # 400 tiles: two batch ranges per workgroup (the cases above: four)
     (64, 64 * 3200, 64 * 3200, 7, 7, -3, -3, 1, 5),    # 800 tiles: one
+    # window rows of 9 to 13 diagonals: a wave per window row, blocks of 7 window rows
+    (64, 64 * 14, 64 * 14, 13, 13, -6, -6, 1, 9),      # the centred 13 x 13: two blocks (7 + 6 rows), a ragged batch
+    (96, 96 * 24, 96 * 24, 9, 11, -4, -5, 2, 20),      # two groups, a narrower last tile column
+    (128, 128 * 10, 128 * 12, 8, 10, -3, -2, 1, 5),    # 7 + 1 window rows, a wider B, less than one group of columns
+    (64, 64 * 20 - 4, 64 * 20 - 8, 15, 12, -7, -6, 1, 17),     # three blocks, row counts that end inside a map row
+    (72, 72 * 9, 72 * 9, 3, 9, -1, -8, 1, 8),          # fewer window rows than waves, all shifts but one to the left
 ]
 
 
@@ -70,7 +76,8 @@ def test_window_projection_matches_the_oracle(oracle, gu, px, h, w, rows, cols, 
     C = _dia(oracle, rng, h, w, offsets)
     A, B = _operands(rng, C, batch)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0, 0.0, _lib.PATH_WINDOW, "window beta0")
-    assert ran == _lib.PATH_WINDOW and _last_kernel().startswith("dd2dia_window_kernel<%d," % cols)
+    name = "dd2dia_window_kernel<%d," if cols <= 8 else "dd2dia_window_long_kernel<%d,"
+    assert ran == _lib.PATH_WINDOW and _last_kernel().startswith(name % cols)
     tiles = -(-px // 64) * -(-(-(-h // px)) // 4) * -(-rows // 8) * channels
     assert _last_kernel().endswith(", %d>" % (1 if tiles >= 768 else 2 if tiles >= 384 else 4)) or cols != 7 or rows != 7
     C.vals[oracle.valid_mask(C)] = rng.uniform(-1, 1, int(oracle.valid_mask(C).sum())).astype(np.float32)
@@ -78,14 +85,15 @@ def test_window_projection_matches_the_oracle(oracle, gu, px, h, w, rows, cols, 
     assert ran == _lib.PATH_WINDOW
 
 
-def test_window_projection_with_padded_operands_and_a_table_in_descending_order(oracle, gu):
+@pytest.mark.parametrize("fs", [7, 13])
+def test_window_projection_with_padded_operands_and_a_table_in_descending_order(oracle, gu, fs):
     """Leading dimensions larger than the row counts (rows of the next column follow a column's last row at a
     distance), and the offsets listed from the last to the first."""
     import torch
     from cuv_amd import _lib, dia as D
     rng = np.random.default_rng(11)
-    px, n, batch = 64, 64 * 10, 12
-    offsets = _window(px, 7, 7, -3, -3)[::-1]
+    px, n, batch = 64, 64 * (fs + 3), 12
+    offsets = _window(px, fs, fs, -(fs // 2), -(fs // 2))[::-1]
     C = _dia(oracle, rng, n, n, offsets)
     A, B = _operands(rng, C, batch)
     ref = oracle.dd2dia(C, A, B, 0.5, 0.0)
@@ -109,12 +117,13 @@ def test_window_projection_with_padded_operands_and_a_table_in_descending_order(
     assert np.isnan(got[~valid]).all()
 
 
-def test_non_finite_values_stay_in_the_slots_that_use_them(oracle, gu):
+@pytest.mark.parametrize("fs", [7, 11])
+def test_non_finite_values_stay_in_the_slots_that_use_them(oracle, gu, fs):
     """An infinity in A and a NaN in B reach exactly the slots whose sums contain them."""
     from cuv_amd import _lib
     rng = np.random.default_rng(3)
-    px, n, batch = 64, 64 * 9, 8
-    C = _dia(oracle, rng, n, n, _window(px, 7, 7, -3, -3))
+    px, n, batch = 64, 64 * (fs + 2), 8
+    C = _dia(oracle, rng, n, n, _window(px, fs, fs, -(fs // 2), -(fs // 2)))
     A, B = _operands(rng, C, batch)
     A[5 * px + 17, 3] = np.inf
     B[2 * px + 40, 6] = np.nan
@@ -161,8 +170,19 @@ def test_the_choice_by_size_and_the_refusals(oracle, gu):
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0 / 32, 0.9, _lib.PATH_AUTO, "four ranges")
     assert ran == _lib.PATH_WINDOW and _last_kernel() == "dd2dia_window_kernel<7, 1, 4>"
     n = 256 * 64
-    # forced on what it does not serve: window rows of 9 diagonals, a period that is no multiple of 4, no window table
-    for offsets, b in ((_window(256, 2, 9, -1, -4), 8), (_window(254, 3, 3, -1, -1), 8), ([-5, -1, 0, 1, 9], 8)):
+    # window rows of 13 diagonals: 512 tiles of a 13 x 13 window on a 256-wide map are taken, of a 9 x 9 not
+    n = 256 * 256
+    C = _dia(oracle, rng, n, n, _window(256, 13, 13, -6, -6))
+    A, B = _operands(rng, C, 4)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 0.25, 0.9, _lib.PATH_AUTO, "long rows taken by size")
+    assert ran == _lib.PATH_WINDOW and _last_kernel() == "dd2dia_window_long_kernel<13, 2>"
+    C = _dia(oracle, rng, n, n, _window(256, 9, 9, -4, -4))
+    A, B = _operands(rng, C, 4)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 0.25, 0.9, _lib.PATH_AUTO, "long rows left alone")
+    assert ran == _lib.PATH_TILED and _last_kernel().startswith("dd2dia_tiled_kernel<9,")
+    n = 256 * 64
+    # forced on what it does not serve: window rows of 14 diagonals, a period that is no multiple of 4, no window table
+    for offsets, b in ((_window(256, 2, 14, -1, -7), 8), (_window(254, 3, 3, -1, -1), 8), ([-5, -1, 0, 1, 9], 8)):
         C = _dia(oracle, rng, n, n, offsets)
         A, B = _operands(rng, C, b)
         Cd = gu.make_dev_dia(C)
@@ -201,6 +221,30 @@ def test_random_window_shapes(oracle, gu, seed):
     alpha, beta = float(rng.choice([1.0, -0.5, 1.0 / batch])), float(rng.choice([0.0, 0.9, -1.5]))
     _, ran = gu.check_dd2dia(oracle, C, A, B, alpha, beta, _lib.PATH_WINDOW, "random window %d" % seed)
     assert ran == _lib.PATH_WINDOW
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_window_shapes_with_rows_of_9_to_13_diagonals(oracle, gu, seed):
+    """The same draw for the kernel that serves rows of 9 to 13 diagonals (a wave per window row)."""
+    from cuv_amd import _lib
+    rng = np.random.default_rng(2000 + seed)
+    px = 4 * int(rng.integers(16, 60)) if seed % 4 else 4 * int(rng.integers(5, 16))
+    rows, cols = int(rng.integers(1, 16)), int(rng.integers(9, 14))
+    dy0, dx0 = -int(rng.integers(0, rows)), -int(rng.integers(0, cols))
+    channels = int(rng.choice([1, 1, 2, 3]))
+    map_elems = px * (rows + int(rng.integers(4, 12)))
+    h = channels * map_elems - 4 * int(rng.integers(0, 3))
+    w = channels * map_elems - 4 * int(rng.integers(0, 3))
+    batch = int(rng.choice([1, 3, 7, 8, 9, 17, 32, 50]))
+    offsets = _window(px, rows, cols, dy0, dx0, channels, map_elems)
+    if seed % 3 == 0:
+        offsets = offsets[::-1]
+    stride = max(h, w) + int(rng.choice([0, 0, 1, 3, 4, 13]))
+    C = _dia(oracle, rng, h, w, offsets, stride)
+    A, B = _operands(rng, C, batch)
+    alpha, beta = float(rng.choice([1.0, -0.5, 1.0 / batch])), float(rng.choice([0.0, 0.9, -1.5]))
+    _, ran = gu.check_dd2dia(oracle, C, A, B, alpha, beta, _lib.PATH_WINDOW, "random long rows %d" % seed)
+    assert ran == _lib.PATH_WINDOW and _last_kernel().startswith("dd2dia_window_long_kernel<%d," % cols)
 
 
 def test_a_sweep_size_against_sampled_exact_sums_and_the_chunk_kernel(gu):
