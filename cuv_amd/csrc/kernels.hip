@@ -22,9 +22,9 @@
 //           A chunk pair: eight sums s_q over g = q (mod 8);
 //           p_q = s_q + s_{q+4}, then total as above.
 //           C = beta*C + alpha*total.  The generic kernel and the window-table
-//           kernel sum the batch serially in ascending column order (the latter,
-//           on launches of few tiles, as 2 or 4 ranges of the batch whose sums
-//           are added in range order).
+//           kernels sum the batch serially in ascending column order (the one
+//           for window rows of at most 8 diagonals, on launches of few tiles,
+//           as 2 or 4 ranges of the batch whose sums are added in range order).
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -2329,8 +2329,9 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
     typedef const int __attribute__((address_space(4))) *sc_int_ptr;
     const sc_int_ptr stab = (sc_int_ptr)tab;
 
-    // workgroup -> (group, block of window rows, tile row, tile column), the tile column fastest: the 64
-    // workgroups an XCD receives together are a band of neighbouring tiles, which share their stretches of B
+    // workgroup -> (group, tile row, block of window rows, tile column), the tile column fastest: the 64
+    // workgroups an XCD receives together are a band of neighbouring tiles, which share their stretches of B, and
+    // the blocks of a tall window sit side by side, where they find the tile's rows of A in the L2
     int rest = xcd_tile(blockIdx.x, gridDim.x);
     const int tx = rest % txn; rest /= txn;
     const int db = rest % ndb; rest /= ndb;
