@@ -5,6 +5,7 @@
 //   src/tests/spmv.cpp:103-129            spmv_dev_correctness{,_trans}
 //   src/tests/densedense_to_dia.cpp:109-197  dd2s_correctness_dev, dd2s_cmp_dev_host (row_fact 4)
 //   src/tests/dia_mat.cpp:103-132         spmv_uninit, spmv_host2dev
+#include <string>
 #include <cuv.hpp>
 #include <cuv_host_ops.hpp>
 
@@ -311,6 +312,32 @@ TEST_CASE(locally_connected_layer_window_projection)
     const int ran = cuvdia_last_path();
     CHECK(cuvdia_set_path(CUVDIA_PATH_AUTO) == CUVDIA_OK);
     CHECK(ran == CUVDIA_PATH_WINDOW);
+    host_block_descriptor<float> bdh(*W);
+    cuv_oracle::densedense_to_dia(*W, bdh, H, V, 1.f / batch, 0.9f);
+    MAT_CMP(*W, Wd, 0.01f);
+    delete W;
+}
+
+TEST_CASE(locally_connected_layer_wide_window_projection)
+{
+    // a 13 x 13 window on a 64 x 64 map: window rows of 13 diagonals, the kernel with a wave per window row
+    filter_factory<float, host_memory_space> ff(64, 64, 13, 1, 1);
+    dia_matrix<float, host_memory_space> *W = ff.get_dia();
+    const int N = W->h(), batch = 12;
+    for (int i = 0; i < (int)W->vec().size(); i++) W->vec()[i] = 0.01f * (float)((i * 37) % 101 + 1);
+    tensor<float, host_memory_space, column_major> V(N, batch), H(N, batch);
+    for (int i = 0; i < N * batch; i++) { V[i] = (float)((i * 13) % 7) / 7.f; H[i] = (float)((i * 29) % 11) / 11.f; }
+    dia_matrix<float, dev_memory_space> Wd(N, N, W->num_dia(), W->stride(), 1);
+    convert(Wd, *W);
+    tensor<float, dev_memory_space, column_major> Vd(V.shape()), Hd(H.shape());
+    convert(Vd, V); convert(Hd, H);
+    CHECK(cuvdia_set_path(CUVDIA_PATH_WINDOW) == CUVDIA_OK);
+    densedense_to_dia(Wd, Hd, Vd, 1.f / batch, 0.9f);
+    const int ran = cuvdia_last_path();
+    const std::string kernel = cuvdia_last_kernel();
+    CHECK(cuvdia_set_path(CUVDIA_PATH_AUTO) == CUVDIA_OK);
+    CHECK(ran == CUVDIA_PATH_WINDOW);
+    CHECK(kernel.rfind("dd2dia_window_long_kernel<13,", 0) == 0);
     host_block_descriptor<float> bdh(*W);
     cuv_oracle::densedense_to_dia(*W, bdh, H, V, 1.f / batch, 0.9f);
     MAT_CMP(*W, Wd, 0.01f);
