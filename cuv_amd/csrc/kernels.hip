@@ -33,10 +33,10 @@
 
 #include "kernels.hpp"
 
-// This file is compiled six times (CUVDIA_PART = 1 .. 6, see the Makefile), each translation unit
+// This file is compiled seven times (CUVDIA_PART = 1 .. 7, see the Makefile), each translation unit
 // instantiating one share of the kernel templates, so that the shares compile in parallel: parts 1 - 3 hold
 // the tiled SpMM kernels by longest chunk (1 - 5, 6 - 9, 10 - 13), part 5 the walking SpMM kernels, part 6
-// the window-table projection, part 4
+// the window-table projection for window rows of at most 8 diagonals, part 7 the one for rows of 9 to 13, part 4
 // everything else.  Without the macro one unit holds everything.
 #ifndef CUVDIA_PART
 #define CUVDIA_PART 0
@@ -2177,7 +2177,15 @@ __device__ __forceinline__ void dd2dia_unit(
 
 // Shape of the blocks the projection's tiles are numbered in (see the kernel): units per block and row tiles per
 // block, 64 positions or nearly.
-constexpr int DW_LONG_ROWS = 7;              // window rows per workgroup of the projection's kernel for rows of 9 to 13 diagonals
+// Window rows per workgroup (= its waves) of the projection's kernel for rows of 9 to 13 diagonals: 7 (two
+// workgroups, 14 waves, per CU) or 5 (three workgroups, 15 waves), whichever leaves fewer wave slots without a window
+// row (13 rows -> 7 + 6, 11 -> 7 + 4, 9 -> 5 + 4, 10 -> 5 + 5).  (6 -- 11 rows as 6 + 5 -- measured slower than 7 + 4:
+// two workgroups of 6 waves leave a CU 12 waves.)
+inline int dw_long_rows(int k)
+{
+    const int waste5 = (k + 4) / 5 * 5 - k, waste7 = (k + 6) / 7 * 7 - k;
+    return waste5 < waste7 ? 5 : 7;
+}
 constexpr int DW_MIN_WGS = 768;               // workgroups from which the window-table projection of a 7 x 7 window is ahead
 constexpr int DD_BLOCKED_MIN_TILES = 1024;   // launches of more than a few rounds number their tiles in blocks
 struct DdBlock {
@@ -2602,13 +2610,13 @@ __global__ __launch_bounds__(256 * SUBS, 4) void dd2dia_window_kernel(
 
 // The same tiling for window rows of 9 to 13 diagonals (a chunk of the products' table: the large layer's 13 x 13
 // window), with the roles turned round: a wave's 2 x 4 x LC sums would not fit its registers, so here a WAVE owns
-// one window row (DwLongShape::WAVES of them per workgroup; a taller window takes several workgroups per tile) and
+// one window row (5 or 7 of them per workgroup, dw_long_rows; a taller window takes several workgroups per tile) and
 // a lane's role is the y of the tile's four: 4 x LC running sums, one 16-byte read of A and one window of B
 // (4 + LC - 1 values) per column.  Staging, ring, waits and the results' way out are those of the kernel above; a
 // wave past the block's last window row only helps with the requests.
-template <int LC, int SH>
+template <int LC, int SH, int NW>
 struct DwLongShape {
-    static constexpr int WAVES = DW_LONG_ROWS, YT = 4, TX = 64;
+    static constexpr int WAVES = NW, YT = 4, TX = 64;
     static constexpr int COLS = 8;                               // batch columns per staged group
     static constexpr int NBUF = 2;                               // (3 or 4 buffers of 4 columns measured 3 - 4 % slower)
     static constexpr int WIN = SH + 4 + LC - 1;
@@ -2624,14 +2632,15 @@ struct DwLongShape {
     static_assert(NBUF >= 2 && NBUF * BUF_PIECES * 16 <= 80 * 1024, "two buffers; two workgroups per CU and to spare");
 };
 
-template <int LC, int SH>
-__global__ __launch_bounds__(64 * DW_LONG_ROWS, 4) void dd2dia_window_long_kernel(
+template <int LC, int SH, int NW>
+__global__ __launch_bounds__(64 * NW, 4) void dd2dia_window_long_kernel(
     const int *__restrict__ tab, int ngroups, int K, int period, int s0, int astep, float *__restrict__ C,
     const float *__restrict__ A, long long lda, const float *__restrict__ B, long long ldb,
     int h, int w, int batch, float alpha, float beta, unsigned a_bytes, unsigned b_bytes, unsigned c_bytes,
     int txn, int tyn, int ndb)
 {
-    typedef DwLongShape<LC, SH> S;
+    typedef DwLongShape<LC, SH, NW> S;
+    static_assert(NW == 5 || NW == 7, "waves per workgroup");
     constexpr int WAVES = S::WAVES, YT = S::YT, COLS = S::COLS, WQ = S::WQ, BPR = S::BPR, NIT = S::NIT;
     __shared__ __attribute__((aligned(16))) float lds[S::NBUF][S::BUF_PIECES * 4];
     const int lane = threadIdx.x & 63;
@@ -2946,6 +2955,7 @@ struct DwLaunch {
     hipStream_t stream;
 };
 hipError_t dd2dia_window_launch(const DwLaunch &L);
+hipError_t dd2dia_window_long_launch(const DwLaunch &L);      // (rows of 9 to 13 diagonals; a unit of its own)
 hipError_t spmm_tiled_launch_1_5(const SpLaunch &L);
 hipError_t spmm_tiled_launch_6_9(const SpLaunch &L);
 hipError_t spmm_tiled_launch_10_13(const SpLaunch &L);
@@ -3048,23 +3058,7 @@ hipError_t dd2dia_window_launch(const DwLaunch &L)
         else if (L.subs == 2) CUVDIA_DW_LAUNCH_SUBS(LC, 2);                                                           \
         else CUVDIA_DW_LAUNCH_SUBS(LC, 1);                                                                            \
         break;
-    if (L.lck > CHUNK_MAX) {
-        if (L.subs != 1) return hipErrorNotSupported;
-        note_kernel("dd2dia_window_long_kernel<%d, %d>", L.lck, sh);
-#define CUVDIA_DWL_LAUNCH(LC)                                                                                          \
-    case LC:                                                                                                           \
-        if (sh == 0) hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 0>), grid, dim3(64 * DwLongShape<LC, 0>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
-        else if (sh == 1) hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 1>), grid, dim3(64 * DwLongShape<LC, 1>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
-        else if (sh == 2) hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 2>), grid, dim3(64 * DwLongShape<LC, 2>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
-        else hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, 3>), grid, dim3(64 * DwLongShape<LC, 3>::WAVES), 0, L.stream, CUVDIA_DW_ARGS); \
-        break;
-        switch (L.lck) {
-            CUVDIA_DWL_LAUNCH(9) CUVDIA_DWL_LAUNCH(10) CUVDIA_DWL_LAUNCH(11) CUVDIA_DWL_LAUNCH(12) CUVDIA_DWL_LAUNCH(13)
-            default: return hipErrorNotSupported;
-        }
-#undef CUVDIA_DWL_LAUNCH
-        return hipGetLastError();
-    }
+    if (L.lck > CHUNK_MAX) return L.subs == 1 ? dd2dia_window_long_launch(L) : hipErrorNotSupported;
     note_kernel("dd2dia_window_kernel<%d, %d, %d>", L.lck, sh, L.subs);
     switch (L.lck) {
         CUVDIA_DW_LAUNCH(2) CUVDIA_DW_LAUNCH(3) CUVDIA_DW_LAUNCH(4) CUVDIA_DW_LAUNCH(5)
@@ -3074,6 +3068,40 @@ hipError_t dd2dia_window_launch(const DwLaunch &L)
 #undef CUVDIA_DW_LAUNCH
 #undef CUVDIA_DW_LAUNCH_SUBS
 #undef CUVDIA_DW_ARGS
+    return hipGetLastError();
+}
+#endif
+#if CUVDIA_IN_PART(7)
+hipError_t dd2dia_window_long_launch(const DwLaunch &L)
+{
+    const long long blocks = (long long)L.ngroups * L.ndb * L.tyn * L.txn;
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)blocks);
+    const int sh = ((L.s0 % 4) + 4) % 4;
+    const int nw = dw_long_rows(L.k);
+#define CUVDIA_DWL_ARGS L.tab, L.ngroups, L.k, L.period, L.s0, L.astep, L.vals, L.A, L.lda, L.B, L.ldb, L.h, L.w, L.batch, \
+                        L.alpha, L.beta, L.a_bytes, L.b_bytes, L.c_bytes, L.txn, L.tyn, L.ndb
+#define CUVDIA_DWL_LAUNCH_NW(LC, SH)                                                                                   \
+    do {                                                                                                               \
+        if (nw == 5) hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, SH, 5>), grid, dim3(320), 0, L.stream, CUVDIA_DWL_ARGS); \
+        else hipLaunchKernelGGL((dd2dia_window_long_kernel<LC, SH, 7>), grid, dim3(448), 0, L.stream, CUVDIA_DWL_ARGS); \
+    } while (0)
+#define CUVDIA_DWL_LAUNCH(LC)                                                                                          \
+    case LC:                                                                                                           \
+        if (sh == 0) CUVDIA_DWL_LAUNCH_NW(LC, 0);                                                                      \
+        else if (sh == 1) CUVDIA_DWL_LAUNCH_NW(LC, 1);                                                                 \
+        else if (sh == 2) CUVDIA_DWL_LAUNCH_NW(LC, 2);                                                                 \
+        else CUVDIA_DWL_LAUNCH_NW(LC, 3);                                                                              \
+        break;
+    if (nw != 5 && nw != 7) return hipErrorNotSupported;
+    note_kernel("dd2dia_window_long_kernel<%d, %d, %d>", L.lck, sh, nw);
+    switch (L.lck) {
+        CUVDIA_DWL_LAUNCH(9) CUVDIA_DWL_LAUNCH(10) CUVDIA_DWL_LAUNCH(11) CUVDIA_DWL_LAUNCH(12) CUVDIA_DWL_LAUNCH(13)
+        default: return hipErrorNotSupported;
+    }
+#undef CUVDIA_DWL_LAUNCH
+#undef CUVDIA_DWL_LAUNCH_NW
+#undef CUVDIA_DWL_ARGS
     return hipGetLastError();
 }
 #endif
@@ -3255,7 +3283,7 @@ long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn, int *t
         return 0;
     const long long image_rows = ((long long)C.h + wk.period - 1) / wk.period;
     const long long tx = ((long long)wk.period + 63) / 64, ty = (image_rows + 3) / 4,
-                    db = wk.lck > CHUNK_MAX ? (wk.k + DW_LONG_ROWS - 1) / DW_LONG_ROWS : (wk.k + 7) / 8;
+                    db = wk.lck > CHUNK_MAX ? (wk.k + dw_long_rows(wk.k) - 1) / dw_long_rows(wk.k) : (wk.k + 7) / 8;
     const long long total = tx * ty * db * wk.ngroups;
     if (total > 0x7fffffffLL || (long long)4 * ty * wk.period + 64 * tx >= (1LL << 30)) return 0;
     if (txn) *txn = (int)tx;
@@ -3288,13 +3316,16 @@ bool dd2dia_window_by_size(const DiaView &C, int batch, long long workgroups)
     const int subs = dd2dia_window_subs(C, workgroups);
     if (C.walk_n.period < 64) return false;
     if (C.walk_n.lck > CHUNK_MAX) {
-        // Rows of 9 to 13 diagonals: a tile saves the more the more units (window rows x groups) shared its rows
-        // under the chunk-by-chunk kernel.  Measured on 9 x 9 to 13 x 13 windows, 1 to 4 channels, maps 128 to 1024
-        // wide, batch 16 to 1024: 1.04 - 1.48 times its rate where taken, 0.75 - 1.0 where not.
+        // Rows of 9 to 13 diagonals.  Measured on 9 x 9 to 13 x 13 windows, 1 to 4 channels, maps 128 to 1024 wide,
+        // batch 16 to 1024: 1.08 - 1.5 times the chunk-by-chunk kernel's rate where taken, 0.75 - 1.0 where not
+        // (windows of 11 rows -- 11 of 14 wave slots -- of one channel, maps 128 wide).
+        const int nw = dw_long_rows(C.walk_n.k), blocks = (C.walk_n.k + nw - 1) / nw;
+        const bool full = C.walk_n.k * 10 >= blocks * nw * 9;      // at most a tenth of the wave slots idle
         const int units = C.walk_n.k * C.walk_n.ngroups;
-        if (C.walk_n.period < 192) return false;        // (four channels of 13 x 13 on a 128-wide map: 0.75)
+        if (C.walk_n.period < 192) return false;
         if (workgroups >= 4096) return true;
-        return units >= 13 && (workgroups >= 1024 || (workgroups >= 512 && C.walk_n.period >= 256));
+        if (full) return workgroups >= 1024 || (workgroups >= 512 && C.walk_n.period >= 256);
+        return units >= 22 && workgroups >= 1024;
     }
     if (subs * workgroups < min_wgs) return false;
     if (subs == 1) return slots >= 25 || batch >= 128;

@@ -346,15 +346,20 @@ def test_window_projection_launch_by_table_shape_and_size():
     # 13 window rows of 7 diagonals: two blocks of 8 window rows per tile
     tall = [dy * 512 + dx for dy in range(-6, 7) for dx in range(-3, 4)]
     assert _window_launch(tall, n, n, n, 128) == 2 * 8 * 128
-    # window rows of 9 to 13 diagonals: blocks of 7 window rows; on maps at least 192 wide taken from 4096
-    # workgroups, or from 1024 (512 on maps at least 256 wide) when window rows x channel groups are at least 13
+    # window rows of 9 to 13 diagonals: blocks of 7 or 5 window rows (13 -> 7 + 6, 9 -> 5 + 4, 11 -> 7 + 4); on maps
+    # at least 192 wide taken from 4096 workgroups, from 1024 (512 on maps at least 256 wide) when the blocks are at
+    # least nine tenths full, from 1024 when window rows x channel groups are at least 22
     assert _window_launch(W.window_offsets(512, 13), n, n, n, 128) == 2 * 8 * 128
-    assert _window_launch(W.window_offsets(512, 9), n, n, n, 128) == 0             # 2048 workgroups of 9 units
-    assert _window_launch(W.window_offsets(1024, 9), 4 * n, 4 * n, 4 * n, 32) == 2 * 16 * 256
+    assert _window_launch(W.window_offsets(512, 9), n, n, n, 128) == 2 * 8 * 128
+    assert _window_launch(W.window_offsets(512, 11), n, n, n, 128) == 0            # 11 of 14 slots, one channel
+    assert _window_launch(W.window_offsets(1024, 11), 4 * n, 4 * n, 4 * n, 32) == 2 * 16 * 256
     assert _window_launch(W.window_offsets(256, 13), 256 * 256, 256 * 256, 256 * 256, 256) == 2 * 4 * 64
+    assert _window_launch(W.window_offsets(256, 9), 256 * 256, 256 * 256, 256 * 256, 256) == 2 * 4 * 64
+    assert _window_launch(W.window_offsets(192, 9), 192 * 192, 192 * 192, 192 * 192, 256) == 0      # 288 workgroups
     assert _window_launch(W.window_offsets(128, 13, 4), 4 * 128 * 128, 4 * 128 * 128, 4 * 128 * 128, 256) == 0
     assert _window_launch(W.window_offsets(256, 13, 4), 4 * 256 * 256, 4 * 256 * 256, 4 * 256 * 256, 256) == 2 * 4 * 256 * 4
     assert _window_launch(W.window_offsets(256, 11, 2), 2 * 256 * 256, 2 * 256 * 256, 2 * 256 * 256, 128) == 2 * 4 * 128 * 2
+    assert _window_launch(W.window_offsets(256, 15), 256 * 256, 256 * 256, 256 * 256, 64) == 0      # rows of 15
     assert _window_launch([dy * 512 + dx for dy in range(2) for dx in range(14)], n, n, n, 128) == 0   # rows of 14
     # a period that is no multiple of 4; no window table; the headline layer (64 tiles)
     assert _window_launch(W.window_offsets(510, 7), 510 * 510, 510 * 510, 510 * 510, 128) == 0

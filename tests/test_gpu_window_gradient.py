@@ -170,16 +170,21 @@ def test_the_choice_by_size_and_the_refusals(oracle, gu):
     _, ran = gu.check_dd2dia(oracle, C, A, B, 1.0 / 32, 0.9, _lib.PATH_AUTO, "four ranges")
     assert ran == _lib.PATH_WINDOW and _last_kernel() == "dd2dia_window_kernel<7, 1, 4>"
     n = 256 * 64
-    # window rows of 13 diagonals: 512 tiles of a 13 x 13 window on a 256-wide map are taken, of a 9 x 9 not
+    # window rows of 9 to 13 diagonals: 512 workgroups of a 13 x 13 or a 9 x 9 window on a 256-wide map are taken
+    # (blocks of 7 and of 5 window rows), of an 11 x 11 (11 of 14 wave slots) not
     n = 256 * 256
     C = _dia(oracle, rng, n, n, _window(256, 13, 13, -6, -6))
     A, B = _operands(rng, C, 4)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 0.25, 0.9, _lib.PATH_AUTO, "long rows taken by size")
-    assert ran == _lib.PATH_WINDOW and _last_kernel() == "dd2dia_window_long_kernel<13, 2>"
+    assert ran == _lib.PATH_WINDOW and _last_kernel() == "dd2dia_window_long_kernel<13, 2, 7>"
     C = _dia(oracle, rng, n, n, _window(256, 9, 9, -4, -4))
     A, B = _operands(rng, C, 4)
+    _, ran = gu.check_dd2dia(oracle, C, A, B, 0.25, 0.9, _lib.PATH_AUTO, "9 rows: blocks of 5")
+    assert ran == _lib.PATH_WINDOW and _last_kernel() == "dd2dia_window_long_kernel<9, 0, 5>"
+    C = _dia(oracle, rng, n, n, _window(256, 11, 11, -5, -5))
+    A, B = _operands(rng, C, 4)
     _, ran = gu.check_dd2dia(oracle, C, A, B, 0.25, 0.9, _lib.PATH_AUTO, "long rows left alone")
-    assert ran == _lib.PATH_TILED and _last_kernel().startswith("dd2dia_tiled_kernel<9,")
+    assert ran == _lib.PATH_TILED and _last_kernel().startswith("dd2dia_tiled_kernel<11,")
     n = 256 * 64
     # forced on what it does not serve: window rows of 14 diagonals, a period that is no multiple of 4, no window table
     for offsets, b in ((_window(256, 2, 14, -1, -7), 8), (_window(254, 3, 3, -1, -1), 8), ([-5, -1, 0, 1, 9], 8)):
