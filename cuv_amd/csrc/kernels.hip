@@ -2179,12 +2179,18 @@ __device__ __forceinline__ void dd2dia_unit(
 // block, 64 positions or nearly.
 // Window rows per workgroup (= its waves) of the projection's kernel for rows of 9 to 13 diagonals: 7 (two
 // workgroups, 14 waves, per CU) or 5 (three workgroups, 15 waves), whichever leaves fewer wave slots without a window
-// row (13 rows -> 7 + 6, 11 -> 7 + 4, 9 -> 5 + 4, 10 -> 5 + 5).  (6 -- 11 rows as 6 + 5 -- measured slower than 7 + 4:
-// two workgroups of 6 waves leave a CU 12 waves.)
-inline int dw_long_rows(int k)
+// row (13 rows -> 7 + 6, 11 -> 7 + 4, 9 -> 5 + 4, 10 -> 5 + 5) -- 5 only where three workgroups' staging buffers fit
+// a CU's 160 KB of LDS (two workgroups of 5 waves: 13 x 13 in blocks of 5 took 1.72 ms on the large layer against
+// 1.17).  (6 -- 11 rows as 6 + 5 -- measured slower than 7 + 4: two workgroups of 6 waves leave a CU 12 waves.)
+// lck: diagonals of a window row; s0: the table's first shift.
+inline int dw_long_rows(int k, int lck, int s0)
 {
     const int waste5 = (k + 4) / 5 * 5 - k, waste7 = (k + 6) / 7 * 7 - k;
-    return waste5 < waste7 ? 5 : 7;
+    // the staging buffers of a workgroup of 5 waves (DwLongShape<lck, sh, 5>: 2 buffers of 8 columns)
+    const int sh = ((s0 % 4) + 4) % 4, wq = (sh + 4 + lck - 1 + 3) / 4, bpr = 16 + wq - 1;
+    const int buf_pieces = (8 * (4 - 1 + 5) * bpr + 63) / 64 * 64 + 8 * 4 * 16;
+    const bool three_fit = 3 * 2 * buf_pieces * 16 <= 160 * 1024;
+    return waste5 < waste7 && three_fit ? 5 : 7;
 }
 constexpr int DW_MIN_WGS = 768;               // workgroups from which the window-table projection of a 7 x 7 window is ahead
 constexpr int DD_BLOCKED_MIN_TILES = 1024;   // launches of more than a few rounds number their tiles in blocks
@@ -2641,6 +2647,7 @@ __global__ __launch_bounds__(64 * NW, 4) void dd2dia_window_long_kernel(
 {
     typedef DwLongShape<LC, SH, NW> S;
     static_assert(NW == 5 || NW == 7, "waves per workgroup");
+    static_assert(S::COLS == 8 && S::NBUF == 2 && S::YT == 4 && S::TX == 64, "dw_long_rows computes the buffers' size from these");
     constexpr int WAVES = S::WAVES, YT = S::YT, COLS = S::COLS, WQ = S::WQ, BPR = S::BPR, NIT = S::NIT;
     __shared__ __attribute__((aligned(16))) float lds[S::NBUF][S::BUF_PIECES * 4];
     const int lane = threadIdx.x & 63;
@@ -3078,7 +3085,7 @@ hipError_t dd2dia_window_long_launch(const DwLaunch &L)
     if (blocks <= 0 || blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)blocks);
     const int sh = ((L.s0 % 4) + 4) % 4;
-    const int nw = dw_long_rows(L.k);
+    const int nw = dw_long_rows(L.k, L.lck, L.s0);
 #define CUVDIA_DWL_ARGS L.tab, L.ngroups, L.k, L.period, L.s0, L.astep, L.vals, L.A, L.lda, L.B, L.ldb, L.h, L.w, L.batch, \
                         L.alpha, L.beta, L.a_bytes, L.b_bytes, L.c_bytes, L.txn, L.tyn, L.ndb
 #define CUVDIA_DWL_LAUNCH_NW(LC, SH)                                                                                   \
@@ -3283,7 +3290,7 @@ long long dd2dia_window_workgroups(const DiaView &C, int batch, int *txn, int *t
         return 0;
     const long long image_rows = ((long long)C.h + wk.period - 1) / wk.period;
     const long long tx = ((long long)wk.period + 63) / 64, ty = (image_rows + 3) / 4,
-                    db = wk.lck > CHUNK_MAX ? (wk.k + dw_long_rows(wk.k) - 1) / dw_long_rows(wk.k) : (wk.k + 7) / 8;
+                    db = wk.lck > CHUNK_MAX ? (wk.k + dw_long_rows(wk.k, wk.lck, wk.s0) - 1) / dw_long_rows(wk.k, wk.lck, wk.s0) : (wk.k + 7) / 8;
     const long long total = tx * ty * db * wk.ngroups;
     if (total > 0x7fffffffLL || (long long)4 * ty * wk.period + 64 * tx >= (1LL << 30)) return 0;
     if (txn) *txn = (int)tx;
@@ -3319,7 +3326,7 @@ bool dd2dia_window_by_size(const DiaView &C, int batch, long long workgroups)
         // Rows of 9 to 13 diagonals.  Measured on 9 x 9 to 13 x 13 windows, 1 to 4 channels, maps 128 to 1024 wide,
         // batch 16 to 1024: 1.08 - 1.5 times the chunk-by-chunk kernel's rate where taken, 0.75 - 1.0 where not
         // (windows of 11 rows -- 11 of 14 wave slots -- of one channel, maps 128 wide).
-        const int nw = dw_long_rows(C.walk_n.k), blocks = (C.walk_n.k + nw - 1) / nw;
+        const int nw = dw_long_rows(C.walk_n.k, C.walk_n.lck, C.walk_n.s0), blocks = (C.walk_n.k + nw - 1) / nw;
         const bool full = C.walk_n.k * 10 >= blocks * nw * 9;      // at most a tenth of the wave slots idle
         const int units = C.walk_n.k * C.walk_n.ngroups;
         if (C.walk_n.period < 192) return false;
