@@ -119,8 +119,9 @@ int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap
  * kernel tiled in the window's plane for an h x w matrix with this table
  * (row_fact 1) and `batch` packed dense columns?  Returns the number of
  * workgroups of that launch (tiles of 4 x 64 positions x blocks of 8 window
- * rows -- of 7 or 5 where a window row has 9 to 13 diagonals, whichever
- * leaves fewer rows of the last block empty -- x channel groups), or 0 when the chunk-by-chunk kernel serves: the table is no
+ * rows -- of 7 where a window row has 9 to 13 diagonals, or of 5 where that
+ * leaves fewer rows of the last block empty and the staging buffers of three
+ * workgroups fit a CU's LDS -- x channel groups), or 0 when the chunk-by-chunk kernel serves: the table is no
  * window table (see cuvdia_plan_walk) of chunks of 2 to 13 diagonals, the
  * period, a channel distance or a row count is no multiple of 4, the period
  * is below 64, or the launch has too few workgroups to fill the chip.  For
@@ -129,8 +130,9 @@ int cuvdia_plan_units(const int *offsets_host, int nd, int *c1, int *c2, int cap
  * then works two or four ranges of the batch side by side --, 1024 from 25
  * slots, 1536 and a batch of at least 128 below.  For chunks of 9 to 13, on
  * periods of at least 192: 4096; or 1024 (512 on periods of at least 256)
- * when the blocks of window rows are at least nine tenths full (9, 10, 13
- * to 15 rows); or 1024 when window rows x channel groups are at least 22.
+ * when the blocks of window rows are at least nine tenths full (13 and 14
+ * rows; 9, 10 and 15 in blocks of 5); or 1024 when window rows x channel
+ * groups are at least 22.
  * Negative: an error.
  * cuvdia_set_path(CUVDIA_PATH_WINDOW) waives the conditions on the period's
  * size, the workgroups and the batch.  No counterpart in the reference. */
