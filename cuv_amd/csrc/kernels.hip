@@ -1469,12 +1469,14 @@ __device__ __forceinline__ void walk_steps(F &step, int u0, int nsteps)
     }
 }
 
-template <int LCK, int K, int T, int SH>
+// EP = true: a tile leaves through `ep` (a bias per output row and/or the logistic sigmoid; a sampled result,
+// ep.act == 2, stays with the tile-by-tile kernel, whose exit holds a row per lane as the generator wants it).
+template <int LCK, int K, int T, int SH, bool EP>
 __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) void spmm_walk_kernel(
     const int *__restrict__ tab,            // group_rows[ngroups], then aoff4[ngroups * K]
     int ngroups, int period, int s0, int astep4, int seg_tiles, const float *__restrict__ vals,
     const float *__restrict__ X, long long ldx, float *__restrict__ Y, long long ldy,
-    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes)
+    int n_out, int n_in, int batch, float alpha, float beta, int col_tiles, unsigned a_bytes, SpEpilogue ep)
 {
     typedef WalkShape<LCK, K, T, SH> S;
     constexpr int WAVES = S::WAVES, ROWS = S::ROWS, XQ = S::XQ, XPITCH = S::XPITCH, AI = S::AI, ATILE = S::ATILE, WQ = S::WQ;
@@ -1703,6 +1705,19 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
             } else {
 #pragma unroll
                 for (int q = 0; q < NST; ++q) v[q] = beta * ypre[q] + alpha * v[q];
+            }
+            if constexpr (EP) {
+                // the lane's 4 rows are the same in every column it stores: one bias value each
+                float b4[4] = {0.f, 0.f, 0.f, 0.f};
+                if (ep.bias) {
+                    const float *bp = ep.bias + (row_first + m * period) + 4 * (lane % LPC);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) b4[e] = bp[e];
+                }
+#pragma unroll
+                for (int q = 0; q < NST; ++q)
+                    v[q] = f4u{sp_finish(v[q].x, b4[0], ep.act), sp_finish(v[q].y, b4[1], ep.act),
+                               sp_finish(v[q].z, b4[2], ep.act), sp_finish(v[q].w, b4[3], ep.act)};
             }
 #pragma unroll
             for (int q = 0; q < NST; ++q)       // non-temporal, like every result of the library
@@ -2943,6 +2958,7 @@ struct WalkLaunch {
     int col_tiles;
     unsigned a_bytes;
     hipStream_t stream;
+    SpEpilogue ep;              // bias and/or sigmoid at the tiles' exit (act == 2 is not served)
 };
 hipError_t spmm_walk_launch(const WalkLaunch &L);
 // The window-table projection's launch (its unit instantiates the kernel for every chunk length and alignment).
@@ -3034,11 +3050,19 @@ hipError_t spmm_walk_launch(const WalkLaunch &L)
     const int nseg = (walk_len + L.seg_tiles - 1) / L.seg_tiles;
     const dim3 grid((unsigned)((long long)nseg * tp * L.col_tiles));
 #define CUVDIA_WALK_ARGS L.tab, L.ngroups, L.period, L.s0, L.astep4, L.seg_tiles, L.vals, L.B, L.ldb, L.dst, L.ldd, \
-                         L.n_out, L.n_in, L.batch, L.alpha, L.beta, L.col_tiles, L.a_bytes
-    note_kernel("spmm_walk_kernel<%d, %d, 8, %d>", L.lck, L.lck, L.lck == 7 ? 1 : L.lck == 5 ? 2 : 3);
-    if (L.lck == 7) hipLaunchKernelGGL((spmm_walk_kernel<7, 7, 8, 1>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
-    else if (L.lck == 5) hipLaunchKernelGGL((spmm_walk_kernel<5, 5, 8, 2>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
-    else hipLaunchKernelGGL((spmm_walk_kernel<3, 3, 8, 3>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS);
+                         L.n_out, L.n_in, L.batch, L.alpha, L.beta, L.col_tiles, L.a_bytes, L.ep
+    if (L.ep.act == 2) return hipErrorNotSupported;
+    const bool fused = L.ep.bias != nullptr || L.ep.act != 0;
+    note_kernel("spmm_walk_kernel<%d, %d, 8, %d, %s>", L.lck, L.lck, L.lck == 7 ? 1 : L.lck == 5 ? 2 : 3, fused ? "true" : "false");
+#define CUVDIA_WALK_LAUNCH(LCK, SH)                                                                                    \
+    do {                                                                                                               \
+        if (fused) hipLaunchKernelGGL((spmm_walk_kernel<LCK, LCK, 8, SH, true>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS); \
+        else hipLaunchKernelGGL((spmm_walk_kernel<LCK, LCK, 8, SH, false>), grid, dim3(512), 0, L.stream, CUVDIA_WALK_ARGS); \
+    } while (0)
+    if (L.lck == 7) CUVDIA_WALK_LAUNCH(7, 1);
+    else if (L.lck == 5) CUVDIA_WALK_LAUNCH(5, 2);
+    else CUVDIA_WALK_LAUNCH(3, 3);
+#undef CUVDIA_WALK_LAUNCH
 #undef CUVDIA_WALK_ARGS
     return hipGetLastError();
 }
@@ -3166,11 +3190,12 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     // along the rows and find each other's dense rows in its L2.
     const int col_group = col_tiles <= 4 ? (int)col_tiles : 2;
     const int lck = trans ? A.max_len_t : A.max_len_n;
-    // A window table on a product of many tiles: the walking kernel (plain products only).
+    // A window table on a product of many tiles: the walking kernel (with a bias and the sigmoid at its tiles' exit,
+    // if asked for; a sampled result stays with the tile-by-tile kernel).
     const WalkView &wk = trans ? A.walk_t : A.walk_n;
-    if (walk >= 0 && wk.tab_dev != nullptr && ep.bias == nullptr && ep.act == 0) {
+    if (walk >= 0 && wk.tab_dev != nullptr && ep.act != 2) {
         WalkLaunch W{wk.tab_dev, wk.ngroups, wk.period, wk.s0, wk.astep4, wk.lck, wk.k, 0, vals, B, ldb, dst, ldd,
-                     n_out, n_in, batch, alpha, beta, (int)col_tiles, (unsigned)((long long)A.nd * A.stride * 4), stream};
+                     n_out, n_in, batch, alpha, beta, (int)col_tiles, (unsigned)((long long)A.nd * A.stride * 4), stream, ep};
         const int seg_tiles = spmm_walk_plan(wk.lck, wk.k, wk.s0, wk.period, n_out, n_in, col_tiles, walk > 0, nullptr);
         if (seg_tiles > 0) {
             W.seg_tiles = seg_tiles;

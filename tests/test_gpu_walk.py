@@ -66,6 +66,53 @@ def test_walk_matches_the_oracle(oracle, gu, px, fs, channels, batch, trans):
     assert ran == _lib.PATH_WALK
 
 
+@pytest.mark.parametrize("px,fs,channels,batch", [(64, 7, 1, 70), (128, 5, 1, 33), (64, 3, 2, 64)])
+@pytest.mark.parametrize("trans", ["n", "t"])
+def test_walk_with_bias_and_sigmoid_at_the_tiles_exit(oracle, gu, px, fs, channels, batch, trans):
+    """dst = sigmoid(beta*dst + alpha*op(A)*B + bias) through the walking kernel against the reference's three host
+    steps; a sampled result is refused (the tile-by-tile kernel serves it).  Tolerances as for the tile-by-tile
+    kernel: 0.25e-5 * magnitude + 4e-7 behind the sigmoid, 1e-5 * magnitude without."""
+    import torch
+    from cuv_amd import dia as D, _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(px + fs + channels + batch)
+    n = px * px * channels
+    A = _window_dia(oracle, rng, n, n, px, fs, channels)
+    B, dst0 = _operands(rng, A, batch, trans)
+    bias = rng.uniform(-2, 2, n).astype(np.float32)
+    dev = gu.make_dev_dia(A)
+    Bd = D.to_device_colmajor(B)
+    bd = torch.from_numpy(bias).cuda()
+    for (alpha, beta, use_bias, act) in ((1.0, 0.0, True, True), (0.5, -1.5, True, True), (1.0, 0.0, True, False),
+                                         (2.0, 0.25, False, True)):
+        dd = D.to_device_colmajor(dst0) if beta != 0 else torch.full((batch, n), float("nan"), device="cuda:0")
+        _lib.check(L.cuvdia_set_path(_lib.PATH_WALK), "set_path")
+        try:
+            D.prod_bias_act(dd, dev, Bd, trans, alpha, beta, bd if use_bias else None,
+                            _lib.ACT_SIGMOID if act else _lib.ACT_NONE)
+            assert L.cuvdia_last_path() == _lib.PATH_WALK
+            assert L.cuvdia_last_kernel().decode().endswith(", true>")
+        finally:
+            L.cuvdia_set_path(_lib.PATH_AUTO)
+        got = D.to_host_colmajor(dd).astype(np.float64)
+        ref = oracle.prod_bias_act(A, B, dst0 if beta != 0 else None, trans, alpha, beta,
+                                   bias if use_bias else None, act).astype(np.float64)
+        mag = oracle.prod_mag(A, B, dst0 if beta != 0 else None, trans, alpha, beta)
+        if use_bias:
+            mag = mag + np.abs(bias)[:, None]
+        assert np.isfinite(got).all()
+        tol = (0.25e-5 * mag + 4e-7) if act else (1e-5 * mag + 1e-30)
+        assert np.all(np.abs(got - ref) <= tol), (alpha, beta, use_bias, act, float((np.abs(got - ref) / tol).max()))
+    dd = torch.full((batch, n), float("nan"), device="cuda:0")
+    L.cuvdia_set_path(_lib.PATH_WALK)
+    try:
+        with pytest.raises(_lib.CuvDiaError) as err:
+            D.prod_bias_act(dd, dev, Bd, trans, 1.0, 0.0, bd, _lib.ACT_SIGMOID_SAMPLE, seed=5)
+    finally:
+        L.cuvdia_set_path(_lib.PATH_AUTO)
+    assert err.value.code == _lib.EUNSUPPORTED
+
+
 @pytest.mark.parametrize("trans", ["n", "t"])
 def test_walk_on_a_rectangular_matrix_with_a_short_last_segment(oracle, gu, trans):
     """60 row tiles per walk: the last segment is shorter than the others, and the window hangs over the
