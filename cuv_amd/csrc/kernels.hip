@@ -1469,8 +1469,9 @@ __device__ __forceinline__ void walk_steps(F &step, int u0, int nsteps)
     }
 }
 
-// EP = true: a tile leaves through `ep` (a bias per output row and/or the logistic sigmoid; a sampled result,
-// ep.act == 2, stays with the tile-by-tile kernel, whose exit holds a row per lane as the generator wants it).
+// EP = true: a tile leaves through `ep` (a bias per output row and/or the logistic sigmoid).  A sampled result,
+// ep.act == 2, leaves row by row instead -- a lane holds one row of its wave's 8 columns, two aligned blocks of 4,
+// as the generator's counter (row, column / 4) wants them; 64 consecutive rows of a column per store.
 template <int LCK, int K, int T, int SH, bool EP>
 __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) void spmm_walk_kernel(
     const int *__restrict__ tab,            // group_rows[ngroups], then aoff4[ngroups * K]
@@ -1681,6 +1682,7 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
     }
     const __amdgpu_buffer_rsrc_t yr = make_rsrc(
         Y + (long long)col0 * ldy, (unsigned)(((long long)(cols_here - 1) * ldy + n_out) * 4));
+    const bool by_row = EP && ep.act == 2;      // (kernel-uniform) the sampled result leaves row by row
     // Stores the tile that step u completes (m = u - K + 1, set (UU + 1) mod K) and clears its set for the tile
     // K steps on.  `ilast` is the step's last block: every wave is through with its buffer (the barrier that
     // ended the block), and the next request into it comes after the second barrier below.
@@ -1695,6 +1697,34 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
                 *reinterpret_cast<float4 *>(out + o_write + t) =
                     make_float4(acc[SET][t], acc[SET][t + 1], acc[SET][t + 2], acc[SET][t + 3]);
             __syncthreads();
+            if (EP && by_row) {
+                static_assert(CPW == 4 * NST && CPW % 4 == 0 && ROWS == 64, "a row per lane, the wave's columns in blocks of 4");
+                float vv[CPW];
+#pragma unroll
+                for (int q = 0; q < CPW; ++q) vv[q] = out[(wave * CPW + q) * OPITCH + lane];
+                const unsigned row = (unsigned)(row_first + m * period + lane);
+                const float bias = ep.bias ? ep.bias[row] : 0.f;
+                SpRand4 rnd[CPW / 4];
+#pragma unroll
+                for (int k = 0; k < CPW / 4; ++k)
+                    rnd[k] = sp_philox(row, (unsigned)(col0 + wave * CPW) / 4u + k, ep.seed_lo, ep.seed_hi);
+                const float yp[CPW] = {ypre[0].x, ypre[0].y, ypre[0].z, ypre[0].w, ypre[1].x, ypre[1].y, ypre[1].z, ypre[1].w};
+                const unsigned tile_off = (unsigned)(row_first + m * period) * 4u;  // wave-uniform
+#pragma unroll
+                for (int q = 0; q < CPW; ++q) {
+                    const int col = wave * CPW + q;                                 // wave-uniform
+                    if (col < cols_here) {
+                        const float r = (beta == 0.f) ? alpha * vv[q] : beta * yp[q] + alpha * vv[q];
+                        __builtin_amdgcn_raw_buffer_store_b32(
+                            __builtin_bit_cast(unsigned, sp_finish(r, bias, ep.act, rnd[q / 4].w[q & 3])), yr,
+                            (unsigned)lane * 4u, tile_off + (unsigned)(col * ldy) * 4u, 2);
+                    }
+                }
+                __syncthreads();
+#pragma unroll
+                for (int t = 0; t < T; ++t) acc[SET][t] = 0.f;
+                return;
+            }
             f4u v[NST];
 #pragma unroll
             for (int q = 0; q < NST; ++q) v[q] = *reinterpret_cast<const f4u *>(out + o_read[q]);
@@ -1739,9 +1769,23 @@ __global__ __launch_bounds__(512, (WalkShape<LCK, K, T, SH>::WAVES_PER_SIMD)) vo
         const int mf = u - (K - 1);
         if (beta != 0.f && mf >= 0 && mf < ntiles) {
             const unsigned tile_off = (unsigned)(row_first + mf * period) * 4u;
+            if (EP && by_row) {
+                // (the row-by-row exit: this lane's row of the wave's 8 columns)
+                float yp[CPW];
 #pragma unroll
-            for (int q = 0; q < NST; ++q)
-                ypre[q] = __builtin_bit_cast(f4u, __builtin_amdgcn_raw_buffer_load_b128(yr, y_lane[q], tile_off, 0));
+                for (int q = 0; q < CPW; ++q) {
+                    const int col = wave * CPW + q;
+                    yp[q] = col < cols_here ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                  yr, (unsigned)lane * 4u, tile_off + (unsigned)(col * ldy) * 4u, 0))
+                                            : 0.f;
+                }
+                ypre[0] = f4u{yp[0], yp[1], yp[2], yp[3]};
+                ypre[1] = f4u{yp[4], yp[5], yp[6], yp[7]};
+            } else {
+#pragma unroll
+                for (int q = 0; q < NST; ++q)
+                    ypre[q] = __builtin_bit_cast(f4u, __builtin_amdgcn_raw_buffer_load_b128(yr, y_lane[q], tile_off, 0));
+            }
         }
         int i = u * ngroups;
         for (int g = 0; g < ngroups; ++g, ++i) {
@@ -2958,7 +3002,7 @@ struct WalkLaunch {
     int col_tiles;
     unsigned a_bytes;
     hipStream_t stream;
-    SpEpilogue ep;              // bias and/or sigmoid at the tiles' exit (act == 2 is not served)
+    SpEpilogue ep;              // bias, sigmoid and sample at the tiles' exit
 };
 hipError_t spmm_walk_launch(const WalkLaunch &L);
 // The window-table projection's launch (its unit instantiates the kernel for every chunk length and alignment).
@@ -3051,7 +3095,6 @@ hipError_t spmm_walk_launch(const WalkLaunch &L)
     const dim3 grid((unsigned)((long long)nseg * tp * L.col_tiles));
 #define CUVDIA_WALK_ARGS L.tab, L.ngroups, L.period, L.s0, L.astep4, L.seg_tiles, L.vals, L.B, L.ldb, L.dst, L.ldd, \
                          L.n_out, L.n_in, L.batch, L.alpha, L.beta, L.col_tiles, L.a_bytes, L.ep
-    if (L.ep.act == 2) return hipErrorNotSupported;
     const bool fused = L.ep.bias != nullptr || L.ep.act != 0;
     note_kernel("spmm_walk_kernel<%d, %d, 8, %d, %s>", L.lck, L.lck, L.lck == 7 ? 1 : L.lck == 5 ? 2 : 3, fused ? "true" : "false");
 #define CUVDIA_WALK_LAUNCH(LCK, SH)                                                                                    \
@@ -3190,10 +3233,10 @@ hipError_t launch_spmm_tiled(const DiaView &A, const float *vals, const float *B
     // along the rows and find each other's dense rows in its L2.
     const int col_group = col_tiles <= 4 ? (int)col_tiles : 2;
     const int lck = trans ? A.max_len_t : A.max_len_n;
-    // A window table on a product of many tiles: the walking kernel (with a bias and the sigmoid at its tiles' exit,
-    // if asked for; a sampled result stays with the tile-by-tile kernel).
+    // A window table on a product of many tiles: the walking kernel (with the bias, the sigmoid and the sample at
+    // its tiles' exit, if asked for).
     const WalkView &wk = trans ? A.walk_t : A.walk_n;
-    if (walk >= 0 && wk.tab_dev != nullptr && ep.act != 2) {
+    if (walk >= 0 && wk.tab_dev != nullptr) {
         WalkLaunch W{wk.tab_dev, wk.ngroups, wk.period, wk.s0, wk.astep4, wk.lck, wk.k, 0, vals, B, ldb, dst, ldd,
                      n_out, n_in, batch, alpha, beta, (int)col_tiles, (unsigned)((long long)A.nd * A.stride * 4), stream, ep};
         const int seg_tiles = spmm_walk_plan(wk.lck, wk.k, wk.s0, wk.period, n_out, n_in, col_tiles, walk > 0, nullptr);

@@ -155,10 +155,9 @@ int cuvdia_plan_walk(const int *offsets_host, int nd, int stride, int transposed
                      int *period, int *k, int *ngroups, int *lck);
 
 /* Pure host function: does the automatic choice of cuvdia_spmm_f32 -- and of
- * cuvdia_spmm_bias_act_f32 and cuvdia_spmm_layer_f32 without sampling: the
- * bias and the sigmoid are applied where the walking kernel's tiles leave;
- * a sampled result is always served tile by tile -- run the walking kernel
- * for the product of an h x w
+ * cuvdia_spmm_bias_act_f32 and cuvdia_spmm_layer_f32: the bias, the sigmoid
+ * and the sample are applied where the walking kernel's tiles leave -- run
+ * the walking kernel for the product of an h x w
  * matrix with this table (row_fact 1) and `batch` packed dense columns?
  * Returns the number of workgroups of that launch, or 0 when another kernel
  * serves: the table is no window table with a walking kernel (see

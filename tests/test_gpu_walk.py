@@ -70,8 +70,8 @@ def test_walk_matches_the_oracle(oracle, gu, px, fs, channels, batch, trans):
 @pytest.mark.parametrize("trans", ["n", "t"])
 def test_walk_with_bias_and_sigmoid_at_the_tiles_exit(oracle, gu, px, fs, channels, batch, trans):
     """dst = sigmoid(beta*dst + alpha*op(A)*B + bias) through the walking kernel against the reference's three host
-    steps; a sampled result is refused (the tile-by-tile kernel serves it).  Tolerances as for the tile-by-tile
-    kernel: 0.25e-5 * magnitude + 4e-7 behind the sigmoid, 1e-5 * magnitude without."""
+    steps, and the sampled form against the oracle's draw.  Tolerances as for the tile-by-tile kernel: 0.25e-5 *
+    magnitude + 4e-7 behind the sigmoid, 1e-5 * magnitude without."""
     import torch
     from cuv_amd import dia as D, _lib
     L = _lib.lib()
@@ -103,14 +103,25 @@ def test_walk_with_bias_and_sigmoid_at_the_tiles_exit(oracle, gu, px, fs, channe
         assert np.isfinite(got).all()
         tol = (0.25e-5 * mag + 4e-7) if act else (1e-5 * mag + 1e-30)
         assert np.all(np.abs(got - ref) <= tol), (alpha, beta, use_bias, act, float((np.abs(got - ref) / tol).max()))
-    dd = torch.full((batch, n), float("nan"), device="cuda:0")
-    L.cuvdia_set_path(_lib.PATH_WALK)
-    try:
-        with pytest.raises(_lib.CuvDiaError) as err:
-            D.prod_bias_act(dd, dev, Bd, trans, 1.0, 0.0, bd, _lib.ACT_SIGMOID_SAMPLE, seed=5)
-    finally:
-        L.cuvdia_set_path(_lib.PATH_AUTO)
-    assert err.value.code == _lib.EUNSUPPORTED
+    # the sampled form: dst = (p > u) with u(row, column) the documented Philox draw; the oracle's bits wherever the two
+    # sides' p cannot straddle u (the rule of the tile-by-tile kernel's test), for beta == 0 and beta != 0
+    for seed, beta in ((0, 0.0), (0x9E3779B97F4A7C15, 0.0), (12345, 0.5)):
+        p_ref = oracle.prod_bias_act(A, B, dst0 if beta != 0 else None, trans, 1.0, beta, bias, True)
+        mag = oracle.prod_mag(A, B, dst0 if beta != 0 else None, trans, 1.0, beta) + np.abs(bias)[:, None]
+        u = oracle.sample_uniform(n, batch, seed)
+        ref = oracle.rnd_binarize(p_ref, u)
+        decided = np.abs(p_ref.astype(np.float64) - u) > 0.25e-5 * mag + 4e-7
+        assert decided.mean() > 0.999
+        dd = D.to_device_colmajor(dst0) if beta != 0 else torch.full((batch, n), float("nan"), device="cuda:0")
+        L.cuvdia_set_path(_lib.PATH_WALK)
+        try:
+            D.prod_bias_act(dd, dev, Bd, trans, 1.0, beta, bd, _lib.ACT_SIGMOID_SAMPLE, seed=seed)
+            assert L.cuvdia_last_path() == _lib.PATH_WALK
+        finally:
+            L.cuvdia_set_path(_lib.PATH_AUTO)
+        got = D.to_host_colmajor(dd)
+        assert np.all((got == 0.0) | (got == 1.0))
+        assert np.array_equal(got[decided], ref[decided]), (seed, beta, int((got != ref)[decided].sum()))
 
 
 @pytest.mark.parametrize("trans", ["n", "t"])
