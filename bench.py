@@ -222,11 +222,17 @@ def measure_scale(cases, torch, D, W, dev):
         Y = torch.rand(batch, n, generator=g, device=dev)
         bd = D.dev_block_descriptor_f(G)
         A.desc
+        bias = torch.randn(n, generator=g, device=dev)
         ops = {
             "up_pass": (lambda: D.prod(Y, A, X, "n", "n", 1.0, 0.0, sync=False), W.spmm_bytes(p, batch, "n", 0.0)),
             "down_pass": (lambda: D.prod(Y, A, H, "t", "n", 1.0, 0.5, sync=False), W.spmm_bytes(p, batch, "t", 0.5)),
             "weight_gradient": (lambda: D.densedense_to_dia(G, bd, X, H, 1.0 / batch, 0.9, sync=False),
                                 W.dd2dia_bytes(p, batch, 0.9)),
+            # the fused layer updates: h = sample(sigmoid(A v + b)), v' = sigmoid(A^T h + b)
+            "layer_up_sampled": (lambda: D.prod_bias_act(Y, A, X, "n", 1.0, 0.0, bias, _lib.ACT_SIGMOID_SAMPLE, 7, sync=False),
+                                 W.spmm_bytes(p, batch, "n", 0.0) + 4 * n),
+            "layer_down_sigmoid": (lambda: D.prod_bias_act(Y, A, H, "t", 1.0, 0.0, bias, _lib.ACT_SIGMOID, sync=False),
+                                   W.spmm_bytes(p, batch, "t", 0.0) + 4 * n),
         }
         flops = W.flops(p, batch)
         row = dict(map=px, rows=n, batch=batch, flops=flops)
@@ -265,7 +271,7 @@ def measure_scale(cases, torch, D, W, dev):
                              tflops=flops / us / 1e6, kernel=kernel)
             del graph
         out.append(row)
-        del A, G, X, H, Y, bd
+        del A, G, X, H, Y, bd, bias
         torch.cuda.empty_cache()
     return out
 
@@ -757,7 +763,7 @@ def main():
                                          "frac_fp32_valu_broadcast against the 78.6 TFLOP/s of FMAs with a "
                                          "DPP-broadcast or scalar operand, the form these kernels use"),
                           scale=dict(config="the headline layer's pattern (7x7 window, 49 diagonals) on a px x px map at "
-                                            "batch b: each product timed alone (full sweep: --workload scale)",
+                                            "batch b: each product timed alone, and the fused layer updates h = sample(sigmoid(A v + b)), v' = sigmoid(A^T h + b) (full sweep: --workload scale)",
                                      cases=measure_scale([(128, 2048), (512, 128), (512, 512)], torch, D, W, dev)))
 
     else:
